@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused P-way gradient reduce + optimizer update on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload adam_f32]
+
+A "step" is one launch of the hot path over the whole shard with inputs resident in HBM.  The default
+workload is BASELINE config 2: fused reduce + bias-corrected Adam, fp32, N = 2^28 parameters, P = 8
+rank-gradient buffers.  One JSON line is printed: whole-job algorithmic GB/s (56 B/param for Adam), the
+roofline of the dominant kernel from HIP events recorded on the launch stream, and the CPU restatement of the
+reference checker loop timed on a bounded sample on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+METRIC = "fused reduce+Adam GB/s & % HBM roofline, N=2^28 P=8; params/s"
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="adam_f32",
+                    choices=["adam_f32", "sgd_f32", "adam_f16g", "lamb_f32", "mlp_outproj", "copy"])
+    ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
+    ap.add_argument("--ranks", type=int, default=None, help="override P")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--stagger", type=int, default=0, help="extra bytes between consecutive buffers of one arena")
+    return ap.parse_args()
+
+
+class Arena:
+    """Carves equally sized buffers out of one torch allocation, optionally staggered by a few KiB so that the
+    P streams do not start on the same HBM channel."""
+
+    def __init__(self, torch, nbytes_each, count, stagger):
+        self.step = nbytes_each + stagger
+        assert self.step % 256 == 0
+        self.buf = torch.empty(self.step * count + 256, dtype=torch.uint8, device="cuda")
+        base = self.buf.data_ptr()
+        self.off0 = (-base) % 256
+        self.k = 0
+        self.nbytes = nbytes_each
+
+    def take(self, torch, dtype):
+        lo = self.off0 + self.k * self.step
+        self.k += 1
+        return self.buf[lo:lo + self.nbytes].view(dtype)
+
+
+def traffic_from_profiles(name):
+    """HBM bytes per launch measured with rocprofv3 --pmc, if a summary for this workload was committed."""
+    path = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(path):
+        return None
+    vals = {}
+    for line in open(path):
+        if "=" in line and line.split("=")[0].strip() in ("FETCH_BYTES_PER_LAUNCH", "WRITE_BYTES_PER_LAUNCH"):
+            k, v = line.split("=", 1)
+            try:
+                vals[k.strip()] = float(v.split()[0])
+            except ValueError:
+                pass
+    if len(vals) == 2:
+        return vals["FETCH_BYTES_PER_LAUNCH"] + vals["WRITE_BYTES_PER_LAUNCH"]
+    return None
+
+
+def cpu_baseline_adam(P, budget_s=12.0):
+    """The oracle's restatement of the reference checker loop (multi-process-adam-scattered.cpp:112-136 with a
+    fixed-order P-way sum), one thread, on a bounded sample of the same workload."""
+    import oracle as orc
+    n = 1 << 24
+    r = np.random.Generator(np.random.Philox(key=[5, 0]))
+    g = [(r.standard_normal(n, dtype=np.float32) * np.float32(1e-3)) for _ in range(P)]
+    w = r.uniform(-0.05, 0.05, n).astype(np.float32)
+    m = np.zeros(n, np.float32)
+    v = np.zeros(n, np.float32)
+    orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 1)          # warm the pages
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, reps + 2)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 50:
+            break
+    per_param = el / (reps * n)
+    return {
+        "value": round(56.0 / per_param / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "params_per_s": round(1.0 / per_param, 1),
+        "sample": f"oracle orc_adam_f32, P={P}, N=2^24 sample of the 2^28 workload, {reps} steps, 1 thread "
+                  f"({os.cpu_count()} host cpus visible)",
+    }
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the reduce over P rank buffers is local); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from coconet_amd import capi
+    capi.load()
+    capi.init(0)
+    torch.cuda.set_device(0)
+    info = capi.device_info()
+    K, W = a.steps, a.warmup
+    wl = a.workload
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+
+    flops = None
+    if wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g"):
+        P = a.ranks or (4 if wl == "sgd_f32" else 8)
+        N = 1 << (a.log2n or (20 if wl == "sgd_f32" else 28))
+        gbytes = 2 if wl == "adam_f16g" else 4
+        ar = Arena(torch, N * gbytes, P, a.stagger)
+        g = []
+        for p in range(P):
+            t = ar.take(torch, torch.float16 if gbytes == 2 else torch.float32)
+            if gbytes == 2:
+                t.copy_((torch.randn(N, device="cuda", generator=gen) * (1e-3 * 65536.0)).to(torch.float16))
+            else:
+                t.normal_(0.0, 1e-3 if wl != "sgd_f32" else 1e-2, generator=gen)
+            g.append(t)
+        ar2 = Arena(torch, N * 4, 3, a.stagger)
+        w, m, v = (ar2.take(torch, torch.float32) for _ in range(3))
+        w.uniform_(-0.05, 0.05, generator=gen)
+        m.zero_()
+        v.zero_()
+        if wl == "adam_f32":
+            per_param = (P + 3) * 4 + 3 * 4
+            step = lambda t: capi.adam_f32(g, w, m, v, N, 1e-3, 0.9, 0.999, 1e-6, t, stream)
+            kernel = "fused_stream_kernel<AdamMath,8,4,2>"
+        elif wl == "sgd_f32":
+            per_param = (P + 1) * 4 + 4
+            step = lambda t: capi.sgd_f32(g, w, N, 0.01, stream)
+            kernel = "fused_stream_kernel<SgdMath>"
+        elif wl == "adam_f16g":
+            w16 = torch.empty(N, dtype=torch.float16, device="cuda")
+            flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+            g[0][::1 << 20] = float("inf")
+            per_param = P * 2 + 12 + 12 + 2
+            step = lambda t: capi.adam_f16g(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, t, 2.0 ** -16, flag, stream)
+            kernel = "fused_stream_kernel<Adam16Math,8,8,1>"
+        else:
+            nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
+            plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
+            per_param = (P + 3) * 4 + 3 * 4
+            step = lambda t: plan.step(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, capi.LAMB_TRUST_RATIO, stream)
+            kernel = "lamb_pass1_kernel<8> + lamb_finalize_kernel + lamb_pass2_kernel"
+        alg_bytes = float(per_param) * N
+        units = N
+        config = {"workload": f"{wl} fused reduce+update, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,
+                  "algorithmic_bytes_per_param": per_param, "stagger_bytes": a.stagger}
+    elif wl == "mlp_outproj":
+        M = Nn = 8192
+        Kd = 1024
+        X = torch.randn(M, Kd, device="cuda", generator=gen).to(torch.bfloat16)
+        Wm = (torch.randn(Kd, Nn, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+        parts = [torch.randn(M, Nn, device="cuda", generator=gen) for _ in range(7)]
+        bias = torch.randn(Nn, device="cuda", generator=gen)
+        resid = torch.randn(M, Nn, device="cuda", generator=gen).to(torch.bfloat16)
+        out = torch.empty(M, Nn, dtype=torch.bfloat16, device="cuda")
+        step = lambda t: capi.mlp_outproj_bf16(X, Wm, parts, bias, resid, out, M, Nn, Kd, 0.1, 0, stream)
+        alg_bytes = float(7 * M * Nn * 4 + M * Kd * 2 + Kd * Nn * 2 + Nn * 4 + 2 * M * Nn * 2)
+        flops = 2.0 * M * Nn * Kd
+        units = M * Nn
+        kernel = "mlp_outproj_kernel<7>"
+        config = {"workload": "mlp_outproj bf16 8192x1024x8192 + 7 fp32 partials + bias + dropout(0.1) + residual",
+                  "M": M, "N": Nn, "K": Kd}
+    else:   # plain device copy, the practical HBM ceiling of this box
+        N = 1 << (a.log2n or 30)
+        src = torch.empty(N, dtype=torch.float32, device="cuda").normal_(generator=gen)
+        dst = torch.empty_like(src)
+        step = lambda t: dst.copy_(src)
+        alg_bytes = 8.0 * N
+        units = N
+        kernel = "torch copy"
+        config = {"workload": f"device copy of 2^{int(np.log2(N))} fp32"}
+
+    for t in range(1, W + 1):
+        step(t)
+    torch.cuda.synchronize()
+    e0, e1 = capi.Event(), capi.Event()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for t in range(W + 1, W + K + 1):
+        step(t)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3 / K
+    ev_ms = e0.elapsed_ms(e1) / K
+
+    gbps = alg_bytes / (wall_ms * 1e-3) / 1e9
+    ach = alg_bytes / (ev_ms * 1e-3) / 1e9
+    line = {
+        "metric": METRIC if wl == "adam_f32" else f"{wl} algorithmic GB/s",
+        "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"adam_f16g": "f16 gradients, f32 state", "mlp_outproj": "bf16 x bf16 -> f32"}.get(wl, "f32"),
+        "data": "synthetic", "config": config,
+        "params_per_s": round(units / (wall_ms * 1e-3), 1),
+        "device": info,
+        "roofline": {"bound": "hbm", "achieved": round(ach, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": traffic_from_profiles(f"{wl}.pmc.txt"),
+                     "kernel": kernel, "avg_launch_ms": round(ev_ms, 5), "algorithmic_bytes_per_launch": alg_bytes},
+    }
+    if flops:
+        line["mfma"] = {"achieved": round(flops / (ev_ms * 1e-3) / 1e12, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    if wl == "adam_f32" and not a.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_adam(8)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

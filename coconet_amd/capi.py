@@ -1,0 +1,259 @@
+"""ctypes binding of libcoconet_hip.so (include/coconet_hip.h).
+
+Thin by design: every function below forwards device pointers and sizes to the C ABI and raises
+CoconetError on a non-zero return code.  torch is used by callers only to own device memory and streams;
+arguments here are raw addresses (ints), torch tensors (their data_ptr() is taken) or None.
+
+There is no CPU fallback: if the shared library is missing, loading raises.
+"""
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libcoconet_hip.so")
+
+CCN_OK = 0
+CCN_EINVAL = -22
+CCN_ENOMEM = -12
+CCN_ENODEV = -19
+CCN_EHIP = -5
+CCN_ERANGE = -34
+CCN_MAX_RANKS = 16
+LAMB_TRUST_RATIO = 0
+LAMB_REFERENCE = 1
+
+# every symbol include/coconet_hip.h declares
+SYMBOLS = [
+    "ccn_version", "ccn_init", "ccn_device_info", "ccn_malloc", "ccn_free", "ccn_memcpy_h2d", "ccn_memcpy_d2h",
+    "ccn_memcpy_d2d", "ccn_fill_f32", "ccn_stream_create", "ccn_stream_destroy", "ccn_stream_sync",
+    "ccn_event_create", "ccn_event_destroy", "ccn_event_record", "ccn_event_elapsed_ms", "ccn_last_hip_error",
+    "ccn_strerror", "ccn_reduce_f32", "ccn_sgd_f32", "ccn_sgd_axpby_f32", "ccn_pseudo_adam_f32", "ccn_adam_f32",
+    "ccn_adam_f16g", "ccn_overflow_check_f16", "ccn_fused_adam_ref_f16g", "ccn_lamb_plan_create",
+    "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
+    "ccn_bias_dropout_residual",
+]
+
+
+class CoconetError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__(f"{what}: error {code} ({strerror(code)})")
+
+
+_lib = None
+
+
+def load():
+    """Load the library (once).  Raises OSError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError(f"{LIB_PATH} is missing: run `python -m coconet_amd.build` (needs hipcc)")
+        L = C.CDLL(LIB_PATH)
+        _declare(L)
+        _lib = L
+    return _lib
+
+
+_vp, _i, _f, _sz, _u64 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint64
+_pp = C.POINTER(C.c_void_p)
+
+
+def _declare(L):
+    def sig(name, args, res=_i):
+        fn = getattr(L, name)
+        fn.argtypes = args
+        fn.restype = res
+
+    sig("ccn_version", [])
+    sig("ccn_init", [_i])
+    sig("ccn_device_info", [C.POINTER(_i), C.POINTER(_sz), C.c_char_p, _sz])
+    sig("ccn_malloc", [_pp, _sz])
+    sig("ccn_free", [_vp])
+    sig("ccn_memcpy_h2d", [_vp, _vp, _sz, _vp])
+    sig("ccn_memcpy_d2h", [_vp, _vp, _sz, _vp])
+    sig("ccn_memcpy_d2d", [_vp, _vp, _sz, _vp])
+    sig("ccn_fill_f32", [_vp, _f, _sz, _vp])
+    sig("ccn_stream_create", [_pp])
+    sig("ccn_stream_destroy", [_vp])
+    sig("ccn_stream_sync", [_vp])
+    sig("ccn_event_create", [_pp])
+    sig("ccn_event_destroy", [_vp])
+    sig("ccn_event_record", [_vp, _vp])
+    sig("ccn_event_elapsed_ms", [_vp, _vp, C.POINTER(_f)])
+    sig("ccn_last_hip_error", [])
+    sig("ccn_strerror", [_i], C.c_char_p)
+    sig("ccn_reduce_f32", [_pp, _i, _vp, _sz, _vp])
+    sig("ccn_sgd_f32", [_pp, _i, _vp, _sz, _f, _vp])
+    sig("ccn_sgd_axpby_f32", [_pp, _i, _vp, _sz, _f, _f, _vp])
+    sig("ccn_pseudo_adam_f32", [_pp, _i, _vp, _vp, _vp, _sz, _f, _f, _f, _vp])
+    sig("ccn_adam_f32", [_pp, _i, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _vp])
+    sig("ccn_adam_f16g", [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _f, _vp, _vp])
+    sig("ccn_overflow_check_f16", [_pp, _i, _sz, _vp, _vp])
+    sig("ccn_fused_adam_ref_f16g", [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _vp])
+    sig("ccn_lamb_plan_create", [C.POINTER(_sz), _i, _pp])
+    sig("ccn_lamb_plan_destroy", [_vp])
+    sig("ccn_lamb_f32", [_vp, _pp, _i, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
+    sig("ccn_lamb_plan_norms", [_vp, _vp, _vp])
+    sig("ccn_mlp_outproj_bf16", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _vp])
+    sig("ccn_bias_dropout_residual", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _vp])
+
+
+def strerror(code):
+    return load().ccn_strerror(int(code)).decode()
+
+
+def _check(rc, what):
+    if rc != CCN_OK:
+        raise CoconetError(rc, what)
+
+
+def addr(x):
+    """Device address of a torch tensor, or an int / None passed through."""
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    return x.data_ptr()
+
+
+def ptr_table(bufs):
+    """Host array of device pointers (what the ABI calls `g` or `partials`)."""
+    tbl = (C.c_void_p * max(len(bufs), 1))()
+    for k, b in enumerate(bufs):
+        tbl[k] = addr(b)
+    return C.cast(tbl, _pp), tbl
+
+
+def current_stream():
+    """The HIP stream torch is currently issuing work on, as an address."""
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+# ---- runtime ---------------------------------------------------------------------------------------------------------
+def version():
+    return load().ccn_version()
+
+
+def init(device=0):
+    _check(load().ccn_init(device), "ccn_init")
+
+
+def device_info():
+    cu, hbm, arch = _i(0), _sz(0), C.create_string_buffer(64)
+    _check(load().ccn_device_info(C.byref(cu), C.byref(hbm), arch, 64), "ccn_device_info")
+    return {"cu_count": cu.value, "hbm_bytes": hbm.value, "arch": arch.value.decode()}
+
+
+class Event:
+    def __init__(self):
+        h = C.c_void_p()
+        _check(load().ccn_event_create(C.byref(h)), "ccn_event_create")
+        self.h = h
+
+    def record(self, stream=None):
+        _check(load().ccn_event_record(self.h, stream), "ccn_event_record")
+
+    def elapsed_ms(self, stop):
+        ms = _f(0)
+        _check(load().ccn_event_elapsed_ms(self.h, stop.h, C.byref(ms)), "ccn_event_elapsed_ms")
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.h:
+                load().ccn_event_destroy(self.h)
+        except Exception:
+            pass
+
+
+# ---- hot path --------------------------------------------------------------------------------------------------------
+def reduce_f32(g, out, n, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_reduce_f32(p, len(g), addr(out), n, stream), "ccn_reduce_f32")
+
+
+def sgd_f32(g, w, n, lr, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_sgd_f32(p, len(g), addr(w), n, lr, stream), "ccn_sgd_f32")
+
+
+def sgd_axpby_f32(g, w, n, alpha, beta, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_sgd_axpby_f32(p, len(g), addr(w), n, alpha, beta, stream), "ccn_sgd_axpby_f32")
+
+
+def pseudo_adam_f32(g, w, m, v, n, lr, beta1, beta2, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_pseudo_adam_f32(p, len(g), addr(w), addr(m), addr(v), n, lr, beta1, beta2, stream),
+           "ccn_pseudo_adam_f32")
+
+
+def adam_f32(g, w, m, v, n, lr, beta1, beta2, eps, step, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_adam_f32(p, len(g), addr(w), addr(m), addr(v), n, lr, beta1, beta2, eps, step, stream),
+           "ccn_adam_f32")
+
+
+def adam_f16g(g, w, m, v, w16, n, lr, beta1, beta2, eps, step, inv_scale, overflow_flag, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_adam_f16g(p, len(g), addr(w), addr(m), addr(v), addr(w16), n, lr, beta1, beta2, eps, step,
+                                inv_scale, addr(overflow_flag), stream), "ccn_adam_f16g")
+
+
+def overflow_check_f16(g, n, overflow_flag, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_overflow_check_f16(p, len(g), n, addr(overflow_flag), stream), "ccn_overflow_check_f16")
+
+
+def fused_adam_ref_f16g(g, w, halfw, m, v, n, lr, beta1, beta2, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_fused_adam_ref_f16g(p, len(g), addr(w), addr(halfw), addr(m), addr(v), n, lr, beta1, beta2,
+                                          stream), "ccn_fused_adam_ref_f16g")
+
+
+class LambPlan:
+    """Device-side segment tables for one segmentation of [0, N) (ccn_lamb_plan)."""
+
+    def __init__(self, seg_offsets):
+        offs = [int(x) for x in seg_offsets]
+        self.nseg = len(offs) - 1
+        arr = (_sz * len(offs))(*offs)
+        h = C.c_void_p()
+        _check(load().ccn_lamb_plan_create(arr, self.nseg, C.byref(h)), "ccn_lamb_plan_create")
+        self.h = h
+
+    def step(self, g, w, m, v, lr, beta1, beta2, eps, wd, step, mode=LAMB_TRUST_RATIO, stream=None):
+        p, _keep = ptr_table(g)
+        _check(load().ccn_lamb_f32(self.h, p, len(g), addr(w), addr(m), addr(v), lr, beta1, beta2, eps, wd, step, mode,
+                                   stream), "ccn_lamb_f32")
+
+    def norms(self, stream=None):
+        import numpy as np
+        out = np.empty((self.nseg, 2), np.float64)
+        _check(load().ccn_lamb_plan_norms(self.h, out.ctypes.data_as(C.c_void_p), stream), "ccn_lamb_plan_norms")
+        return out
+
+    def close(self):
+        if self.h:
+            _check(load().ccn_lamb_plan_destroy(self.h), "ccn_lamb_plan_destroy")
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def mlp_outproj_bf16(X, W, partials, bias, resid, out, M, N, K, p_drop, seed, stream=None):
+    p, _keep = ptr_table(partials)
+    _check(load().ccn_mlp_outproj_bf16(addr(X), addr(W), p, len(partials), addr(bias), addr(resid), addr(out), M, N, K,
+                                       p_drop, seed, stream), "ccn_mlp_outproj_bf16")
+
+
+def bias_dropout_residual(acc, partials, bias, resid, out, M, N, p_drop, seed, stream=None):
+    p, _keep = ptr_table(partials)
+    _check(load().ccn_bias_dropout_residual(addr(acc), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
+                                            p_drop, seed, stream), "ccn_bias_dropout_residual")

@@ -1,0 +1,158 @@
+// Shared device/host helpers of libcoconet_hip (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+#include "coconet_hip.h"
+
+namespace ccn {
+
+constexpr int kBlock = 256;        // 4 wavefronts of 64 lanes
+constexpr int kWave = 64;
+
+// ---- host-side error plumbing -----------------------------------------------------------------------------------
+extern thread_local int g_last_hip_error;
+int hip_fail(hipError_t e);                        // records e, returns the CCN_E* code for it
+#define CCN_HIP(expr)                                                      \
+  do {                                                                     \
+    hipError_t _e = (expr);                                                \
+    if (_e != hipSuccess) return ::ccn::hip_fail(_e);                      \
+  } while (0)
+
+struct DeviceInfo {
+  int device = -1;
+  int cu_count = 0;
+  size_t hbm_bytes = 0;
+  char arch[64] = {0};
+};
+int current_device_info(const DeviceInfo** out);   // lazily initialises the current device
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- packs: N elements of T held in registers and moved with 16-byte memory instructions ---------------------------
+// (N == 1: one scalar access).  Addresses must be 16-byte aligned when N > 1.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T, int N> struct Pack {
+  T d[N];
+};
+
+// Gradients and partial sums are touched once per step: stream them past the caches (nontemporal).
+template <typename T, int N> __device__ __forceinline__ Pack<T, N> load_stream(const T* p) {
+  Pack<T, N> r;
+  if constexpr (N == 1) {
+    r.d[0] = __builtin_nontemporal_load(p);
+  } else {
+    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
+    constexpr int C = (N * (int)sizeof(T)) / 16;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      const u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p) + c);
+      __builtin_memcpy(reinterpret_cast<char*>(r.d) + 16 * c, &x, 16);
+    }
+  }
+  return r;
+}
+template <typename T, int N> __device__ __forceinline__ Pack<T, N> load_keep(const T* p) {
+  Pack<T, N> r;
+  if constexpr (N == 1) {
+    r.d[0] = *p;
+  } else {
+    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
+    constexpr int C = (N * (int)sizeof(T)) / 16;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      const u32x4 x = *(reinterpret_cast<const u32x4*>(p) + c);
+      __builtin_memcpy(reinterpret_cast<char*>(r.d) + 16 * c, &x, 16);
+    }
+  }
+  return r;
+}
+template <typename T, int N> __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
+  if constexpr (N == 1) {
+    *p = v.d[0];
+  } else {
+    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
+    constexpr int C = (N * (int)sizeof(T)) / 16;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      u32x4 x;
+      __builtin_memcpy(&x, reinterpret_cast<const char*>(v.d) + 16 * c, 16);
+      *(reinterpret_cast<u32x4*>(p) + c) = x;
+    }
+  }
+}
+
+// ---- table of P source pointers, passed by value in the kernel argument segment ----------------------------------
+template <typename T, int CAP> struct SrcTable { const T* p[CAP]; };
+
+// ---- wavefront / workgroup reductions (64-wide) -------------------------------------------------------------------
+__device__ __forceinline__ double wave_sum(double x) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, kWave);
+  return x;   // valid in lane 0
+}
+
+// Sum of `x` over a kBlock-thread workgroup; result valid in thread 0.  lds must hold kBlock/kWave doubles.
+__device__ __forceinline__ double block_sum(double x, double* lds) {
+  const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+  x = wave_sum(x);
+  if (lane == 0) lds[wv] = x;
+  __syncthreads();
+  double r = 0.0;
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < kBlock / kWave; k++) r += lds[k];
+  }
+  __syncthreads();
+  return r;
+}
+
+// ---- half / bfloat16 scalars -----------------------------------------------------------------------------------------
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  _Float16 x = __builtin_bit_cast(_Float16, h);
+  return (float)x;
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {   // round-to-nearest-even
+  _Float16 x = (_Float16)f;
+  return __builtin_bit_cast(uint16_t, x);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {  // round-to-nearest-even, quiet nan
+  uint32_t x = __float_as_uint(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return (uint16_t)(x >> 16);
+}
+
+// ---- Philox-4x32-10, and the dropout keep decision built on it -----------------------------------------------------
+struct Philox4 { uint32_t x, y, z, w; };
+__host__ __device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                                          uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    const uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return Philox4{c0, c1, c2, c3};
+}
+__host__ __device__ __forceinline__ bool keep_from_word(uint32_t word, float p_drop) {
+  const float u = (float)(word >> 8) * 5.9604644775390625e-08f;
+  return u >= p_drop;
+}
+
+// ---- launch geometry for streaming kernels ----------------------------------------------------------------------------
+// Number of workgroups for a grid-stride kernel whose workgroup consumes `tile` units per iteration.
+unsigned stream_grid(size_t units, size_t tile);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace ccn

@@ -1,0 +1,286 @@
+// Model-parallel MLP out-projection for gfx950: bf16 MFMA GEMM with the all-reduce partial sum, bias,
+// dropout and residual fused into the tile write-back, plus the same epilogue as a standalone kernel.
+//
+// GEMM tiling: a 256-thread workgroup owns a 128(m) x 128(n) tile of C and walks K in steps of 64.
+// The four wavefronts form a 2x2 grid; each owns 64x64 as 2x2 v_mfma_f32_32x32x16_bf16 blocks.
+// The MFMA computes C^T blocks (rows = n from W, columns = m from X) so that every lane ends up with
+// four CONSECUTIVE n of one row m in its accumulator quads: the epilogue then moves 16-byte pieces of
+// the fp32 partial buffers and 8-byte pieces of the bf16 residual/output.
+// W is [K x N] row-major (n contiguous) while the MFMA wants k contiguous per lane, so the W tile is
+// transposed in registers on its way into LDS.  LDS rows are 128 bytes (64 k) with the eight 16-byte
+// chunks XOR-swizzled by (row%8)^((row/8)%8): conflict-free for the 8-byte transposed writes and the
+// 16-byte fragment reads.
+#include "ccn_common.hpp"
+
+namespace ccn {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 64;
+
+struct EpiPrm {
+  float p_drop, keep_scale;
+  uint32_t seed_lo, seed_hi;
+  int apply_dropout;
+};
+
+// Epilogue for four consecutive columns n..n+3 (n % 4 == 0) of row m.  acc holds the local product.
+template <int NP>
+__device__ __forceinline__ void epilogue_quad(f32x4 acc, const SrcTable<float, 8>& parts, int nPartials,
+                                              const float* __restrict__ bias, const uint16_t* __restrict__ resid,
+                                              uint16_t* __restrict__ out, size_t m, size_t n, size_t N, const EpiPrm& k) {
+  const size_t idx = m * N + n;
+  f32x4 pv[NP > 0 ? NP : 1];
+  if constexpr (NP > 0) {
+#pragma unroll
+    for (int q = 0; q < NP; q++) pv[q] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts.p[q] + idx));
+  }
+  const f32x4 bv = *reinterpret_cast<const f32x4*>(bias + n);
+  u32x2 rv = {0u, 0u};
+  if (resid) rv = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(resid + idx));
+  f32x4 s = acc;
+  if constexpr (NP > 0) {
+#pragma unroll
+    for (int q = 0; q < NP; q++) s = s + pv[q];
+  } else {
+    for (int q = 0; q < nPartials; q++) s = s + __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts.p[q] + idx));
+  }
+  const f32x4 t = s + bv;
+  f32x4 d = t;
+  if (k.apply_dropout) {
+    const uint64_t blk = (uint64_t)idx >> 2;
+    const Philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u, k.seed_lo, k.seed_hi);
+    d[0] = keep_from_word(r.x, k.p_drop) ? t[0] * k.keep_scale : 0.0f;
+    d[1] = keep_from_word(r.y, k.p_drop) ? t[1] * k.keep_scale : 0.0f;
+    d[2] = keep_from_word(r.z, k.p_drop) ? t[2] * k.keep_scale : 0.0f;
+    d[3] = keep_from_word(r.w, k.p_drop) ? t[3] * k.keep_scale : 0.0f;
+  }
+  const float y0 = d[0] + bf16_bits_to_f32((uint16_t)(rv[0] & 0xffffu));
+  const float y1 = d[1] + bf16_bits_to_f32((uint16_t)(rv[0] >> 16));
+  const float y2 = d[2] + bf16_bits_to_f32((uint16_t)(rv[1] & 0xffffu));
+  const float y3 = d[3] + bf16_bits_to_f32((uint16_t)(rv[1] >> 16));
+  u32x2 o;
+  o[0] = (uint32_t)f32_to_bf16_bits(y0) | ((uint32_t)f32_to_bf16_bits(y1) << 16);
+  o[1] = (uint32_t)f32_to_bf16_bits(y2) | ((uint32_t)f32_to_bf16_bits(y3) << 16);
+  *reinterpret_cast<u32x2*>(out + idx) = o;
+}
+
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 7); }
+
+template <int NP>
+__global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
+                                                             const SrcTable<float, 8> parts, const int nPartials,
+                                                             const float* __restrict__ bias,
+                                                             const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
+                                                             const int M, const int N, const int K, const EpiPrm ep) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds_x[BM * BK * 2];   // [m][k] swizzled
+  __shared__ __attribute__((aligned(16))) uint8_t lds_w[BN * BK * 2];   // [n][k] swizzled (W tile transposed)
+
+  // ---- workgroup -> tile.  Workgroups are dealt round-robin to the 8 XCDs; give each XCD a band of tile rows and
+  //      walk it column by column so that the tiles resident on one XCD share X and W panels in its L2.
+  const int tilesM = M / BM;
+  int tm, tn;
+  {
+    const int b = blockIdx.x;
+    if ((tilesM & 7) == 0) {
+      const int band = tilesM >> 3;          // tile rows per XCD
+      const int xcd = b & 7, slot = b >> 3;  // slot in [0, band*tilesN)
+      tm = xcd * band + slot % band;
+      tn = slot / band;
+    } else {
+      tm = b % tilesM;
+      tn = b / tilesM;
+    }
+  }
+  const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // global -> register staging assignments
+  const int xr = t >> 3, xc = t & 7;          // X: rows xr + 32*j, 16-byte chunk xc
+  const int wg = t & 15, wq = t >> 4;         // W: k rows wq*4 + j, columns wg*8..+7
+  u32x4 xreg[4], wreg[4];
+
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      xreg[j] = *reinterpret_cast<const u32x4*>(X + (m0 + xr + 32 * j) * (size_t)K + k0 + xc * 8);
+      wreg[j] = *reinterpret_cast<const u32x4*>(W + (size_t)(k0 + wq * 4 + j) * N + n0 + wg * 8);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int row = xr + 32 * j;
+      *reinterpret_cast<u32x4*>(lds_x + row * 128 + ((xc ^ swz(row)) << 4)) = xreg[j];
+    }
+    // transpose 4(k) x 8(n) -> 8 rows of 4 k
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const uint32_t a0 = wreg[0][q], a1 = wreg[1][q], a2 = wreg[2][q], a3 = wreg[3][q];
+      u32x2 lo, hi;   // lo: column 2q, hi: column 2q+1; each k0..k3
+      lo[0] = (a0 & 0xffffu) | (a1 << 16);
+      lo[1] = (a2 & 0xffffu) | (a3 << 16);
+      hi[0] = (a0 >> 16) | (a1 & 0xffff0000u);
+      hi[1] = (a2 >> 16) | (a3 & 0xffff0000u);
+      const int r0 = wg * 8 + 2 * q, r1 = r0 + 1;
+      *reinterpret_cast<u32x2*>(lds_w + r0 * 128 + (((wq >> 1) ^ swz(r0)) << 4) + ((wq & 1) << 3)) = lo;
+      *reinterpret_cast<u32x2*>(lds_w + r1 * 128 + (((wq >> 1) ^ swz(r1)) << 4) + ((wq & 1) << 3)) = hi;
+    }
+  };
+
+  f32x16 acc[2][2];   // [bn][bm]
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
+
+  const int nk = K / BK;
+  load_tile(0);
+  store_tile();
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt++) {
+    if (kt + 1 < nk) load_tile((kt + 1) * BK);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      const int c = ks * 2 + (lane >> 5);
+      bf16x8 fa[2], fb[2];
+#pragma unroll
+      for (int bn = 0; bn < 2; bn++) {
+        const int row = wn * 64 + bn * 32 + (lane & 31);
+        fa[bn] = *reinterpret_cast<const bf16x8*>(lds_w + row * 128 + ((c ^ swz(row)) << 4));
+      }
+#pragma unroll
+      for (int bm = 0; bm < 2; bm++) {
+        const int row = wm * 64 + bm * 32 + (lane & 31);
+        fb[bm] = *reinterpret_cast<const bf16x8*>(lds_x + row * 128 + ((c ^ swz(row)) << 4));
+      }
+#pragma unroll
+      for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+        for (int bm = 0; bm < 2; bm++)
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[bn], fb[bm], acc[bn][bm], 0, 0, 0);
+    }
+    __syncthreads();
+    if (kt + 1 < nk) {
+      store_tile();
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: accumulator register 4*i4+e of block (bn,bm) is C[m][n+e] with
+  //      n = n0 + wn*64 + bn*32 + i4*8 + (lane/32)*4,  m = m0 + wm*64 + bm*32 + lane%32
+#pragma unroll
+  for (int bm = 0; bm < 2; bm++) {
+    const size_t m = m0 + wm * 64 + bm * 32 + (lane & 31);
+#pragma unroll
+    for (int bn = 0; bn < 2; bn++) {
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const size_t n = n0 + wn * 64 + bn * 32 + i4 * 8 + (lane >> 5) * 4;
+        f32x4 a;
+        a[0] = acc[bn][bm][i4 * 4 + 0];
+        a[1] = acc[bn][bm][i4 * 4 + 1];
+        a[2] = acc[bn][bm][i4 * 4 + 2];
+        a[3] = acc[bn][bm][i4 * 4 + 3];
+        epilogue_quad<NP>(a, parts, nPartials, bias, resid, out, m, n, (size_t)N, ep);
+      }
+    }
+  }
+}
+
+// Standalone epilogue over an fp32 product in memory: one thread per four columns.
+template <int NP>
+__global__ __launch_bounds__(kBlock) void bias_dropout_residual_kernel(const float* __restrict__ acc,
+                                                                       const SrcTable<float, 8> parts, const int nPartials,
+                                                                       const float* __restrict__ bias,
+                                                                       const uint16_t* __restrict__ resid,
+                                                                       uint16_t* __restrict__ out, const size_t M,
+                                                                       const size_t N, const EpiPrm ep) {
+  const size_t nq = N / 4, total = M * nq;
+  for (size_t q = (size_t)blockIdx.x * kBlock + threadIdx.x; q < total; q += (size_t)gridDim.x * kBlock) {
+    const size_t m = q / nq, n = (q - m * nq) * 4;
+    const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(acc + m * N + n));
+    epilogue_quad<NP>(a, parts, nPartials, bias, resid, out, m, n, N, ep);
+  }
+}
+
+static int make_epi(float p_drop, uint64_t seed, EpiPrm* ep) {
+  if (!(p_drop >= 0.0f) || !(p_drop < 1.0f)) return CCN_EINVAL;
+  ep->p_drop = p_drop;
+  ep->keep_scale = 1.0f / (1.0f - p_drop);
+  ep->seed_lo = (uint32_t)seed;
+  ep->seed_hi = (uint32_t)(seed >> 32);
+  ep->apply_dropout = p_drop > 0.0f ? 1 : 0;
+  return CCN_OK;
+}
+
+}  // namespace ccn
+
+using namespace ccn;
+
+extern "C" {
+
+int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                         const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
+                         uint64_t seed, void* stream) {
+  if (!X || !W || !bias || !out || nPartials < 0 || nPartials > 8 || (nPartials > 0 && !partials)) return CCN_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0) return CCN_EINVAL;
+  if (M % BM || N % BN || K % BK) return CCN_ERANGE;   // whole tiles only
+  SrcTable<float, 8> tbl;
+  for (int q = 0; q < 8; q++) {
+    tbl.p[q] = q < nPartials ? partials[q] : nullptr;
+    if (q < nPartials && (!partials[q] || !aligned16(partials[q]))) return CCN_EINVAL;
+  }
+  if (!aligned16(X) || !aligned16(W) || !aligned16(bias) || !aligned16(out) || (resid && !aligned16(resid))) return CCN_EINVAL;
+  EpiPrm ep;
+  int rc = make_epi(p_drop, seed, &ep);
+  if (rc != CCN_OK) return rc;
+  const DeviceInfo* di = nullptr;
+  rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
+  hipStream_t s = as_stream(stream);
+  if (nPartials == 7)
+    hipLaunchKernelGGL((mlp_outproj_kernel<7>), grid, block, 0, s, X, W, tbl, nPartials, bias, resid, out, M, N, K, ep);
+  else
+    hipLaunchKernelGGL((mlp_outproj_kernel<0>), grid, block, 0, s, X, W, tbl, nPartials, bias, resid, out, M, N, K, ep);
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
+}
+
+int ccn_bias_dropout_residual(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                              const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                              void* stream) {
+  if (!acc || !bias || !out || nPartials < 0 || nPartials > 8 || (nPartials > 0 && !partials)) return CCN_EINVAL;
+  if (M <= 0 || N <= 0) return CCN_EINVAL;
+  if (N % 4) return CCN_ERANGE;
+  SrcTable<float, 8> tbl;
+  for (int q = 0; q < 8; q++) {
+    tbl.p[q] = q < nPartials ? partials[q] : nullptr;
+    if (q < nPartials && (!partials[q] || !aligned16(partials[q]))) return CCN_EINVAL;
+  }
+  if (!aligned16(acc) || !aligned16(bias) || !aligned16(out) || (resid && !aligned16(resid))) return CCN_EINVAL;
+  EpiPrm ep;
+  int rc = make_epi(p_drop, seed, &ep);
+  if (rc != CCN_OK) return rc;
+  const DeviceInfo* di = nullptr;
+  rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  const size_t total = (size_t)M * (size_t)(N / 4);
+  const unsigned grid = stream_grid(total, kBlock);
+  hipStream_t s = as_stream(stream);
+  if (nPartials == 7)
+    hipLaunchKernelGGL((bias_dropout_residual_kernel<7>), dim3(grid), dim3(kBlock), 0, s, acc, tbl, nPartials, bias, resid,
+                       out, (size_t)M, (size_t)N, ep);
+  else
+    hipLaunchKernelGGL((bias_dropout_residual_kernel<0>), dim3(grid), dim3(kBlock), 0, s, acc, tbl, nPartials, bias, resid,
+                       out, (size_t)M, (size_t)N, ep);
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
+}
+
+}  // extern "C"

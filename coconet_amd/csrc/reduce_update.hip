@@ -1,0 +1,417 @@
+// Fused "reduce P rank-gradient buffers + optimizer update" kernels for gfx950.
+//
+// One streaming skeleton (fused_stream_kernel) is instantiated with a math policy per optimizer.
+// The skeleton owns the memory behaviour: 128-bit loads of every operand, all loads of a tile issued
+// before the first use, grid-stride over the shard, in-place 128-bit stores.  The policy owns the
+// arithmetic, written operation by operation in the order of the reference's checker loops so that
+// every fp32 rounding happens where the checker's does (the library is compiled with
+// -ffp-contract=off; division and square root are the correctly rounded ones).
+#include "ccn_common.hpp"
+
+#include <cmath>
+
+namespace ccn {
+
+template <int NS> struct StateTable { float* p[NS > 0 ? NS : 1]; };
+
+// ------------------------------------------------------------------------------------------------------------------
+// Math policies.
+//   G        storage type of one gradient element (float, or uint16_t holding fp16 bits)
+//   NS       number of fp32 state arrays, read and rewritten in place (order: w, m, v)
+//   OUT16    one extra uint16 output per element          OUTF   one extra fp32 output per element
+//   FLAG     the kernel ORs a "bad element seen" bit into *flag
+//   Acc      running gradient sum;  first()/next() fold the P ranks in ascending order
+//   apply()  consumes the sum and the state of one element; returns true if the element was "bad"
+// ------------------------------------------------------------------------------------------------------------------
+struct SumF32 {
+  using G = float;
+  using Acc = float;
+  template <class Prm> static __device__ __forceinline__ Acc first(G x, const Prm&) { return x; }
+  template <class Prm> static __device__ __forceinline__ void next(Acc& a, G x, const Prm&) { a = a + x; }
+};
+
+struct ReduceMath : SumF32 {
+  static constexpr int NS = 0, UNROLL = 2;
+  static constexpr bool OUT16 = false, OUTF = true, FLAG = false;
+  struct Prm {};
+  static __device__ __forceinline__ bool apply(Acc gs, float*, uint16_t&, float& of, const Prm&) {
+    of = gs;
+    return false;
+  }
+};
+
+// examples/test-sgd.cu:17-18
+struct SgdMath : SumF32 {
+  static constexpr int NS = 1, UNROLL = 2;
+  static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
+  struct Prm { float lr; };
+  static __device__ __forceinline__ bool apply(Acc gs, float* st, uint16_t&, float&, const Prm& k) {
+    st[0] = (st[0] - (k.lr * gs));
+    return false;
+  }
+};
+
+// nccl-overlap/samples/single-process-wX.cu:141
+struct AxpbyMath : SumF32 {
+  static constexpr int NS = 1, UNROLL = 2;
+  static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
+  struct Prm { float alpha, beta; };
+  static __device__ __forceinline__ bool apply(Acc gs, float* st, uint16_t&, float&, const Prm& k) {
+    st[0] = k.alpha * st[0] + k.beta * gs;
+    return false;
+  }
+};
+
+// examples/test-adam.cu:14-38
+struct PseudoAdamMath : SumF32 {
+  static constexpr int NS = 3, UNROLL = 2;
+  static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
+  struct Prm { float lr, b1, omb1, b2, omb2; };
+  static __device__ __forceinline__ bool apply(Acc S0, float* st, uint16_t&, float&, const Prm& k) {
+    const float S2 = ((k.b2 * st[2]) + (k.omb2 * (S0 * S0)));
+    const float S4 = (S2 / k.b2);
+    const float S1 = ((k.b1 * st[1]) + (k.omb1 * S0));
+    const float S3 = (S1 / k.b1);
+    st[0] = (st[0] - ((k.lr * S3) / S4));
+    st[1] = S1;
+    st[2] = S2;
+    return false;
+  }
+};
+
+// nccl-overlap/samples/multi-process-adam-scattered.cpp:112-136
+struct AdamPrm {
+  float b1, omb1, b2, omb2, eps, stepsize, inv_scale;
+  double bc1, bc2;   // 1 - beta^t, evaluated in double on the host like the checker's pow()
+};
+__device__ __forceinline__ void adam_step(float gs, float* st, const AdamPrm& k) {
+  const float mi = k.b1 * st[1] + k.omb1 * gs;
+  const float vi = k.b2 * st[2] + k.omb2 * gs * gs;
+  const float m_ = (float)((double)mi / k.bc1);
+  const float v_ = (float)((double)vi / k.bc2);
+  const float x = k.stepsize * m_ / (sqrtf(v_) + k.eps);
+  st[0] = st[0] + x;
+  st[1] = mi;
+  st[2] = vi;
+}
+
+struct AdamMath : SumF32 {
+  static constexpr int NS = 3, UNROLL = 2;
+  static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
+  using Prm = AdamPrm;
+  static __device__ __forceinline__ bool apply(Acc gs, float* st, uint16_t&, float&, const Prm& k) {
+    adam_step(gs, st, k);
+    return false;
+  }
+};
+
+// fp16 gradients with a loss scale; overflow = any rank's element has exponent 0x1F.
+struct Adam16Math {
+  using G = uint16_t;
+  struct Acc { float s; bool bad; };
+  static constexpr int NS = 3, UNROLL = 1;
+  static constexpr bool OUT16 = true, OUTF = false, FLAG = true;
+  using Prm = AdamPrm;
+  static __device__ __forceinline__ Acc first(G h, const Prm& k) {
+    return Acc{f16_bits_to_f32(h) * k.inv_scale, (h & 0x7c00u) == 0x7c00u};
+  }
+  static __device__ __forceinline__ void next(Acc& a, G h, const Prm& k) {
+    a.s = a.s + f16_bits_to_f32(h) * k.inv_scale;
+    a.bad = a.bad | ((h & 0x7c00u) == 0x7c00u);
+  }
+  static __device__ __forceinline__ bool apply(Acc a, float* st, uint16_t& o16, float&, const Prm& k) {
+    if (!a.bad) adam_step(a.s, st, k);
+    o16 = f32_to_f16_bits(st[0]);
+    return a.bad;
+  }
+};
+
+struct Overflow16Math {
+  using G = uint16_t;
+  using Acc = bool;
+  static constexpr int NS = 0, UNROLL = 2;
+  static constexpr bool OUT16 = false, OUTF = false, FLAG = true;
+  struct Prm {};
+  static __device__ __forceinline__ Acc first(G h, const Prm&) { return (h & 0x7c00u) == 0x7c00u; }
+  static __device__ __forceinline__ void next(Acc& a, G h, const Prm&) { a = a | ((h & 0x7c00u) == 0x7c00u); }
+  static __device__ __forceinline__ bool apply(Acc a, float*, uint16_t&, float&, const Prm&) { return a; }
+};
+
+// nccl/src/collectives/device/reduce_kernel.h:36-68 in the call order of common_kernel.h:875-921
+struct FusedAdamRefMath {
+  using G = uint16_t;
+  using Acc = uint16_t;   // the ring carries the running sum in fp16
+  static constexpr int NS = 3, UNROLL = 1;
+  static constexpr bool OUT16 = true, OUTF = false, FLAG = false;
+  struct Prm { float lr, b1, b2, omb2; };
+  static __device__ __forceinline__ Acc first(G h, const Prm&) { return h; }
+  static __device__ __forceinline__ void next(Acc& a, G h, const Prm&) {
+    a = f32_to_f16_bits(f16_bits_to_f32(a) + f16_bits_to_f32(h));
+  }
+  static __device__ __forceinline__ bool apply(Acc S0, float* st, uint16_t& o16, float&, const Prm& k) {
+    const float s0f = f16_bits_to_f32(S0);
+    const float sq = f16_bits_to_f32(f32_to_f16_bits(s0f * s0f));           // S0*S0 evaluated in half
+    const float S2 = ((st[2] * k.b2) + (sq * k.omb2));
+    const float S4 = (S2 / k.b2);
+    const float S1 = ((st[1] * k.b2) + (s0f * k.omb2));                      // beta2 on the first moment, as the kernel
+    const float S3 = (S1 / k.b1);
+    const float S5 = ((S3 * k.lr) / sqrtf(S4));
+    st[2] = S2;
+    st[1] = S1;
+    st[0] = st[0] - S5;
+    o16 = f32_to_f16_bits(st[0]);
+    return false;
+  }
+};
+
+// ------------------------------------------------------------------------------------------------------------------
+// The streaming skeleton.  P > 0: rank count known at compile time (all P loads in flight together).
+// P == 0: rank count nP read at run time (ranks 9..16), loads folded one rank at a time.
+// VEC elements per thread per access; n counts elements.  Elements [ (n/VEC)*VEC, n ) are finished
+// by the first lanes of workgroup 0 with scalar accesses.
+// ------------------------------------------------------------------------------------------------------------------
+template <class M, int P>
+__device__ __forceinline__ void one_element(const SrcTable<typename M::G, (P ? P : CCN_MAX_RANKS)>& g, int nP,
+                                            const StateTable<M::NS>& st, uint16_t* out16, float* outf, size_t i,
+                                            const typename M::Prm& prm, bool& bad) {
+  const int np = P ? P : nP;
+  typename M::Acc a = M::first(g.p[0][i], prm);
+  for (int p = 1; p < np; p++) M::next(a, g.p[p][i], prm);
+  float s[M::NS > 0 ? M::NS : 1];
+#pragma unroll
+  for (int k = 0; k < M::NS; k++) s[k] = st.p[k][i];
+  uint16_t o16 = 0;
+  float of = 0.f;
+  bad |= M::apply(a, s, o16, of, prm);
+#pragma unroll
+  for (int k = 0; k < M::NS; k++) st.p[k][i] = s[k];
+  if constexpr (M::OUT16) out16[i] = o16;
+  if constexpr (M::OUTF) outf[i] = of;
+}
+
+template <class M, int P, int VEC, int UNROLL>
+__global__ __launch_bounds__(kBlock) void fused_stream_kernel(
+    const SrcTable<typename M::G, (P ? P : CCN_MAX_RANKS)> g, const int nP, const StateTable<M::NS> st,
+    uint16_t* out16, float* outf, uint32_t* flag, const size_t n, const typename M::Prm prm) {
+  using G = typename M::G;
+  constexpr int NSX = M::NS > 0 ? M::NS : 1;
+  constexpr int PX = P > 0 ? P : 1;
+  const size_t nvec = n / VEC;
+  const size_t tile = (size_t)kBlock * UNROLL;
+  bool bad = false;
+
+  for (size_t t0 = (size_t)blockIdx.x * tile; t0 < nvec; t0 += (size_t)gridDim.x * tile) {
+    Pack<G, VEC> gv[UNROLL][PX];
+    Pack<float, VEC> sv[UNROLL][NSX];
+    typename M::Acc acc[UNROLL][VEC];
+    // ---- issue every load of the tile -------------------------------------------------------------------------
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      const size_t e0 = (t0 + (size_t)u * kBlock + threadIdx.x) * VEC;   // first element of this thread's pack
+      if (e0 < nvec * VEC) {
+        if constexpr (P > 0) {
+#pragma unroll
+          for (int p = 0; p < P; p++) gv[u][p] = load_stream<G, VEC>(g.p[p] + e0);
+        }
+#pragma unroll
+        for (int k = 0; k < M::NS; k++) sv[u][k] = load_keep<float, VEC>(st.p[k] + e0);
+        if constexpr (P == 0) {
+          for (int p = 0; p < nP; p++) {
+            const Pack<G, VEC> x = load_stream<G, VEC>(g.p[p] + e0);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+              if (p == 0) acc[u][e] = M::first(x.d[e], prm);
+              else M::next(acc[u][e], x.d[e], prm);
+            }
+          }
+        }
+      }
+    }
+    // ---- fold, update, store ---------------------------------------------------------------------------------
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      const size_t e0 = (t0 + (size_t)u * kBlock + threadIdx.x) * VEC;
+      if (e0 < nvec * VEC) {
+        Pack<uint16_t, VEC> o16v;
+        Pack<float, VEC> ofv;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          if constexpr (P > 0) {
+            acc[u][e] = M::first(gv[u][0].d[e], prm);
+#pragma unroll
+            for (int p = 1; p < P; p++) M::next(acc[u][e], gv[u][p].d[e], prm);
+          }
+          float s[NSX];
+#pragma unroll
+          for (int k = 0; k < M::NS; k++) s[k] = sv[u][k].d[e];
+          uint16_t o16 = 0;
+          float of = 0.f;
+          bad |= M::apply(acc[u][e], s, o16, of, prm);
+#pragma unroll
+          for (int k = 0; k < M::NS; k++) sv[u][k].d[e] = s[k];
+          o16v.d[e] = o16;
+          ofv.d[e] = of;
+        }
+#pragma unroll
+        for (int k = 0; k < M::NS; k++) store_pack<float, VEC>(st.p[k] + e0, sv[u][k]);
+        if constexpr (M::OUT16) store_pack<uint16_t, VEC>(out16 + e0, o16v);
+        if constexpr (M::OUTF) store_pack<float, VEC>(outf + e0, ofv);
+      }
+    }
+  }
+
+  if constexpr (VEC > 1) {
+    const size_t rem = n - nvec * VEC;
+    if (blockIdx.x == 0 && threadIdx.x < rem) one_element<M, P>(g, nP, st, out16, outf, nvec * VEC + threadIdx.x, prm, bad);
+  }
+
+  if constexpr (M::FLAG) {
+    // one atomic per wavefront that saw a bad element (none in the common case)
+    if (__ballot(bad) != 0ull && (threadIdx.x & (kWave - 1)) == 0) atomicOr(flag, 1u);
+  }
+}
+
+__global__ void set_u32_kernel(uint32_t* p, uint32_t v) { *p = v; }
+
+__global__ __launch_bounds__(kBlock) void fill_f32_kernel(float* __restrict__ dst, float value, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) dst[i] = value;
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Host side: validation, alignment-based choice of the access width, dispatch on P.
+// ------------------------------------------------------------------------------------------------------------------
+template <class M, int P, int VEC, int UNROLL>
+static int launch_one(const typename M::G* const* g, int nP, const StateTable<M::NS>& st, uint16_t* out16, float* outf,
+                      uint32_t* flag, size_t n, const typename M::Prm& prm, hipStream_t s) {
+  SrcTable<typename M::G, (P ? P : CCN_MAX_RANKS)> tbl;
+  for (int p = 0; p < (P ? P : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < nP ? p : 0];
+  const size_t nvec = n / VEC;
+  const unsigned grid = stream_grid(nvec, (size_t)kBlock * UNROLL);
+  hipLaunchKernelGGL((fused_stream_kernel<M, P, VEC, UNROLL>), dim3(grid), dim3(kBlock), 0, s, tbl, nP, st, out16, outf,
+                     flag, n, prm);
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
+}
+
+template <class M, int VEC, int UNROLL>
+static int launch_p(const typename M::G* const* g, int P, const StateTable<M::NS>& st, uint16_t* out16, float* outf,
+                    uint32_t* flag, size_t n, const typename M::Prm& prm, hipStream_t s) {
+  switch (P) {
+#define CCN_CASE(K) case K: return launch_one<M, K, VEC, UNROLL>(g, P, st, out16, outf, flag, n, prm, s);
+    CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
+#undef CCN_CASE
+    default: return launch_one<M, 0, VEC, UNROLL>(g, P, st, out16, outf, flag, n, prm, s);
+  }
+}
+
+template <class M>
+static int launch(const typename M::G* const* g, int P, float* const* state, uint16_t* out16, float* outf,
+                  uint32_t* flag, size_t n, const typename M::Prm& prm, void* stream) {
+  if (!g || P < 1 || P > CCN_MAX_RANKS) return CCN_EINVAL;
+  for (int p = 0; p < P; p++) if (!g[p]) return CCN_EINVAL;
+  StateTable<M::NS> st;
+  st.p[0] = nullptr;
+  for (int k = 0; k < M::NS; k++) {
+    if (!state[k]) return CCN_EINVAL;
+    st.p[k] = state[k];
+  }
+  if (M::OUT16 && !out16) return CCN_EINVAL;
+  if (M::OUTF && !outf) return CCN_EINVAL;
+  if (M::FLAG && !flag) return CCN_EINVAL;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  if (M::FLAG) {
+    hipLaunchKernelGGL(set_u32_kernel, dim3(1), dim3(1), 0, s, flag, 0u);
+    CCN_HIP(hipGetLastError());
+  }
+  if (n == 0) return CCN_OK;
+
+  bool al = true;
+  for (int p = 0; p < P; p++) al = al && aligned16(g[p]);
+  for (int k = 0; k < M::NS; k++) al = al && aligned16(state[k]);
+  if (M::OUT16) al = al && aligned16(out16);
+  if (M::OUTF) al = al && aligned16(outf);
+  constexpr int VEC = 16 / (int)sizeof(typename M::G);
+  if (al) return launch_p<M, VEC, M::UNROLL>(g, P, st, out16, outf, flag, n, prm, s);
+  return launch_p<M, 1, 4>(g, P, st, out16, outf, flag, n, prm, s);
+}
+
+static AdamPrm make_adam_prm(float lr, float beta1, float beta2, float eps, int step, float inv_scale) {
+  AdamPrm k;
+  k.b1 = beta1;
+  k.omb1 = 1 - beta1;
+  k.b2 = beta2;
+  k.omb2 = 1 - beta2;
+  k.eps = eps;
+  k.stepsize = -lr;
+  k.inv_scale = inv_scale;
+  k.bc1 = 1 - std::pow((double)beta1, (double)step);
+  k.bc2 = 1 - std::pow((double)beta2, (double)step);
+  return k;
+}
+
+}  // namespace ccn
+
+using namespace ccn;
+
+extern "C" {
+
+int ccn_fill_f32(float* dst, float value, size_t n, void* stream) {
+  if (n == 0) return CCN_OK;
+  if (!dst) return CCN_EINVAL;
+  const unsigned grid = stream_grid(n, kBlock);
+  hipLaunchKernelGGL(fill_f32_kernel, dim3(grid), dim3(kBlock), 0, as_stream(stream), dst, value, n);
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
+}
+
+int ccn_reduce_f32(const float* const* g, int P, float* out, size_t N, void* stream) {
+  return launch<ReduceMath>(g, P, nullptr, nullptr, out, nullptr, N, ReduceMath::Prm{}, stream);
+}
+
+int ccn_sgd_f32(const float* const* g, int P, float* w, size_t N, float lr, void* stream) {
+  float* st[1] = {w};
+  return launch<SgdMath>(g, P, st, nullptr, nullptr, nullptr, N, SgdMath::Prm{lr}, stream);
+}
+
+int ccn_sgd_axpby_f32(const float* const* g, int P, float* w, size_t N, float alpha, float beta, void* stream) {
+  float* st[1] = {w};
+  return launch<AxpbyMath>(g, P, st, nullptr, nullptr, nullptr, N, AxpbyMath::Prm{alpha, beta}, stream);
+}
+
+int ccn_pseudo_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N, float lr, float beta1,
+                        float beta2, void* stream) {
+  float* st[3] = {w, m, v};
+  PseudoAdamMath::Prm k{lr, beta1, 1 - beta1, beta2, 1 - beta2};
+  return launch<PseudoAdamMath>(g, P, st, nullptr, nullptr, nullptr, N, k, stream);
+}
+
+int ccn_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N, float lr, float beta1,
+                 float beta2, float eps, int step, void* stream) {
+  if (step < 1) return CCN_EINVAL;
+  float* st[3] = {w, m, v};
+  return launch<AdamMath>(g, P, st, nullptr, nullptr, nullptr, N, make_adam_prm(lr, beta1, beta2, eps, step, 1.0f), stream);
+}
+
+int ccn_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16, size_t N, float lr,
+                  float beta1, float beta2, float eps, int step, float inv_scale, uint32_t* overflow_flag, void* stream) {
+  if (step < 1) return CCN_EINVAL;
+  float* st[3] = {w, m, v};
+  return launch<Adam16Math>(g, P, st, w16, nullptr, overflow_flag, N, make_adam_prm(lr, beta1, beta2, eps, step, inv_scale),
+                            stream);
+}
+
+int ccn_overflow_check_f16(const uint16_t* const* g, int P, size_t N, uint32_t* overflow_flag, void* stream) {
+  return launch<Overflow16Math>(g, P, nullptr, nullptr, nullptr, overflow_flag, N, Overflow16Math::Prm{}, stream);
+}
+
+int ccn_fused_adam_ref_f16g(const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v, size_t N,
+                            float lr, float beta1, float beta2, void* stream) {
+  float* st[3] = {w, m, v};
+  FusedAdamRefMath::Prm k{lr, beta1, beta2, 1 - beta2};
+  return launch<FusedAdamRefMath>(g, P, st, halfw, nullptr, nullptr, N, k, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,196 @@
+// Runtime glue of libcoconet_hip: device set-up, memory, streams, events, error strings.
+#include "ccn_common.hpp"
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+namespace ccn {
+
+thread_local int g_last_hip_error = 0;
+
+int hip_fail(hipError_t e) {
+  g_last_hip_error = (int)e;
+  (void)hipGetLastError();   // clear the sticky per-thread error so that later calls are not blamed for it
+  switch (e) {
+    case hipErrorOutOfMemory: return CCN_ENOMEM;
+    case hipErrorInvalidValue:
+    case hipErrorInvalidDevicePointer: return CCN_EINVAL;
+    case hipErrorNoDevice:
+    case hipErrorInvalidDevice: return CCN_ENODEV;
+    default: return CCN_EHIP;
+  }
+}
+
+namespace {
+constexpr int kMaxDevices = 16;
+DeviceInfo g_info[kMaxDevices];
+std::once_flag g_once[kMaxDevices];
+int g_init_rc[kMaxDevices];
+
+int query_device(int dev) {
+  hipDeviceProp_t prop;
+  CCN_HIP(hipGetDeviceProperties(&prop, dev));
+  DeviceInfo& di = g_info[dev];
+  di.cu_count = prop.multiProcessorCount;
+  di.hbm_bytes = prop.totalGlobalMem;
+  std::strncpy(di.arch, prop.gcnArchName, sizeof(di.arch) - 1);
+  if (std::strncmp(di.arch, "gfx950", 6) != 0) return CCN_ENODEV;   // the code object holds gfx950 ISA only
+  di.device = dev;
+  return CCN_OK;
+}
+}  // namespace
+
+int current_device_info(const DeviceInfo** out) {
+  int dev = -1;
+  CCN_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return CCN_ENODEV;
+  std::call_once(g_once[dev], [dev] { g_init_rc[dev] = query_device(dev); });
+  if (g_init_rc[dev] != CCN_OK) return g_init_rc[dev];
+  *out = &g_info[dev];
+  return CCN_OK;
+}
+
+unsigned stream_grid(size_t units, size_t tile) {
+  const DeviceInfo* di = nullptr;
+  int cus = 256;
+  if (current_device_info(&di) == CCN_OK) cus = di->cu_count;
+  // Workgroups per CU for the grid-stride loop.  8 x 256 threads = one full CU of wavefronts.
+  static const int per_cu = [] {
+    const char* e = std::getenv("CCN_BLOCKS_PER_CU");
+    int v = e ? std::atoi(e) : 8;
+    return v > 0 ? v : 8;
+  }();
+  size_t need = (units + tile - 1) / tile;
+  size_t cap = (size_t)cus * (size_t)per_cu;
+  if (need < 1) need = 1;
+  return (unsigned)(need < cap ? need : cap);
+}
+
+}  // namespace ccn
+
+using namespace ccn;
+
+extern "C" {
+
+int ccn_version(void) { return 1; }
+
+int ccn_init(int device) {
+  int count = 0;
+  CCN_HIP(hipGetDeviceCount(&count));
+  if (device < 0 || device >= count) return CCN_ENODEV;
+  CCN_HIP(hipSetDevice(device));
+  const DeviceInfo* di = nullptr;
+  return current_device_info(&di);
+}
+
+int ccn_device_info(int* cu_count, size_t* hbm_bytes, char* arch, size_t arch_len) {
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  if (cu_count) *cu_count = di->cu_count;
+  if (hbm_bytes) *hbm_bytes = di->hbm_bytes;
+  if (arch && arch_len) {
+    std::strncpy(arch, di->arch, arch_len - 1);
+    arch[arch_len - 1] = 0;
+  }
+  return CCN_OK;
+}
+
+int ccn_malloc(void** p, size_t bytes) {
+  if (!p) return CCN_EINVAL;
+  *p = nullptr;
+  if (bytes == 0) return CCN_OK;
+  CCN_HIP(hipMalloc(p, bytes));
+  return CCN_OK;
+}
+
+int ccn_free(void* p) {
+  if (!p) return CCN_OK;
+  CCN_HIP(hipFree(p));
+  return CCN_OK;
+}
+
+int ccn_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return CCN_OK;
+  if (!dst || !src) return CCN_EINVAL;
+  CCN_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+  return CCN_OK;
+}
+
+int ccn_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return CCN_OK;
+  if (!dst || !src) return CCN_EINVAL;
+  CCN_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+  CCN_HIP(hipStreamSynchronize(as_stream(stream)));
+  return CCN_OK;
+}
+
+int ccn_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return CCN_OK;
+  if (!dst || !src) return CCN_EINVAL;
+  CCN_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+  return CCN_OK;
+}
+
+int ccn_stream_create(void** stream) {
+  if (!stream) return CCN_EINVAL;
+  hipStream_t s;
+  CCN_HIP(hipStreamCreate(&s));   // default priority only
+  *stream = (void*)s;
+  return CCN_OK;
+}
+
+int ccn_stream_destroy(void* stream) {
+  if (!stream) return CCN_OK;
+  CCN_HIP(hipStreamDestroy(as_stream(stream)));
+  return CCN_OK;
+}
+
+int ccn_stream_sync(void* stream) {
+  CCN_HIP(hipStreamSynchronize(as_stream(stream)));
+  return CCN_OK;
+}
+
+int ccn_event_create(void** ev) {
+  if (!ev) return CCN_EINVAL;
+  hipEvent_t e;
+  CCN_HIP(hipEventCreate(&e));
+  *ev = (void*)e;
+  return CCN_OK;
+}
+
+int ccn_event_destroy(void* ev) {
+  if (!ev) return CCN_OK;
+  CCN_HIP(hipEventDestroy((hipEvent_t)ev));
+  return CCN_OK;
+}
+
+int ccn_event_record(void* ev, void* stream) {
+  if (!ev) return CCN_EINVAL;
+  CCN_HIP(hipEventRecord((hipEvent_t)ev, as_stream(stream)));
+  return CCN_OK;
+}
+
+int ccn_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!start || !stop || !ms) return CCN_EINVAL;
+  CCN_HIP(hipEventSynchronize((hipEvent_t)stop));
+  CCN_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return CCN_OK;
+}
+
+int ccn_last_hip_error(void) { return g_last_hip_error; }
+
+const char* ccn_strerror(int code) {
+  switch (code) {
+    case CCN_OK: return "success";
+    case CCN_EINVAL: return "invalid argument (null pointer, zero size, rank count out of range, bad mode or misaligned buffer)";
+    case CCN_ENOMEM: return "out of device memory";
+    case CCN_ENODEV: return "no such device, or the device is not gfx950";
+    case CCN_EHIP: return "HIP runtime error (see ccn_last_hip_error)";
+    case CCN_ERANGE: return "size out of the supported range";
+    default: return "unknown error code";
+  }
+}
+
+}  // extern "C"

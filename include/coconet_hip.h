@@ -1,0 +1,158 @@
+/*
+ * coconet_hip.h -- C ABI of libcoconet_hip.so: the MI355X (gfx950) backend for CoCoNet's fused
+ * "reduce P rank-gradient buffers + optimizer update" kernels and the model-parallel GEMM epilogue.
+ *
+ * Boundary.  In the reference, generated programs reach this functionality through entry points of a
+ * modified NCCL (AllReduce_pipe, ncclAllReduceScatteredAdam, ...) and through emitted CUDA kernels.
+ * On one GPU the collective degenerates to a local multi-operand reduce, so each entry point here takes
+ * a host table of P device pointers (one gradient buffer per simulated rank) instead of a communicator.
+ *
+ * Conventions
+ *   - plain C types only; every pointer named g/w/m/v/... is a DEVICE pointer unless marked "host".
+ *   - `g` is a HOST array of P device pointers; it is read during the call and may be freed afterwards.
+ *   - gradient buffers are read-only (the reference clobbers them; callers must not rely on that).
+ *   - w, m, v are updated in place.
+ *   - calls are asynchronous: work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     null stream); the caller synchronises.  No entry point calls exit(); errors are returned.
+ *   - return value: 0 on success, a negative CCN_E* code otherwise (ccn_strerror() names it).
+ *   - gradient sum order is fixed: ((g[0]+g[1])+g[2])+... in fp32, no fused multiply-add anywhere.
+ *   - thread-compatible: concurrent calls on different streams are allowed; ccn_init is idempotent.
+ */
+#ifndef COCONET_HIP_H
+#define COCONET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CCN_OK        0
+#define CCN_EINVAL  (-22)  /* null pointer, N == 0 where not allowed, P out of range, bad mode, misaligned bf16/fp16 buffer */
+#define CCN_ENOMEM  (-12)  /* hipMalloc failed */
+#define CCN_ENODEV  (-19)  /* no such device / not a gfx950 device */
+#define CCN_EHIP     (-5)  /* any other HIP runtime error (ccn_last_hip_error() gives the hipError_t) */
+#define CCN_ERANGE  (-34)  /* size beyond what the kernel supports */
+
+#define CCN_MAX_RANKS 16   /* 1 <= P <= CCN_MAX_RANKS */
+
+#define CCN_LAMB_TRUST_RATIO 0  /* scale = W/R                         (textbook)                      */
+#define CCN_LAMB_REFERENCE   1  /* scale = (W/R)/R  as the reference's kernel and checker compute it   */
+
+/* ---- runtime glue: what the generated driver needs instead of cudaMalloc / events
+ *      (reference: emitted main(), src/codegen.cpp:4583-4784; examples/header.h:36-53) ---- */
+int  ccn_version(void);
+int  ccn_init(int device);                       /* hipSetDevice + device query; idempotent */
+int  ccn_device_info(int* cu_count, size_t* hbm_bytes, char* arch, size_t arch_len);
+int  ccn_malloc(void** p, size_t bytes);
+int  ccn_free(void* p);
+int  ccn_memcpy_h2d(void* dst, const void* src_host, size_t bytes, void* stream);
+int  ccn_memcpy_d2h(void* dst_host, const void* src, size_t bytes, void* stream);
+int  ccn_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+int  ccn_fill_f32(float* dst, float value, size_t n, void* stream);    /* memset_value, examples/header.h:85-101 */
+int  ccn_stream_create(void** stream);
+int  ccn_stream_destroy(void* stream);
+int  ccn_stream_sync(void* stream);
+int  ccn_event_create(void** ev);
+int  ccn_event_destroy(void* ev);
+int  ccn_event_record(void* ev, void* stream);
+int  ccn_event_elapsed_ms(void* start, void* stop, float* ms);        /* synchronises on `stop` */
+int  ccn_last_hip_error(void);
+const char* ccn_strerror(int code);
+
+/* ---- plain P-way reduce: out[i] = sum_p g[p][i].
+ *      Replaces the stock ncclAllReduce of the unfused schedules (src/codegen.cpp:4146-4189;
+ *      device loop nccl/src/collectives/device/common_kernel.h:1310-1427 ReduceOrCopyMulti).
+ *      `out` may alias g[0] (in-place, as the reference's all-reduce). ---- */
+int  ccn_reduce_f32(const float* const* g, int P, float* out, size_t N, void* stream);
+
+/* ---- SGD: w <- w - lr * sum_p g[p].
+ *      Replaces AllReduce_pipe(lr, g, w, SZ, ...) of the sgd example (examples/test-sgd.cu:3;
+ *      checker :17-18) and the emitted kernel of examples/sgd/sgd.cpp:14-15. ---- */
+int  ccn_sgd_f32(const float* const* g, int P, float* w, size_t N, float lr, void* stream);
+
+/* ---- SGD, axpby form: w <- alpha*w + beta*sum_p g[p].
+ *      Replaces ncclAllReduce2 / the SGD branch of ReduceCopy128bMulti
+ *      (nccl-overlap/src/collectives/device/common_kernel.h:969-986; checker
+ *      nccl-overlap/samples/single-process-wX.cu:141). ---- */
+int  ccn_sgd_axpby_f32(const float* const* g, int P, float* w, size_t N, float alpha, float beta, void* stream);
+
+/* ---- the adam example as the DSL states it (no sqrt, divides by beta instead of bias correction):
+ *      v <- beta2*v + (1-beta2)*gs*gs; m <- beta1*m + (1-beta1)*gs; w <- w - (lr*(m/beta1))/(v/beta2).
+ *      Replaces AllReduce_pipe(lr,beta1,beta2,g,w,m,v,SZ,...) of examples/test-adam.cu:3 (checker :14-38). ---- */
+int  ccn_pseudo_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
+                         float lr, float beta1, float beta2, void* stream);
+
+/* ---- bias-corrected Adam, fp32:  step >= 1 is the 1-based step number t (the reference passes epoch = t-1).
+ *      m <- b1*m + (1-b1)*gs;  v <- b2*v + (1-b2)*gs*gs;  w <- w - lr * (m/(1-b1^t)) / (sqrt(v/(1-b2^t)) + eps)
+ *      Replaces ncclAllReduceScatteredAdam / ncclAllReduceAdam
+ *      (nccl-overlap/src/collectives/all_reduce.cc:47-60, :142-155; device math
+ *      nccl-overlap/src/collectives/device/common_kernel.h:905-968; checker
+ *      nccl-overlap/samples/multi-process-adam-scattered.cpp:112-136).  The reference's stepsize
+ *      alpha corresponds to -lr and its hard-coded epsilon 1e-6 to `eps`. ---- */
+int  ccn_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
+                  float lr, float beta1, float beta2, float eps, int step, void* stream);
+
+/* ---- mixed-precision Adam: fp16 gradients carrying a loss scale, fp32 master state, fp16 weight copy.
+ *      gs = sum_p float(g[p][i])*inv_scale.  overflow_flag (device, one uint32) is SET by the call:
+ *      1 if any g[p][i] is inf/nan, else 0.  Elements whose gradients overflow keep w, m, v unchanged;
+ *      all other elements take the Adam step above; w16[i] = fp16(w[i]) is written for every element.
+ *      Takes the place of the mixed-precision AllReduce_pipe(lr,b1,b2,(half*)g,w,(half*)halfw,m,v,count,...)
+ *      (nccl/src/nccl.h.in:212; nccl/src/collectives/device/common_kernel.h:830-1172), which has no
+ *      loss scaling or overflow detection; those semantics are defined by this library. ---- */
+int  ccn_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16, size_t N,
+                   float lr, float beta1, float beta2, float eps, int step, float inv_scale,
+                   uint32_t* overflow_flag, void* stream);
+
+/* ---- overflow pre-check for callers that want all-or-nothing steps: *overflow_flag <- any(!isfinite(g)). ---- */
+int  ccn_overflow_check_f16(const uint16_t* const* g, int P, size_t N, uint32_t* overflow_flag, void* stream);
+
+/* ---- the modified NCCL's fused mixed-precision Adam exactly as its kernel computes it (fp16 gradient sum,
+ *      square taken in fp16, first moment decayed with beta2, no eps):
+ *      nccl/src/collectives/device/reduce_kernel.h:36-68, common_kernel.h:875-921.
+ *      Same signature shape as AllReduce_pipe (nccl/src/nccl.h.in:212). ---- */
+int  ccn_fused_adam_ref_f16g(const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
+                             size_t N, float lr, float beta1, float beta2, void* stream);
+
+/* ---- LAMB with per-segment ("per-layer", the reference's "parent buffer") norms; two passes.
+ *      A plan owns the device-side segment tables and the norm partials for one segmentation of [0,N).
+ *      seg_offsets: HOST array of nseg+1 ascending element offsets, seg_offsets[0]==0, last == N.
+ *      pass 1: m,v update; r = mhat/(sqrt(vhat)+eps) + wd*w; per-segment sum w^2, sum r^2 in float64
+ *      finalize: W_b = sqrt(sum w^2 / n_b), R_b = sqrt(sum r^2 / n_b), scale_b (see CCN_LAMB_*)
+ *      pass 2: w <- w - (lr*scale_b)*r   (r recomputed from m, v, w; no r buffer is needed)
+ *      Replaces ncclAllReduceScatteredLAMB (nccl-overlap/src/collectives/all_reduce.cc:61-76; kernel
+ *      nccl-overlap/src/collectives/device/all_reduce_scattered.h:107-262; checker
+ *      nccl-overlap/samples/multi-process-adam-scattered.cpp:402-449).  wd = 1.0f is the reference. ---- */
+typedef struct ccn_lamb_plan ccn_lamb_plan;
+int  ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** plan);
+int  ccn_lamb_plan_destroy(ccn_lamb_plan* plan);
+int  ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, float* m, float* v,
+                  float lr, float beta1, float beta2, float eps, float wd, int step, int mode, void* stream);
+/* copies W_b, R_b of the last ccn_lamb_f32 on this plan to a HOST array of 2*nseg doubles (synchronises) */
+int  ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream);
+
+/* ---- model-parallel MLP out-projection, one rank's K-slice, epilogue fused into the GEMM write-back:
+ *      out = bf16( dropout( X[MxK].W[KxN] + sum_q partials[q] + bias[col] ) + resid )
+ *      X, W, resid, out: bf16 bit patterns, row-major; partials: HOST array of nPartials device pointers to
+ *      fp32 [MxN]; bias fp32 [N]; resid may be NULL.  Dropout: element idx=row*N+col is dropped when
+ *      u(seed, idx) < p_drop, survivors are scaled by 1/(1-p_drop); u comes from Philox-4x32-10 with
+ *      counter (idx/4, 0) and key seed, word idx%4, u = (word>>8)*2^-24.
+ *      Replaces MatMul + AllReduce + (sum+b) + Dropout + r of examples/model-parallel/model-parallel.cpp:18-21
+ *      (emitted cublasGemmEx src/codegen.cpp:1058-1136; fused epilogue
+ *      nccl-overlap/src/collectives/device/common_kernel.h:1037-1057, reduce_kernel.h:192-213). ---- */
+int  ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                          const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K,
+                          float p_drop, uint64_t seed, void* stream);
+
+/* ---- standalone epilogue on an fp32 [MxN] product already in memory (the unfused schedule):
+ *      out = bf16( dropout( acc + sum_q partials[q] + bias[col] ) + resid ).
+ *      Replaces ncclAllReduceDropoutBiasLayernorm (nccl-overlap/src/collectives/all_reduce.cc:78-90). ---- */
+int  ccn_bias_dropout_residual(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                               const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                               void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COCONET_HIP_H */

@@ -1,0 +1,359 @@
+/*
+ * ccn_oracle.c -- CPU oracle (test infrastructure, never shipped in the product library).
+ * See ccn_oracle.h for the conventions and for what pins each routine.
+ * Build: gcc -O2 -ffp-contract=off -fPIC -shared (see Makefile); -ffp-contract=off is load-bearing.
+ */
+#include "ccn_oracle.h"
+#include <math.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------------------------------
+ * conversions
+ * ---------------------------------------------------------------------------------------------- */
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* fp32 -> fp16, round-to-nearest-even; the rounding the reference obtains from __floats2half2_rn
+ * (nccl/src/collectives/device/common_kernel.h:655-670). */
+uint16_t orc_f32_to_f16(float f) {
+  uint32_t x = f2u(f);
+  uint32_t sign = (x >> 16) & 0x8000u;
+  uint32_t absx = x & 0x7fffffffu;
+  if (absx >= 0x7f800000u) {                       /* inf / nan */
+    if (absx > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((absx >> 13) & 0x3ffu));
+    return (uint16_t)(sign | 0x7c00u);
+  }
+  if (absx >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);   /* >= 65520 rounds to inf */
+  if (absx < 0x33000001u) return (uint16_t)sign;                /* <= 2^-25 rounds to zero (tie -> even 0) */
+  int32_t e = (int32_t)(absx >> 23) - 127;                      /* unbiased exponent */
+  uint32_t mant = (absx & 0x7fffffu) | 0x800000u;               /* 24-bit significand */
+  int shift;                                                    /* bits dropped from the significand */
+  uint32_t hexp;
+  if (e < -14) { shift = 13 + (-14 - e); hexp = 0; }            /* subnormal half */
+  else         { shift = 13;             hexp = (uint32_t)(e + 15); }
+  uint32_t kept = mant >> shift;
+  uint32_t rem  = mant & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (kept & 1u))) kept++;
+  uint32_t h;
+  if (hexp == 0) h = kept;                                      /* may carry into exponent 1: correct */
+  else           h = ((hexp - 1) << 10) + kept;                 /* kept includes the hidden bit (0x400) */
+  return (uint16_t)(sign | h);
+}
+
+float orc_f16_to_f32(uint16_t h) {
+  uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1fu;
+  uint32_t m = h & 0x3ffu;
+  if (e == 0x1f) return u2f(sign | 0x7f800000u | (m << 13));
+  if (e == 0) {
+    if (m == 0) return u2f(sign);
+    /* subnormal: m * 2^-24 */
+    float v = (float)m * 5.9604644775390625e-08f;
+    return (sign ? -v : v);
+  }
+  return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+uint16_t orc_f32_to_bf16(float f) {
+  uint32_t x = f2u(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);  /* quiet nan */
+  uint32_t lsb = (x >> 16) & 1u;
+  x += 0x7fffu + lsb;
+  return (uint16_t)(x >> 16);
+}
+
+float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+void orc_f32_to_f16_array(const float* s, uint16_t* d, size_t n) { for (size_t i = 0; i < n; i++) d[i] = orc_f32_to_f16(s[i]); }
+void orc_f16_to_f32_array(const uint16_t* s, float* d, size_t n) { for (size_t i = 0; i < n; i++) d[i] = orc_f16_to_f32(s[i]); }
+void orc_f32_to_bf16_array(const float* s, uint16_t* d, size_t n) { for (size_t i = 0; i < n; i++) d[i] = orc_f32_to_bf16(s[i]); }
+void orc_bf16_to_f32_array(const uint16_t* s, float* d, size_t n) { for (size_t i = 0; i < n; i++) d[i] = orc_bf16_to_f32(s[i]); }
+
+/* ------------------------------------------------------------------------------------------------
+ * comparators
+ * ---------------------------------------------------------------------------------------------- */
+/* examples/header.h:52-62  absRelDiff / eqFloat */
+int orc_eqFloat_1e3(float u, float v) {
+  if (u == 0.0f || v == 0.0f) return u == v;
+  return fabsf((u - v) / u) <= 1e-3;
+}
+/* nccl-overlap/samples/multi-process-adam-scattered.cpp:60-66  eq_float */
+int orc_eq_float_1e5(float f1, float f2) {
+  if (f1 == 0.0f && f2 == 0.0f) return 1;
+  float mx = f1 > f2 ? f1 : f2;
+  return fabs((f1 - f2) / mx) <= 1e-5;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * reduce / SGD
+ * ---------------------------------------------------------------------------------------------- */
+static inline float reduce_at(const float* const* g, int P, size_t i) {
+  float s = g[0][i];
+  for (int p = 1; p < P; p++) s = s + g[p][i];
+  return s;
+}
+
+void orc_reduce_f32(const float* const* g, int P, size_t N, float* out) {
+  for (size_t i = 0; i < N; i++) out[i] = reduce_at(g, P, i);
+}
+
+/* examples/test-sgd.cu:17-18   __S1[i0] = (__w[i0] - (__lr * __S0[i0])) */
+void orc_sgd_f32(const float* const* g, int P, float* w, size_t N, float lr) {
+  for (size_t i = 0; i < N; i++) {
+    float s0 = reduce_at(g, P, i);
+    w[i] = (w[i] - (lr * s0));
+  }
+}
+
+/* nccl-overlap/samples/single-process-wX.cu:141   new_weight = alpha * w + beta * reduced_grad */
+void orc_sgd_axpby_f32(const float* const* g, int P, float* w, size_t N, float alpha, float beta) {
+  for (size_t i = 0; i < N; i++) {
+    float s0 = reduce_at(g, P, i);
+    w[i] = alpha * w[i] + beta * s0;
+  }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * examples/test-adam.cu:14-38  (the saved checker of the DSL's adam example)
+ *   S2 = beta2*v + (1-beta2)*(S0*S0);  S4 = S2/beta2;  S1 = beta1*m + (1-beta1)*S0;  S3 = S1/beta1;
+ *   S5 = w - (lr*S3)/S4
+ * The DSL program declares m and v as Update targets (examples/adam/adam.cpp:18-23), so S1 and S2
+ * are stored back.
+ * ---------------------------------------------------------------------------------------------- */
+void orc_pseudo_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
+                         float lr, float beta1, float beta2) {
+  for (size_t i = 0; i < N; i++) {
+    float S0 = reduce_at(g, P, i);
+    float S2 = ((beta2 * v[i]) + ((1 - beta2) * (S0 * S0)));
+    float S4 = (S2 / beta2);
+    float S1 = ((beta1 * m[i]) + ((1 - beta1) * S0));
+    float S3 = (S1 / beta1);
+    float S5 = (w[i] - ((lr * S3) / S4));
+    v[i] = S2; m[i] = S1; w[i] = S5;
+  }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * The modified NCCL's fused mixed-precision "Adam":
+ *   functors  nccl/src/collectives/device/reduce_kernel.h:36-68
+ *   call order nccl/src/collectives/device/common_kernel.h:875-887, fp16 store :910-921
+ * Faithful to the kernel, including: gradient sum carried in fp16 (__hadd2 chain), the square taken
+ * in fp16, and the first moment updated with beta2 in place of beta1 (the kernel invokes the
+ * mixedbinOp3 functor through .mixedbinOp1(beta2, ...)).
+ * ---------------------------------------------------------------------------------------------- */
+static inline uint16_t hadd(uint16_t a, uint16_t b) { return orc_f32_to_f16(orc_f16_to_f32(a) + orc_f16_to_f32(b)); }
+static inline uint16_t hmul(uint16_t a, uint16_t b) { return orc_f32_to_f16(orc_f16_to_f32(a) * orc_f16_to_f32(b)); }
+
+void orc_fused_adam_a3(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* halfw,
+                       size_t N, float lr, float beta1, float beta2) {
+  for (size_t i = 0; i < N; i++) {
+    uint16_t S0 = g[0][i];
+    for (int p = 1; p < P; p++) S0 = hadd(S0, g[p][i]);
+    float S2 = ((v[i] * beta2) + ((orc_f16_to_f32(hmul(S0, S0))) * (1 - beta2)));   /* mixedbinOp1 */
+    float S4 = (S2 / beta2);                                                         /* binOp2 */
+    float S1 = ((m[i] * beta2) + ((orc_f16_to_f32(S0)) * (1 - beta2)));              /* mixedbinOp3 called with beta2 */
+    float S3 = (S1 / beta1);                                                         /* binOp2 with beta1 */
+    float S5 = ((S3 * lr) / sqrtf(S4));                                              /* delta */
+    v[i] = S2; m[i] = S1;
+    float fw = w[i] - S5;                                                            /* weightUpdate */
+    w[i] = fw;
+    halfw[i] = orc_f32_to_f16(fw);
+  }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * nccl-overlap/samples/multi-process-adam-scattered.cpp:112-136  (check_epoch_results_adam, T=float)
+ *   m  = beta1*old_m + (1-beta1)*gs
+ *   v  = beta2*old_v + (1-beta2)*gs*gs                  -- ((1-beta2)*gs)*gs, left to right
+ *   m_ = m/(1 - pow(beta1, epoch+1))                     -- pow and the division are double, result float
+ *   v_ = v/(1 - pow(beta2, epoch+1))
+ *   x  = stepsize * m_ / (sqrt(v_) + epsilon)            -- (stepsize*m_) / (sqrtf(v_)+eps), fp32
+ *   w  = w + x
+ * The reference passes stepsize = +alpha; BASELINE's "w -= lr*..." is stepsize = -lr, which is the
+ * same fp32 result as subtracting (negation is exact).
+ * sqrt: the unqualified call resolves to the float overload when the C++ <math.h> wrapper is in
+ * scope (it is pulled in by the CUDA runtime header); the device functor computes
+ * (float)sqrt((double)v_), which is the same correctly rounded value.
+ * ---------------------------------------------------------------------------------------------- */
+void orc_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
+                  float lr, float beta1, float beta2, float eps, int step) {
+  const double bc1 = 1 - pow((double)beta1, (double)step);
+  const double bc2 = 1 - pow((double)beta2, (double)step);
+  const float stepsize = -lr;
+  for (size_t i = 0; i < N; i++) {
+    float gs = reduce_at(g, P, i);
+    float mi = beta1 * m[i] + (1 - beta1) * gs;
+    float vi = beta2 * v[i] + (1 - beta2) * gs * gs;
+    float m_ = (float)((double)mi / bc1);
+    float v_ = (float)((double)vi / bc2);
+    float x = stepsize * m_ / (sqrtf(v_) + eps);
+    w[i] = w[i] + x;
+    m[i] = mi;
+    v[i] = vi;
+  }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Mixed-precision Adam with loss-scale removal and overflow detection.  The reference has neither
+ * (its only mention of an overflow buffer is the Apex baseline script, experiments/optimbench.py:61-81),
+ * so the semantics are defined by this build:
+ *   - element i "overflows" when any g[p][i] has fp16 exponent 0x1F (inf or nan);
+ *     flag = OR over all elements and ranks;
+ *   - gs = sum_p ( float(g[p][i]) * inv_scale ), fp32, p ascending (unscale before the sum);
+ *   - an overflowing element leaves w, m, v untouched (the optimizer state is never poisoned);
+ *     every other element takes the Adam step of orc_adam_f32;
+ *   - w16[i] = fp16_rne(w[i]) is written for every element.
+ * ---------------------------------------------------------------------------------------------- */
+uint32_t orc_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16,
+                       size_t N, float lr, float beta1, float beta2, float eps, int step, float inv_scale) {
+  const double bc1 = 1 - pow((double)beta1, (double)step);
+  const double bc2 = 1 - pow((double)beta2, (double)step);
+  const float stepsize = -lr;
+  uint32_t flag = 0;
+  for (size_t i = 0; i < N; i++) {
+    int bad = 0;
+    float gs = 0.0f;
+    for (int p = 0; p < P; p++) {
+      uint16_t h = g[p][i];
+      if ((h & 0x7c00u) == 0x7c00u) bad = 1;
+      float t = orc_f16_to_f32(h) * inv_scale;
+      gs = (p == 0) ? t : gs + t;
+    }
+    if (bad) {
+      flag = 1;
+    } else {
+      float mi = beta1 * m[i] + (1 - beta1) * gs;
+      float vi = beta2 * v[i] + (1 - beta2) * gs * gs;
+      float m_ = (float)((double)mi / bc1);
+      float v_ = (float)((double)vi / bc2);
+      float x = stepsize * m_ / (sqrtf(v_) + eps);
+      w[i] = w[i] + x;
+      m[i] = mi;
+      v[i] = vi;
+    }
+    w16[i] = orc_f32_to_f16(w[i]);
+  }
+  return flag;
+}
+
+uint32_t orc_overflow_f16(const uint16_t* const* g, int P, size_t N) {
+  for (int p = 0; p < P; p++)
+    for (size_t i = 0; i < N; i++)
+      if ((g[p][i] & 0x7c00u) == 0x7c00u) return 1;
+  return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * nccl-overlap/samples/multi-process-adam-scattered.cpp:402-449 (check_epoch_results_lamb, T=float),
+ * applied once per segment ("parent buffer"):
+ *   first loop : m, v as Adam;  r = m_/(sqrt(v_)+eps) + 1.0f*w;
+ *                rNorm += (r*r)/n   (fp32 quotient, double accumulator);  wNorm += w*w (fp32 product)
+ *   rNorm = sqrt(rNorm);  wNorm = sqrt(wNorm/n)
+ *   second loop: r recomputed from the stored m, v;
+ *                scale = (float)( ((wNorm>0) ? (rNorm>0 ? wNorm/rNorm : 1) : 1) / rNorm )
+ *                w = w - (stepsize*scale)*r
+ * The hard-coded 1.0f is the weight-decay factor wd here (wd = 1.0f reproduces the reference bit for bit).
+ * mode 1 keeps the reference's second division by rNorm; mode 0 drops it (textbook trust ratio).
+ * ---------------------------------------------------------------------------------------------- */
+void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
+                  const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2,
+                  float eps, float wd, int step, int mode, double* norms_out) {
+  const double bc1 = 1 - pow((double)beta1, (double)step);
+  const double bc2 = 1 - pow((double)beta2, (double)step);
+  const float stepsize = lr;
+  for (int b = 0; b < nseg; b++) {
+    const size_t lo = seg_offsets[b], hi = seg_offsets[b + 1];
+    const uint64_t n = (uint64_t)(hi - lo);
+    double rNorm = 0.0, wNorm = 0.0;
+    for (size_t i = lo; i < hi; i++) {
+      float gs = reduce_at(g, P, i);
+      float mi = beta1 * m[i] + (1 - beta1) * gs;
+      float vi = beta2 * v[i] + (1 - beta2) * gs * gs;
+      float m_ = (float)((double)mi / bc1);
+      float v_ = (float)((double)vi / bc2);
+      float r = m_ / (sqrtf(v_) + eps) + wd * w[i];
+      rNorm += (r * r) / (float)n;
+      wNorm += (w[i] * w[i]);
+      v[i] = vi;
+      m[i] = mi;
+    }
+    rNorm = sqrt(rNorm);
+    wNorm = sqrt(wNorm / (double)n);
+    if (norms_out) { norms_out[2 * b] = wNorm; norms_out[2 * b + 1] = rNorm; }
+    double ratio = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f);
+    float scale = (float)(mode == 1 ? ratio / rNorm : ratio);
+    for (size_t i = lo; i < hi; i++) {
+      float m_ = (float)((double)m[i] / bc1);
+      float v_ = (float)((double)v[i] / bc2);
+      float r = m_ / (sqrtf(v_) + eps) + wd * w[i];
+      float x = stepsize * scale * r;
+      w[i] = w[i] - x;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Philox-4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11)
+ * ---------------------------------------------------------------------------------------------- */
+void orc_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
+  uint32_t k0 = key[0], k1 = key[1];
+  for (int r = 0; r < 10; r++) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* Dropout mask, build-defined (the reference's mask is curand_init(0,0,0) evaluated identically for
+ * every element, src/codegen.cpp:634-640, which is degenerate):
+ *   block = idx/4 -> Philox counter (lo, hi, 0, 0), key = (seed lo, seed hi), word = out[idx%4];
+ *   u = (word >> 8) * 2^-24 in [0,1);  keep <=> u >= p_drop. */
+int orc_dropout_keep(uint64_t seed, uint64_t idx, float p_drop) {
+  uint64_t blk = idx >> 2;
+  uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u};
+  uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  uint32_t out[4];
+  orc_philox4x32_10(ctr, key, out);
+  float u = (float)(out[idx & 3] >> 8) * 5.9604644775390625e-08f;
+  return u >= p_drop;
+}
+
+void orc_dropout_mask(uint64_t seed, uint64_t first_idx, size_t n, float p_drop, uint8_t* keep) {
+  for (size_t i = 0; i < n; i++) keep[i] = (uint8_t)orc_dropout_keep(seed, first_idx + i, p_drop);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * MLP out-projection with fused epilogue.  DSL shape: examples/model-parallel/model-parallel.cpp:18-21
+ *   layer = MatMul(in, w); sum = AllReduce(layer); sum2 = sum + b; out = Dropout(sum2, p) + r
+ * On one GPU the all-reduce is "own product + (P-1) partial products of the peers".
+ * Dropout here is the standard one (drop with probability p, survivors scaled by 1/(1-p)); the
+ * reference keeps with probability p and does not rescale (src/codegen.cpp:634-640).
+ * ---------------------------------------------------------------------------------------------- */
+void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                     const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                     int M, int N, int K, float p_drop, uint64_t seed) {
+  const float scale = 1.0f / (1.0f - p_drop);
+  for (int i = 0; i < M; i++) {
+    for (int j = 0; j < N; j++) {
+      double acc = 0.0;
+      for (int k = 0; k < K; k++)
+        acc += (double)orc_bf16_to_f32(X[(size_t)i * K + k]) * (double)orc_bf16_to_f32(W[(size_t)k * N + j]);
+      float s = (float)acc;
+      size_t idx = (size_t)i * N + j;
+      for (int q = 0; q < nPartials; q++) s = s + partials[q][idx];
+      float t = s + bias[j];
+      float d = orc_dropout_keep(seed, idx, p_drop) ? t * scale : 0.0f;
+      float y = d + (resid ? orc_bf16_to_f32(resid[idx]) : 0.0f);
+      if (out_f32) out_f32[idx] = y;
+      if (out) out[idx] = orc_f32_to_bf16(y);
+    }
+  }
+}

@@ -1,0 +1,105 @@
+/*
+ * ccn_oracle.h -- CPU oracle for the fused reduce+update path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This is a scalar C restatement of the host-side checker loops that the reference
+ * (parasailteam/coconet) uses to validate its fused all-reduce + optimizer kernels.  It is the
+ * checker for the HIP kernels of this repository and the "cpu_baseline" leg of bench.py; the product
+ * library (libcoconet_hip.so) never links, loads or calls it.
+ *
+ * Conventions shared by every routine:
+ *   - "P rank-gradient buffers": g[0..P-1] are P arrays of N elements; the all-reduce of the
+ *     reference becomes gs[i] = (((g[0][i] + g[1][i]) + g[2][i]) + ... ) in fp32, p ascending.
+ *     (MPI_Allreduce in the reference checkers leaves the order open; the oracle fixes it.)
+ *   - compile with -O2 -ffp-contract=off: no fused multiply-add may be formed.
+ *   - state (w, m, v) is updated in place; g is read-only.
+ *
+ * Pin status per routine (what independent evidence the tests hold for it):
+ *   orc_reduce_f32        closed form on integers, permutation bound            pinned
+ *   orc_sgd_f32           examples/test-sgd.cu:17-18; numpy axpy identity       pinned
+ *   orc_sgd_axpby_f32     nccl-overlap/samples/single-process-wX.cu:141        pinned (numpy identity)
+ *   orc_pseudo_adam_f32   examples/test-adam.cu:14-38; known answer w=-1/P      pinned
+ *   orc_fused_adam_a3     nccl/.../reduce_kernel.h:36-68 functors; known answer w=-1, half 0xBC00   pinned
+ *   orc_adam_f32          nccl-overlap/samples/multi-process-adam-scattered.cpp:112-136;
+ *                         reference integer fixture, torch.optim.Adam (CPU) cross-check, step-1 closed form   pinned
+ *   orc_lamb_f32          same file :402-449; single-segment/w==0 special cases, float64 brute force  pinned
+ *   orc_adam_f16g         no counterpart in the reference (it has no loss scaling / overflow detection):
+ *                         build-defined, pinned by closed forms only; parity with Apex "parity unpinned"
+ *   orc_philox4x32_10     Random123 known-answer vectors                         pinned
+ *   orc_mlp_outproj       no reference test beyond the all-ones C == K check
+ *                         (nccl-overlap/samples/matmul-allreduce-bias-dropout-layernorm.cu:520-526);
+ *                         float64 brute force; dropout mask build-defined ("parity unpinned" vs cuRAND)
+ */
+#ifndef CCN_ORACLE_H
+#define CCN_ORACLE_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- scalar conversions (IEEE binary16 / bfloat16, round-to-nearest-even) ---- */
+uint16_t orc_f32_to_f16(float f);
+float    orc_f16_to_f32(uint16_t h);
+uint16_t orc_f32_to_bf16(float f);
+float    orc_bf16_to_f32(uint16_t h);
+void orc_f32_to_f16_array(const float* src, uint16_t* dst, size_t n);
+void orc_f16_to_f32_array(const uint16_t* src, float* dst, size_t n);
+void orc_f32_to_bf16_array(const float* src, uint16_t* dst, size_t n);
+void orc_bf16_to_f32_array(const uint16_t* src, float* dst, size_t n);
+
+/* ---- the reference's comparators ---- */
+int orc_eqFloat_1e3(float u, float v);   /* examples/header.h:52-59 */
+int orc_eq_float_1e5(float f1, float f2); /* nccl-overlap/samples/multi-process-adam-scattered.cpp:60-66 */
+
+/* ---- P-way reduce ---- */
+void orc_reduce_f32(const float* const* g, int P, size_t N, float* out);
+
+/* ---- SGD ---- */
+void orc_sgd_f32(const float* const* g, int P, float* w, size_t N, float lr);
+void orc_sgd_axpby_f32(const float* const* g, int P, float* w, size_t N, float alpha, float beta);
+
+/* ---- the DSL example's pseudo-Adam (no sqrt, "bias correction" = divide by beta) ---- */
+void orc_pseudo_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
+                         float lr, float beta1, float beta2);
+
+/* ---- the modified-NCCL fused mixed-precision Adam (fp16 ring sum, square in half, beta2 used for m) ---- */
+void orc_fused_adam_a3(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* halfw,
+                       size_t N, float lr, float beta1, float beta2);
+
+/* ---- bias-corrected Adam; step = epoch+1 >= 1; w <- w - lr * mhat/(sqrt(vhat)+eps) ---- */
+void orc_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
+                  float lr, float beta1, float beta2, float eps, int step);
+
+/* ---- mixed-precision Adam: fp16 gradients, loss-scale removal, overflow flag, fp16 weight copy ---- */
+/* returns the overflow flag (0/1) */
+uint32_t orc_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16,
+                       size_t N, float lr, float beta1, float beta2, float eps, int step, float inv_scale);
+uint32_t orc_overflow_f16(const uint16_t* const* g, int P, size_t N);
+
+/* ---- LAMB with per-segment norms.  seg_offsets has nseg+1 entries, seg_offsets[nseg] == N.
+ *      mode 0: scale = trust ratio W/R;  mode 1 (reference): scale = (W/R)/R.
+ *      norms_out (optional, 2*nseg doubles): W_b, R_b after the square root. ---- */
+void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
+                  const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2,
+                  float eps, float wd, int step, int mode, double* norms_out);
+
+/* ---- counter-based RNG ---- */
+void orc_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+/* keep decision for element idx of a dropout with drop probability p_drop (1 = keep) */
+int  orc_dropout_keep(uint64_t seed, uint64_t idx, float p_drop);
+void orc_dropout_mask(uint64_t seed, uint64_t first_idx, size_t n, float p_drop, uint8_t* keep);
+
+/* ---- model-parallel MLP out-projection, one rank's K-slice:
+ *      acc = X[MxK] (bf16) . W[KxN] (bf16), float64 accumulation rounded once to fp32;
+ *      s = acc + partial[0] + ... + partial[nPartials-1]  (fp32, ascending);
+ *      t = s + bias[col]; d = keep ? t * (1/(1-p)) : 0;  y = d + resid;  out = bf16(y)
+ *      out_f32 (optional) receives y before the bf16 rounding. ---- */
+void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                     const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                     int M, int N, int K, float p_drop, uint64_t seed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,417 @@
+"""GPU parity tests: the HIP kernels behind the C ABI against the CPU oracle on identical seeded inputs.
+
+Bars (BASELINE north star): fp32 state within 1e-6 relative, fp16 weight copies within 1e-3, overflow
+flags exact.  The kernels are written to round where the oracle rounds, so the tests first ask for
+bit-identical results and report the largest ulp distance if that ever fails.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from util import (REF_BUFF_SIZES_HEAD, REF_BUFF_SIZES_TAIL, grads_f32, ref_integer_pattern, rel_err, rng, ulp_diff_f32,
+                  weights_f32)
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+FP32_TOL = 1e-6
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def dev_u16(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).to(DEV)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def host_u16(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy().view(np.uint16)
+
+
+def assert_f32_parity(got, want, what):
+    """North-star bar, then the stronger bit-exact claim."""
+    scale = max(float(np.max(np.abs(want))), 1e-30) if want.size else 1.0
+    assert np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)), initial=0.0) <= FP32_TOL * scale, what
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), \
+        f"{what}: not bit-identical, max ulp distance {ulp_diff_f32(got, want)}, rel {rel_err(got, want):.3g}"
+
+
+SIZES = [1, 3, 4, 5, 255, 1024, 4099, (1 << 20) + 3]
+RANKS = [1, 2, 3, 4, 7, 8, 9, 16]
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("P", RANKS)
+def test_reduce_and_sgd_ranks(ccn, P):
+    N = 70001
+    g = grads_f32(11, P, N, 1e-2)
+    gd = [dev(x) for x in g]
+    out = torch.empty(N, device=DEV)
+    ccn.reduce_f32(gd, out, N)
+    assert_f32_parity(host(out), orc.reduce_f32(g), f"reduce P={P}")
+    w0 = weights_f32(11, N, 0.1)
+    wd = dev(w0)
+    ccn.sgd_f32(gd, wd, N, 0.01)
+    w = w0.copy()
+    orc.sgd_f32(g, w, 0.01)
+    assert_f32_parity(host(wd), w, f"sgd P={P}")
+    ccn.sgd_axpby_f32(gd, wd, N, 0.75, -0.01)
+    orc.sgd_axpby_f32(g, w, 0.75, -0.01)
+    assert_f32_parity(host(wd), w, f"axpby P={P}")
+
+
+@pytest.mark.parametrize("N", SIZES)
+def test_sgd_sizes_and_tails(ccn, N):
+    P = 4
+    g = grads_f32(12, P, N, 1e-2)
+    w0 = weights_f32(12, N, 0.1)
+    # guard elements after the end must stay untouched
+    wd = torch.full((N + 8,), 7.0, device=DEV)
+    wd[:N] = dev(w0)
+    ccn.sgd_f32([dev(x) for x in g], wd, N, 0.01)
+    w = w0.copy()
+    orc.sgd_f32(g, w, 0.01)
+    got = host(wd)
+    assert_f32_parity(got[:N], w, f"sgd N={N}")
+    assert np.all(got[N:] == 7.0)
+
+
+def test_sgd_config1_full_size(ccn):
+    # BASELINE config 1: N = 2^20, P = 4, g ~ N(0, 1e-2), w ~ U(-0.1, 0.1), lr = 0.01
+    P, N = 4, 1 << 20
+    g = grads_f32(0, P, N, 1e-2)
+    w0 = weights_f32(0, N, 0.1)
+    wd = dev(w0)
+    ccn.sgd_f32([dev(x) for x in g], wd, N, 0.01)
+    w = w0.copy()
+    orc.sgd_f32(g, w, 0.01)
+    got = host(wd)
+    assert_f32_parity(got, w, "config 1")
+    # the reference's own acceptance test for this program (examples/test-sgd.cu:19, eqFloat rel 1e-3)
+    assert all(orc.eqFloat(a, b) for a, b in zip(w[::997], got[::997]))
+
+
+def test_reduce_in_place_and_empty(ccn):
+    P, N = 4, 5000
+    g = grads_f32(13, P, N, 1e-2)
+    gd = [dev(x) for x in g]
+    ccn.reduce_f32(gd, gd[0], N)            # all-reduce in place, as the reference does
+    assert_f32_parity(host(gd[0]), orc.reduce_f32(g), "in-place reduce")
+    ccn.sgd_f32(gd, gd[1], 0, 0.1)          # N == 0 is a no-op
+    assert np.array_equal(host(gd[1]), g[1])
+
+
+def test_misaligned_buffers_take_the_scalar_path(ccn):
+    P, N = 3, 10007
+    g = grads_f32(14, P, N, 1e-2)
+    w0 = weights_f32(14, N, 0.1)
+    # shift every buffer by one element so that no pointer is 16-byte aligned
+    gbuf = [torch.zeros(N + 1, device=DEV) for _ in range(P)]
+    for b, x in zip(gbuf, g):
+        b[1:] = dev(x)
+    wbuf = torch.zeros(N + 1, device=DEV)
+    wbuf[1:] = dev(w0)
+    mbuf = torch.zeros(N + 1, device=DEV)
+    vbuf = torch.zeros(N + 1, device=DEV)
+    ccn.adam_f32([b[1:] for b in gbuf], wbuf[1:], mbuf[1:], vbuf[1:], N, 1e-3, 0.9, 0.999, 1e-6, 1)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 1)
+    assert_f32_parity(host(wbuf)[1:], w, "misaligned adam w")
+    assert_f32_parity(host(mbuf)[1:], m, "misaligned adam m")
+    assert host(wbuf)[0] == 0.0
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+def test_pseudo_adam_known_answer_and_parity(ccn):
+    for P in (1, 4, 8):
+        N = 3001
+        ones = [torch.ones(N, device=DEV) for _ in range(P)]
+        w, m, v = (torch.zeros(N, device=DEV) for _ in range(3))
+        ccn.pseudo_adam_f32(ones, w, m, v, N, 1.0, 0.5, 0.5)
+        assert np.all(host(w) == np.float32(-1.0 / P))          # examples/test-adam.cu:73-88
+    P, N = 8, 50001
+    g = grads_f32(15, P, N, 1e-2)
+    w0, m0 = weights_f32(15, N, 0.1), weights_f32(16, N, 0.01)
+    v0 = np.abs(weights_f32(17, N, 0.01)) + np.float32(1e-3)
+    wd, md, vd = dev(w0), dev(m0), dev(v0)
+    ccn.pseudo_adam_f32([dev(x) for x in g], wd, md, vd, N, 0.1, 0.9, 0.99)
+    w, m, v = w0.copy(), m0.copy(), v0.copy()
+    orc.pseudo_adam_f32(g, w, m, v, 0.1, 0.9, 0.99)
+    assert_f32_parity(host(wd), w, "pseudo-adam w")
+    assert_f32_parity(host(md), m, "pseudo-adam m")
+    assert_f32_parity(host(vd), v, "pseudo-adam v")
+
+
+@pytest.mark.parametrize("P,N", [(8, 1 << 20), (8, 4099), (1, 1000), (5, 12345), (12, 7777)])
+def test_adam_config2_ten_steps(ccn, P, N):
+    # BASELINE config 2 at reduced N: fresh gradients every step, bias correction at t = 1..10
+    w0 = weights_f32(0, N, 0.05)
+    wd, md, vd = dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    for t in range(1, 11):
+        g = grads_f32(0, P, N, 1e-3, step=t)
+        ccn.adam_f32([dev(x) for x in g], wd, md, vd, N, 1e-3, 0.9, 0.999, 1e-6, t)
+        orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t)
+    assert_f32_parity(host(wd), w, "adam w")
+    assert_f32_parity(host(md), m, "adam m")
+    assert_f32_parity(host(vd), v, "adam v")
+
+
+def test_adam_reference_fixture(ccn):
+    """The reference's own harness (multi-process-adam-scattered.cpp:156-369): integer pattern, beta = .5,
+    alpha = +1, 5 checked steps, judged with its eq_float (rel 1e-5)."""
+    P = 4
+    for buff, n in enumerate(REF_BUFF_SIZES_TAIL):
+        g0 = ref_integer_pattern(buff, n)
+        gd = [dev(g0) for _ in range(P)]
+        wd, md, vd = dev(g0), torch.zeros(n, device=DEV), torch.zeros(n, device=DEV)
+        w, m, v = g0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+        for epoch in range(5):
+            ccn.adam_f32(gd, wd, md, vd, n, -1.0, 0.5, 0.5, 1e-6, epoch + 1)
+            orc.adam_f32([g0] * P, w, m, v, -1.0, 0.5, 0.5, 1e-6, epoch + 1)
+            got = host(wd)
+            assert all(orc.eq_float(a, b) for a, b in zip(w, got))
+            assert_f32_parity(got, w, f"fixture buff {buff} epoch {epoch}")
+
+
+def test_adam_full_size_sampled(ccn):
+    """BASELINE config 2 at its full size (N = 2^28, P = 8).  Adam is elementwise, so the oracle is run on
+    the elements gathered at sampled indices (first/last elements, block edges and random positions)."""
+    P, N = 8, 1 << 28
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(1234)
+    g = [torch.randn(N, device=DEV, generator=gen) * 1e-3 for _ in range(P)]
+    w = (torch.rand(N, device=DEV, generator=gen) - 0.5) * 0.1
+    m = torch.zeros(N, device=DEV)
+    v = torch.zeros(N, device=DEV)
+    r = rng(20)
+    idx = np.unique(np.concatenate([
+        np.arange(0, 4096), np.arange(N - 4096, N), r.integers(0, N, 200000),
+        (np.arange(1, 2048) * 131072)[:, None].repeat(8, 1).ravel() + np.tile(np.arange(-4, 4), 2047),
+    ]))
+    it = torch.from_numpy(idx).to(DEV)
+    hw, hm, hv = (host(x[it]).copy() for x in (w, m, v))
+    for t in (1, 2, 3):
+        hg = [host(x[it]).copy() for x in g]
+        ccn.adam_f32(g, w, m, v, N, 1e-3, 0.9, 0.999, 1e-6, t)
+        orc.adam_f32(hg, hw, hm, hv, 1e-3, 0.9, 0.999, 1e-6, t)
+        for x in g:            # next step's gradients: a cheap deterministic change of every buffer
+            x.mul_(-0.5)
+    assert_f32_parity(host(w[it]), hw, "full-size adam w")
+    assert_f32_parity(host(m[it]), hm, "full-size adam m")
+    assert_f32_parity(host(v[it]), hv, "full-size adam v")
+    # size-independent property: with m, v restarted at zero and every rank holding the same g, the step-1
+    # update is lr*G/(|G|+eps) with G = P*g, on every one of the 2^28 elements
+    m.zero_(); v.zero_()
+    w_before = w.clone()
+    ccn.adam_f32([g[0]] * P, w, m, v, N, 1e-3, 0.9, 0.999, 1e-6, 1)
+    G = g[0].double() * P
+    expect = w_before.double() - 1e-3 * G / (G.abs() + 1e-6)
+    assert float((w.double() - expect).abs().max()) < 1e-8
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+def _mixed_inputs(seed, P, N, plant):
+    scale = np.float32(2.0 ** 16)
+    g16 = [orc.f32_to_f16(x * scale) for x in grads_f32(seed, P, N, 1e-3)]
+    r = rng(seed, 77)
+    for _ in range(plant):
+        g16[int(r.integers(0, P))][int(r.integers(0, N))] = [0x7C00, 0xFC00, 0x7E00][int(r.integers(0, 3))]
+    return g16
+
+
+@pytest.mark.parametrize("P,N,plant", [(8, 1 << 20, 0), (8, 1 << 20, 1), (8, 100003, 5), (3, 8, 1), (9, 4099, 2),
+                                       (1, 1, 1), (8, 7, 0)])
+def test_mixed_precision_adam(ccn, P, N, plant):
+    g16 = _mixed_inputs(21, P, N, plant)
+    w0 = weights_f32(21, N, 0.05)
+    wd, md, vd = dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w16d = torch.zeros(N, dtype=torch.int16, device=DEV)
+    flag = torch.full((1,), 123, dtype=torch.int32, device=DEV)      # stale value must be overwritten
+    gd = [dev_u16(x) for x in g16]
+    w, m, v, w16 = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros(N, np.uint16)
+    for t in (1, 2):
+        ccn.adam_f16g(gd, wd, md, vd, w16d, N, 1e-3, 0.9, 0.999, 1e-6, t, 2.0 ** -16, flag)
+        want = orc.adam_f16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, t, np.float32(2.0 ** -16))
+        assert int(host(flag)[0]) == want == (1 if plant else 0)
+    assert_f32_parity(host(wd), w, "mixed w")
+    assert_f32_parity(host(md), m, "mixed m")
+    assert_f32_parity(host(vd), v, "mixed v")
+    got16 = host_u16(w16d)
+    assert rel_err(orc.f16_to_f32(got16), orc.f16_to_f32(w16)) <= 1e-3
+    assert np.array_equal(got16, w16)
+    ccn.overflow_check_f16(gd, N, flag)
+    assert int(host(flag)[0]) == orc.overflow_f16(g16)
+
+
+def test_mixed_precision_full_size_flag_and_skips(ccn):
+    """BASELINE config 3 at full size: one in 2^20 entries forced to inf.  Checked through properties:
+    flag == 1, exactly the planted elements keep their state, fp16 copy == fp16(w) everywhere."""
+    P, N = 8, 1 << 28
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(99)
+    g = [(torch.randn(N, device=DEV, generator=gen) * (1e-3 * 65536.0)).to(torch.float16) for _ in range(P)]
+    r = rng(22)
+    planted = np.unique(r.integers(0, N, (N * P) >> 20))
+    ranks = r.integers(0, P, planted.size)
+    inf16 = torch.tensor(float("inf"), dtype=torch.float16, device=DEV)
+    for p in range(P):
+        sel = torch.from_numpy(planted[ranks == p]).to(DEV)
+        g[p][sel] = inf16
+    w = (torch.rand(N, device=DEV, generator=gen) - 0.5) * 0.1
+    w0 = w.clone()
+    m = torch.zeros(N, device=DEV)
+    v = torch.zeros(N, device=DEV)
+    w16 = torch.zeros(N, dtype=torch.float16, device=DEV)
+    flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ccn.adam_f16g(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, 1, 2.0 ** -16, flag)
+    assert int(host(flag)[0]) == 1
+    # which elements overflow, and which have an exactly zero gradient sum, recomputed with torch
+    bad = torch.zeros(N, dtype=torch.bool, device=DEV)
+    gs = torch.zeros(N, device=DEV)
+    for p in range(P):
+        bad |= ~torch.isfinite(g[p])
+        gs = g[p].float() * (2.0 ** -16) if p == 0 else gs + g[p].float() * (2.0 ** -16)
+    assert np.array_equal(torch.nonzero(bad).flatten().cpu().numpy(), planted)
+    unchanged = (w == w0) & (m == 0) & (v == 0)
+    assert bool(torch.equal(unchanged, bad | (gs == 0)))      # exactly the overflowing elements are skipped
+    del bad, gs, unchanged
+    assert bool(torch.equal(w16, w.to(torch.float16)))
+    assert bool(torch.isfinite(w).all()) and bool(torch.isfinite(m).all()) and bool(torch.isfinite(v).all())
+    # sampled parity against the oracle, planted positions included
+    idx = np.unique(np.concatenate([planted[:2000], r.integers(0, N, 100000), np.arange(N - 64, N)]))
+    it = torch.from_numpy(idx).to(DEV)
+    hg = [host(x[it]).view(np.uint16).copy() for x in g]
+    hw, hm, hv = host(w0[it]).copy(), np.zeros(idx.size, np.float32), np.zeros(idx.size, np.float32)
+    h16 = np.zeros(idx.size, np.uint16)
+    orc.adam_f16g(hg, hw, hm, hv, h16, 1e-3, 0.9, 0.999, 1e-6, 1, np.float32(2.0 ** -16))
+    assert_f32_parity(host(w[it]), hw, "full-size mixed w")
+    assert_f32_parity(host(v[it]), hv, "full-size mixed v")
+    assert np.array_equal(host(w16[it]).view(np.uint16), h16)
+
+
+def test_fused_adam_reference_variant(ccn):
+    # the modified NCCL's kernel arithmetic: known answer (common_kernel.h:658-660) and parity on random data
+    for P in (2, 8):
+        N = 5003
+        ones = [torch.ones(N, dtype=torch.float16, device=DEV) for _ in range(P)]
+        w, m, v = (torch.zeros(N, device=DEV) for _ in range(3))
+        hw = torch.zeros(N, dtype=torch.int16, device=DEV)
+        ccn.fused_adam_ref_f16g(ones, w, hw, m, v, N, 1.0, 0.5, 0.5)
+        assert np.all(host(w) == -1.0) and np.all(host_u16(hw) == 0xBC00)
+    P, N = 8, 100001
+    g16 = [orc.f32_to_f16(x) for x in grads_f32(23, P, N, 0.5)]
+    w0 = weights_f32(23, N, 0.05)
+    m0 = weights_f32(24, N, 0.05)
+    v0 = np.abs(weights_f32(25, N, 0.05)) + np.float32(0.01)
+    wd, md, vd = dev(w0), dev(m0), dev(v0)
+    hwd = torch.zeros(N, dtype=torch.int16, device=DEV)
+    ccn.fused_adam_ref_f16g([dev_u16(x) for x in g16], wd, hwd, md, vd, N, 0.01, 0.9, 0.99)
+    w, m, v, hw = w0.copy(), m0.copy(), v0.copy(), np.zeros(N, np.uint16)
+    orc.fused_adam_a3(g16, w, m, v, hw, 0.01, 0.9, 0.99)
+    assert_f32_parity(host(wd), w, "A3 w")
+    assert_f32_parity(host(md), m, "A3 m")
+    assert_f32_parity(host(vd), v, "A3 v")
+    assert np.array_equal(host_u16(hwd), hw)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+def _lamb_compare(ccn, g, w0, segs, lr, b1, b2, eps, wd_, steps, mode, what, m0=None, v0=None):
+    N = w0.size
+    gd = [dev(x) for x in g]
+    wd, md, vd = dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    plan = ccn.LambPlan(segs)
+    for t in range(1, steps + 1):
+        plan.step(gd, wd, md, vd, lr, b1, b2, eps, wd_, t, mode)
+        norms = orc.lamb_f32(g, w, m, v, segs, lr, b1, b2, eps, wd_, t, mode)
+        gn = plan.norms()
+        assert rel_err(gn, norms) < 1e-9, what           # float64 sums, different association only
+    gw, gm, gv = host(wd), host(md), host(vd)
+    plan.close()
+    # m and v do not depend on the norms: bit-exact.  w goes through scale = (float)(W/R): 1e-6 bar.
+    assert_f32_parity(gm, m, what + " m")
+    assert_f32_parity(gv, v, what + " v")
+    scale = float(np.max(np.abs(w)))
+    assert np.max(np.abs(gw.astype(np.float64) - w)) <= FP32_TOL * scale, what
+    return ulp_diff_f32(gw, w)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_lamb_ragged_segments(ccn, mode):
+    P = 4
+    segs = [0, 5, 1029, 1030, 4096, 10000, 10000 + 8192, 10000 + 3 * 8192 + 1, 70001]
+    N = segs[-1]
+    g = grads_f32(26, P, N, 1e-3)
+    w0 = weights_f32(26, N, 0.05)
+    ulps = _lamb_compare(ccn, g, w0, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 3, mode, f"ragged mode {mode}")
+    assert ulps <= 2
+
+
+def test_lamb_config4_reduced(ccn):
+    # BASELINE config 4 layout at reduced size: 16 segments of 2^16, P = 8, wd = 0.01, two-pass norm + update
+    P, nseg, seglen = 8, 16, 1 << 16
+    N = nseg * seglen
+    segs = [i * seglen for i in range(nseg + 1)]
+    g = grads_f32(0, P, N, 1e-3)
+    w0 = weights_f32(0, N, 0.05)
+    _lamb_compare(ccn, g, w0, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 3, 0, "config 4 reduced")
+
+
+def test_lamb_reference_fixture(ccn):
+    """Reference harness for LAMB (multi-process-adam-scattered.cpp:464-698): integer pattern, beta = .5,
+    alpha = 1, weight decay 1.0, reference scale; head and tail of its buffer-size list scaled to fit a test."""
+    P = 2
+    sizes = [s // 16 if s > 1 << 20 else s for s in REF_BUFF_SIZES_HEAD] + REF_BUFF_SIZES_TAIL
+    segs = np.concatenate([[0], np.cumsum(sizes)]).tolist()
+    g0 = np.concatenate([ref_integer_pattern(i, n) for i, n in enumerate(sizes)])
+    N = g0.size
+    gd = [dev(g0) for _ in range(P)]
+    wd, md, vd = dev(g0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w, m, v = g0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    plan = ccn.LambPlan(segs)
+    for epoch in range(5):
+        plan.step(gd, wd, md, vd, 1.0, 0.5, 0.5, 1e-6, 1.0, epoch + 1, ccn.LAMB_REFERENCE)
+        orc.lamb_f32([g0] * P, w, m, v, segs, 1.0, 0.5, 0.5, 1e-6, 1.0, epoch + 1, 1)
+        got = host(wd)
+        bad = [i for i in range(0, N, 37) if not orc.eq_float(w[i], got[i])]      # the reference's comparator
+        assert not bad, (epoch, bad[:5])
+        assert np.max(np.abs(got.astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
+    plan.close()
+
+
+def test_lamb_full_size_segments(ccn):
+    """BASELINE config 4 at full size (N = 2^28 as 256 segments of 2^20, P = 8): the oracle is run on four
+    whole segments (first, two inner, last); segments are independent, so this is exact for them."""
+    P, nseg, seglen = 8, 256, 1 << 20
+    N = nseg * seglen
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(4321)
+    g = [torch.randn(N, device=DEV, generator=gen) * 1e-3 for _ in range(P)]
+    w = (torch.rand(N, device=DEV, generator=gen) - 0.5) * 0.1
+    m = torch.zeros(N, device=DEV)
+    v = torch.zeros(N, device=DEV)
+    check = [0, 77, 200, 255]
+    hg = {b: [host(x[b * seglen:(b + 1) * seglen]).copy() for x in g] for b in check}
+    hw = {b: host(w[b * seglen:(b + 1) * seglen]).copy() for b in check}
+    plan = ccn.LambPlan([i * seglen for i in range(nseg + 1)])
+    plan.step(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, ccn.LAMB_TRUST_RATIO)
+    norms = plan.norms()
+    for b in check:
+        ww, mm, vv = hw[b].copy(), np.zeros(seglen, np.float32), np.zeros(seglen, np.float32)
+        on = orc.lamb_f32(hg[b], ww, mm, vv, [0, seglen], 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, 0)
+        assert rel_err(norms[b], on[0]) < 1e-9
+        sl = slice(b * seglen, (b + 1) * seglen)
+        assert_f32_parity(host(m[sl]), mm, f"segment {b} m")
+        assert np.max(np.abs(host(w[sl]).astype(np.float64) - ww)) <= FP32_TOL * np.max(np.abs(ww))
+    del g
+    plan.close()
+    assert norms.shape == (nseg, 2) and np.all(norms > 0)

@@ -1,0 +1,397 @@
+"""Pins the CPU oracle (oracle/ccn_oracle.c) before anything is compared against it.
+
+Each routine is checked against evidence that does not come from the oracle itself: the reference's own
+fixtures and known answers, closed forms, library routines (numpy / torch on the CPU) and float64 brute
+force.  None of these tests needs a GPU.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from util import REF_BUFF_SIZES_TAIL, grads_f32, ref_integer_pattern, rel_err, rng, weights_f32
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# conversions
+# ---------------------------------------------------------------------------------------------------------------------
+def test_f16_exhaustive_decode_and_roundtrip():
+    allh = np.arange(65536, dtype=np.uint16)
+    ref = allh.view(np.float16).astype(np.float32)
+    got = orc.f16_to_f32(allh)
+    finite_or_inf = ~np.isnan(ref)
+    assert np.array_equal(got.view(np.uint32)[finite_or_inf], ref.view(np.uint32)[finite_or_inf])
+    assert np.all(np.isnan(got[~finite_or_inf]))
+    assert np.array_equal(orc.f32_to_f16(got)[finite_or_inf], allh[finite_or_inf])
+
+
+def test_f32_to_f16_rne_against_numpy():
+    r = rng(1)
+    x = (r.standard_normal(1 << 20) * np.exp(r.uniform(-20, 12, 1 << 20))).astype(np.float32)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(orc.f32_to_f16(x), x.astype(np.float16).view(np.uint16))
+    # every tie between two neighbouring halfs, both signs
+    h = np.arange(0, 0x7bff, dtype=np.uint16)
+    mid = ((orc.f16_to_f32(h).astype(np.float64) + orc.f16_to_f32(h + 1).astype(np.float64)) / 2).astype(np.float32)
+    for s in (1.0, -1.0):
+        m = (mid * np.float32(s)).astype(np.float32)
+        assert np.array_equal(orc.f32_to_f16(m), m.astype(np.float16).view(np.uint16))
+    special = np.array([np.inf, -np.inf, 65504.0, 65519.99, 65520.0, 1e9, 2.0 ** -25, 2.0 ** -24, 0.0, -0.0], np.float32)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(orc.f32_to_f16(special), special.astype(np.float16).view(np.uint16))
+    assert (orc.f32_to_f16(np.array([np.nan], np.float32))[0] & 0x7c00) == 0x7c00
+
+
+def test_bf16_against_torch():
+    r = rng(2)
+    x = (r.standard_normal(1 << 20) * np.exp(r.uniform(-30, 30, 1 << 20))).astype(np.float32)
+    t = torch.from_numpy(x).to(torch.bfloat16)
+    assert np.array_equal(orc.f32_to_bf16(x).view(np.int16), t.view(torch.int16).numpy())
+    allb = np.arange(65536, dtype=np.uint16)
+    back = torch.from_numpy(allb.view(np.int16)).view(torch.bfloat16).to(torch.float32).numpy()
+    got = orc.bf16_to_f32(allb)
+    ok = ~np.isnan(back)
+    assert np.array_equal(got.view(np.uint32)[ok], back.view(np.uint32)[ok])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# comparators of the reference
+# ---------------------------------------------------------------------------------------------------------------------
+def test_reference_comparators():
+    assert orc.eqFloat(1.0, 1.0005) and not orc.eqFloat(1.0, 1.002)
+    assert orc.eqFloat(0.0, 0.0) and not orc.eqFloat(0.0, 1e-9)
+    assert orc.eq_float(1.0, 1.000005) and not orc.eq_float(1.0, 1.00002)
+    assert orc.eq_float(0.0, 0.0)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# reduce / SGD
+# ---------------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("P", [1, 2, 4, 8, 16])
+def test_reduce_integers_exact_and_order(P):
+    N = 1000
+    g = [np.full(N, p + 1, np.float32) for p in range(P)]
+    assert np.array_equal(orc.reduce_f32(g), np.full(N, P * (P + 1) / 2, np.float32))
+    # order: ascending p, one fp32 rounding per add.  1 + 2^-24 + 2^-24 is 1 when added left to right in
+    # fp32 (each 2^-24 is a tie that rounds to even), but 1 + 2^-23 if the small terms were paired first.
+    if P >= 3:
+        g = [np.zeros(4, np.float32) for _ in range(P)]
+        g[0][:] = 1.0
+        g[1][:] = 2.0 ** -24
+        g[2][:] = 2.0 ** -24
+        assert np.all(orc.reduce_f32(g) == np.float32(1.0))
+    gr = grads_f32(3, P, N, 1e-2)
+    seq = gr[0].copy()
+    for p in range(1, P):
+        seq = seq + gr[p]
+    assert np.array_equal(orc.reduce_f32(gr), seq)
+    # permutation bound: any order agrees within P ulps of sum |g|
+    rev = orc.reduce_f32(gr[::-1])
+    bound = P * np.finfo(np.float32).eps * np.sum(np.abs(np.stack(gr)), axis=0)
+    assert np.all(np.abs(rev - seq) <= bound)
+
+
+def test_sgd_closed_form_and_axpy():
+    P, N = 4, 64
+    g = [np.full(N, p + 1, np.float32) for p in range(P)]           # sum = 10
+    w = np.full(N, 8.0, np.float32)
+    orc.sgd_f32(g, w, 0.5)
+    assert np.all(w == 3.0)
+    gr = grads_f32(4, P, 1 << 12, 1e-2)
+    w0 = weights_f32(4, 1 << 12, 0.1)
+    w = w0.copy()
+    orc.sgd_f32(gr, w, np.float32(0.01))
+    s = ((gr[0] + gr[1]) + gr[2]) + gr[3]
+    assert np.array_equal(w, w0 - np.float32(0.01) * s)
+    # independent library cross-check in float64
+    ref = w0.astype(np.float64) - 0.01 * np.sum(np.stack(gr).astype(np.float64), axis=0)
+    assert rel_err(w, ref) < 1e-6
+    w = w0.copy()
+    orc.sgd_axpby_f32(gr, w, np.float32(0.75), np.float32(-0.01))
+    assert np.array_equal(w, np.float32(0.75) * w0 + np.float32(-0.01) * s)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the DSL example's pseudo-Adam and the modified NCCL's fused kernel: known answers held by the reference
+# ---------------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("P", [1, 2, 4, 8, 16])
+def test_pseudo_adam_known_answer(P):
+    # examples/test-adam.cu:73-88: g = 1, w = m = v = 0, lr = 1, beta1 = beta2 = 0.5  =>  w = -1/P
+    N = 257
+    g = [np.ones(N, np.float32) for _ in range(P)]
+    w, m, v = (np.zeros(N, np.float32) for _ in range(3))
+    orc.pseudo_adam_f32(g, w, m, v, 1.0, 0.5, 0.5)
+    assert np.all(w == np.float32(-1.0 / P))
+    assert np.all(m == np.float32(P / 2)) and np.all(v == np.float32(P * P / 2))
+
+
+@pytest.mark.parametrize("P", [2, 4, 8])
+def test_fused_adam_a3_known_answer(P):
+    # nccl/src/collectives/device/common_kernel.h:658-660: same inputs => w == -1.0, fp16 copy == 0xBC00
+    N = 129
+    g = [np.full(N, 0x3C00, np.uint16) for _ in range(P)]       # 1.0 in fp16
+    w, m, v = (np.zeros(N, np.float32) for _ in range(3))
+    hw = np.zeros(N, np.uint16)
+    orc.fused_adam_a3(g, w, m, v, hw, 1.0, 0.5, 0.5)
+    assert np.all(w == -1.0) and np.all(hw == 0xBC00)
+
+
+def test_fused_adam_a3_half_precision_effects():
+    # the sum is carried in fp16: 2048 + 1 is not representable in half (spacing 2), so the second rank's
+    # gradient is lost; an fp32 sum would give 2049.  The square is also rounded to half: 3.001^2.
+    g = [np.array([0x6800], np.uint16), np.array([0x3C00], np.uint16)]      # 2048, 1
+    w, m, v = (np.zeros(1, np.float32) for _ in range(3))
+    hw = np.zeros(1, np.uint16)
+    orc.fused_adam_a3(g, w, m, v, hw, 1.0, 0.5, 0.5)
+    assert m[0] == np.float32(2048 * 0.5)                    # (1-beta2) * fp16 sum; 2049 would give 1024.5
+    g = [np.array([0x4201], np.uint16)]                      # 3.001953125
+    w[:] = 0; m[:] = 0; v[:] = 0
+    orc.fused_adam_a3(g, w, m, v, hw, 1.0, 0.5, 0.5)
+    x = np.float16(3.001953125)
+    assert v[0] == np.float32(np.float16(x * x)) * np.float32(0.5)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# bias-corrected Adam
+# ---------------------------------------------------------------------------------------------------------------------
+def test_adam_step1_closed_form():
+    # m = v = 0 and one rank: mhat = c, vhat = c^2, update = lr*c/(|c|+eps), whatever the betas are
+    N = 4096
+    c = grads_f32(5, 1, N, 1e-3)
+    for b1, b2 in [(0.9, 0.999), (0.5, 0.5), (0.0, 0.99)]:
+        w0 = weights_f32(5, N, 0.05)
+        w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+        orc.adam_f32(c, w, m, v, 1e-3, b1, b2, 1e-6, 1)
+        cd = c[0].astype(np.float64)
+        upd = 1e-3 * cd / (np.abs(cd) + 1e-6)
+        assert rel_err(w0.astype(np.float64) - w.astype(np.float64), upd) < 5e-4   # w-w0 cancels ~13 bits
+        assert np.max(np.abs(w.astype(np.float64) - (w0.astype(np.float64) - upd))) < 4e-9   # one ulp of |w| <= 0.05
+        omb1, omb2 = float(np.float32(1) - np.float32(b1)), float(np.float32(1) - np.float32(b2))   # fp32 betas
+        assert rel_err(m, omb1 * cd) < 1e-6 and rel_err(v, omb2 * cd * cd) < 1e-6
+
+
+def test_adam_against_torch_optim():
+    # textbook Adam from a library (torch.optim.Adam on the CPU), 10 steps of BASELINE config 2 at small N
+    P, N = 8, 1 << 14
+    w0 = weights_f32(6, N, 0.05)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    tw = torch.nn.Parameter(torch.from_numpy(w0.astype(np.float64)))
+    f32 = lambda x: float(np.float32(x))      # the library sees the same fp32-rounded hyper-parameters
+    opt = torch.optim.Adam([tw], lr=f32(1e-3), betas=(f32(0.9), f32(0.999)), eps=f32(1e-6))
+    for t in range(1, 11):
+        g = grads_f32(6, P, N, 1e-3, step=t)
+        orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t)
+        tw.grad = torch.from_numpy(orc.reduce_f32(g).astype(np.float64))   # the reduce is pinned separately
+        opt.step()
+    st = opt.state[tw]
+    # torch adds eps to sqrt(v)/sqrt(1-b2^t) exactly as the checker adds it to sqrt(vhat); float64 vs fp32 state
+    tw_np = tw.detach().numpy()
+    assert np.max(np.abs(w - tw_np)) < 1e-6 * np.max(np.abs(tw_np))
+    big = np.abs(tw_np) > 1e-3                      # relative error where w is not itself near zero
+    assert rel_err(w[big], tw_np[big]) < 1e-5
+    d, dref = w - w0.astype(np.float64), tw_np - w0           # the accumulated update itself
+    assert np.max(np.abs(d - dref)) < 1e-5 * np.max(np.abs(dref))
+    assert np.max(np.abs(m - st["exp_avg"].numpy())) < 1e-6 * np.max(np.abs(m))
+    assert np.max(np.abs(v - st["exp_avg_sq"].numpy())) < 1e-6 * np.max(np.abs(v))
+
+
+@pytest.mark.parametrize("P", [1, 2, 4])
+def test_adam_reference_integer_fixture(P):
+    # the reference's fixture: every rank holds g = w0 = (i%2+1)*(index%20+1), beta = .5, alpha = +1 (lr = -1),
+    # eps 1e-6, 5 checked steps.  With a constant gradient G = P*g: mhat = G, vhat = G^2, so every step adds
+    # alpha*G/(G+eps) = 1 - eps/(G+eps).
+    for buff in (0, 1):
+        n = 2048
+        g0 = ref_integer_pattern(buff, n)
+        w, m, v = g0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+        G = P * g0.astype(np.float64)
+        for t in range(1, 6):
+            orc.adam_f32([g0] * P, w, m, v, -1.0, 0.5, 0.5, 1e-6, t)
+            expect = g0.astype(np.float64) + t * (1.0 - 1e-6 / (G + 1e-6))
+            assert rel_err(w, expect) < 1e-6
+            assert rel_err(m, (1 - 0.5 ** t) * G) < 1e-6
+            assert rel_err(v, (1 - 0.5 ** t) * G * G) < 1e-6
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# LAMB
+# ---------------------------------------------------------------------------------------------------------------------
+def lamb_float64(g, w, m, v, seg_offsets, lr, b1, b2, eps, wd, step, mode):
+    """Independent float64 restatement of LAMB with RMS-normalised per-segment norms (numpy, vectorised).
+    Hyper-parameters are first rounded to fp32, as the fp32 routine receives them."""
+    lr, b1, b2, eps, wd = (float(np.float32(x)) for x in (lr, b1, b2, eps, wd))
+    gs = np.sum(np.stack(g).astype(np.float64), axis=0)
+    m = b1 * m.astype(np.float64) + (1 - b1) * gs
+    v = b2 * v.astype(np.float64) + (1 - b2) * gs * gs
+    mh, vh = m / (1 - b1 ** step), v / (1 - b2 ** step)
+    w = w.astype(np.float64)
+    r = mh / (np.sqrt(vh) + eps) + wd * w
+    out = w.copy()
+    norms = []
+    for b in range(len(seg_offsets) - 1):
+        lo, hi = seg_offsets[b], seg_offsets[b + 1]
+        W = np.sqrt(np.mean(w[lo:hi] ** 2))
+        R = np.sqrt(np.mean(r[lo:hi] ** 2))
+        ratio = (W / R if R > 0 else 1.0) if W > 0 else 1.0
+        scale = ratio / R if mode == 1 else ratio
+        out[lo:hi] = w[lo:hi] - lr * scale * r[lo:hi]
+        norms.append((W, R))
+    return out, m, v, np.array(norms)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_lamb_float64_brute_force(mode):
+    P = 4
+    segs = [0, 5, 1029, 1030, 4096, 10000]
+    N = segs[-1]
+    g = grads_f32(7, P, N, 1e-3)
+    w0 = weights_f32(7, N, 0.05)
+    m0 = (rng(7, 50).standard_normal(N) * 1e-3).astype(np.float32)
+    v0 = (rng(7, 51).uniform(0, 1e-5, N)).astype(np.float32)
+    w, m, v = w0.copy(), m0.copy(), v0.copy()
+    norms = orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 3, mode)
+    ew, em, ev, en = lamb_float64(g, w0, m0, v0, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 3, mode)
+    assert rel_err(norms, en) < 1e-6
+    assert np.max(np.abs(w - ew)) < 1e-6 * np.max(np.abs(ew))
+    assert np.max(np.abs(m - em)) < 1e-6 * np.max(np.abs(em)) and np.max(np.abs(v - ev)) < 1e-6 * np.max(np.abs(ev))
+    # the update itself (w - w0), not only w: a wrong scale would hide behind w's magnitude otherwise
+    d, dref = w.astype(np.float64) - w0, ew - w0
+    assert np.max(np.abs(d - dref)) < 1e-3 * np.max(np.abs(dref))     # fp32 rounding of w is ~2e-4 of a step here
+
+
+def test_lamb_special_cases():
+    P, n = 2, 3000
+    g = grads_f32(8, P, n, 1e-3)
+    # w == 0: W = 0 => ratio 1; trust-ratio mode steps by lr*r, reference mode by lr*r/R
+    for mode in (0, 1):
+        w, m, v = (np.zeros(n, np.float32) for _ in range(3))
+        norms = orc.lamb_f32(g, w, m, v, [0, n], 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, mode)
+        gs = (g[0] + g[1]).astype(np.float64)
+        r = gs / (np.abs(gs) + 1e-6)          # step 1, m = v = 0: mhat/(sqrt(vhat)+eps) = gs/(|gs|+eps)
+        R = np.sqrt(np.mean(r * r))
+        assert norms[0, 0] == 0.0 and abs(norms[0, 1] - R) < 1e-6 * R
+        expect = -1e-3 * r / (R if mode == 1 else 1.0)
+        assert rel_err(w, expect) < 1e-5
+    # segments are independent: a 3-segment call equals three 1-segment calls
+    segs = [0, 1000, 1001, n]
+    w0 = weights_f32(8, n, 0.05)
+    w, m, v = w0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, 0)
+    for b in range(3):
+        lo, hi = segs[b], segs[b + 1]
+        ws, ms, vs = w0[lo:hi].copy(), np.zeros(hi - lo, np.float32), np.zeros(hi - lo, np.float32)
+        orc.lamb_f32([x[lo:hi].copy() for x in g], ws, ms, vs, [0, hi - lo], 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, 0)
+        assert np.array_equal(ws, w[lo:hi]) and np.array_equal(ms, m[lo:hi])
+
+
+def test_lamb_reference_integer_fixture():
+    # reference fixture (multi-process-adam-scattered.cpp:221-226 and the tail of its buffer list): constant
+    # gradient G per element, so step 1 gives r = G/(G+eps) + w with w = g; reference mode (second /R kept).
+    P = 2
+    sizes = REF_BUFF_SIZES_TAIL
+    segs = np.concatenate([[0], np.cumsum(sizes)])
+    g0 = np.concatenate([ref_integer_pattern(i, n) for i, n in enumerate(sizes)])
+    w, m, v = g0.copy(), np.zeros_like(g0), np.zeros_like(g0)
+    orc.lamb_f32([g0] * P, w, m, v, segs, 1.0, 0.5, 0.5, 1e-6, 1.0, 1, 1)
+    G = P * g0.astype(np.float64)
+    r = G / (G + 1e-6) + g0
+    for b in range(len(sizes)):
+        lo, hi = segs[b], segs[b + 1]
+        W, R = np.sqrt(np.mean(g0[lo:hi].astype(np.float64) ** 2)), np.sqrt(np.mean(r[lo:hi] ** 2))
+        expect = g0[lo:hi] - (W / R / R) * r[lo:hi]
+        assert np.max(np.abs(w[lo:hi] - expect)) < 1e-5 * np.max(np.abs(g0[lo:hi]))
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# mixed-precision Adam with overflow flag (build-defined semantics, pinned by reduction to orc_adam_f32)
+# ---------------------------------------------------------------------------------------------------------------------
+def test_adam_f16g_reduces_to_adam_and_flags():
+    P, N = 8, 1 << 13
+    scale = 2.0 ** 16
+    g32 = grads_f32(9, P, N, 1e-3)
+    g16 = [orc.f32_to_f16(x * np.float32(scale)) for x in g32]
+    w0 = weights_f32(9, N, 0.05)
+    # no overflow: equals fp32 Adam on the decoded, unscaled gradients, bit for bit; flag 0
+    w, m, v, w16 = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros(N, np.uint16)
+    flag = orc.adam_f16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, 1, np.float32(1 / scale))
+    dec = [orc.f16_to_f32(x) * np.float32(1 / scale) for x in g16]
+    wr, mr, vr = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    orc.adam_f32(dec, wr, mr, vr, 1e-3, 0.9, 0.999, 1e-6, 1)
+    assert flag == 0 and orc.overflow_f16(g16) == 0
+    assert np.array_equal(w, wr) and np.array_equal(m, mr) and np.array_equal(v, vr)
+    assert np.array_equal(w16, w.astype(np.float16).view(np.uint16))
+    # plant +inf, -inf and a nan in different ranks: flag 1, exactly those elements keep their state
+    bad = {17: (0, 0x7C00), 4096: (3, 0xFC00), N - 1: (7, 0x7E01)}
+    for i, (p, bits) in bad.items():
+        g16[p][i] = bits
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    flag = orc.adam_f16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, 1, np.float32(1 / scale))
+    assert flag == 1 and orc.overflow_f16(g16) == 1
+    keep = np.ones(N, bool)
+    keep[list(bad)] = False
+    assert np.array_equal(w[keep], wr[keep]) and np.array_equal(m[keep], mr[keep])
+    assert np.array_equal(w[~keep], w0[~keep]) and np.all(m[~keep] == 0) and np.all(v[~keep] == 0)
+    assert np.array_equal(w16, w.astype(np.float16).view(np.uint16))
+    assert np.all(np.isfinite(w)) and np.all(np.isfinite(m)) and np.all(np.isfinite(v))
+    # the largest finite half (exponent 0x1E) is not an overflow
+    g16[0][5] = 0x7BFF
+    for i, (p, bits) in bad.items():
+        g16[p][i] = 0
+    assert orc.overflow_f16(g16) == 0
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Philox, dropout mask, GEMM epilogue
+# ---------------------------------------------------------------------------------------------------------------------
+def test_philox_known_answers():
+    # Random123 known-answer vectors for philox4x32-10
+    kat = [
+        ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+        ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+        ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+         [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+    ]
+    for ctr, key, out in kat:
+        assert [int(x) for x in orc.philox4x32_10(ctr, key)] == out
+
+
+def test_dropout_mask_definition():
+    n = 1 << 16
+    keep = orc.dropout_mask(0, 0, n, 0.1)
+    assert abs(keep.mean() - 0.9) < 0.005
+    assert np.array_equal(keep, orc.dropout_mask(0, 0, n, 0.1))
+    assert not np.array_equal(keep, orc.dropout_mask(1, 0, n, 0.1))
+    assert np.array_equal(keep[4096:], orc.dropout_mask(0, 4096, n - 4096, 0.1))      # counter-based: offsets compose
+    assert orc.dropout_mask(0, 0, n, 0.0).all()
+    # word -> uniform mapping, element 6 = word 2 of block 1
+    word = int(orc.philox4x32_10([1, 0, 0, 0], [0, 0])[2])
+    u = np.float32(word >> 8) * np.float32(2.0 ** -24)
+    for p in (0.05, 0.5, 0.95):
+        assert bool(orc.dropout_mask(0, 6, 1, p)[0]) == bool(u >= np.float32(p))
+
+
+def _bf16(x):
+    return orc.f32_to_bf16(np.ascontiguousarray(x, np.float32))
+
+
+def test_mlp_outproj_float64_brute_force_and_all_ones():
+    M, N, K, nP = 8, 12, 16, 3
+    r = rng(10)
+    X = _bf16(r.standard_normal((M, K)))
+    W = _bf16(r.standard_normal((K, N)) * 0.02)
+    parts = [r.standard_normal((M, N)).astype(np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N).astype(np.float32)
+    resid = _bf16(r.standard_normal((M, N)))
+    out, outf = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, 0.1, 0)
+    acc = orc.bf16_to_f32(X).astype(np.float64) @ orc.bf16_to_f32(W).astype(np.float64)
+    s = acc + np.sum(np.stack(parts).astype(np.float64), axis=0) + bias
+    keep = orc.dropout_mask(0, 0, M * N, 0.1).reshape(M, N).astype(bool)
+    y = np.where(keep, s / 0.9, 0.0) + orc.bf16_to_f32(resid)
+    assert np.max(np.abs(outf - y)) < 1e-5
+    assert np.array_equal(out, _bf16(outf))
+    # reference's only check at this boundary: all-ones operands give C == K*ranks
+    # (nccl-overlap/samples/matmul-allreduce-bias-dropout-layernorm.cu:520-526)
+    X1, W1 = _bf16(np.ones((M, K))), _bf16(np.ones((K, N)))
+    parts1 = [np.full((M, N), K, np.float32) for _ in range(7)]
+    _, outf = orc.mlp_outproj(X1, W1, parts1, np.zeros(N, np.float32), None, M, N, K, 0.0, 0)
+    assert np.all(outf == K * 8)
