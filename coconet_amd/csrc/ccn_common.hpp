@@ -85,6 +85,22 @@ template <typename T, int N> __device__ __forceinline__ void store_pack(T* p, co
   }
 }
 
+// Streaming store: the updated state is not read again before the next step has streamed ~15 GB past it.
+template <typename T, int N> __device__ __forceinline__ void store_stream(T* p, const Pack<T, N>& v) {
+  if constexpr (N == 1) {
+    __builtin_nontemporal_store(v.d[0], p);
+  } else {
+    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
+    constexpr int C = (N * (int)sizeof(T)) / 16;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      u32x4 x;
+      __builtin_memcpy(&x, reinterpret_cast<const char*>(v.d) + 16 * c, 16);
+      __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(p) + c);
+    }
+  }
+}
+
 // ---- table of P source pointers, passed by value in the kernel argument segment ----------------------------------
 template <typename T, int CAP> struct SrcTable { const T* p[CAP]; };
 
@@ -150,8 +166,18 @@ __host__ __device__ __forceinline__ bool keep_from_word(uint32_t word, float p_d
 }
 
 // ---- launch geometry for streaming kernels ----------------------------------------------------------------------------
-// Number of workgroups for a grid-stride kernel whose workgroup consumes `tile` units per iteration.
+// Number of workgroups for a grid-stride kernel whose workgroup consumes `tile` units per iteration
+// (a few workgroups per CU; used by the small helper kernels).
 unsigned stream_grid(size_t units, size_t tile);
+
+// Geometry of the fused reduce+update kernels.  One workgroup per tile (the kernels keep a grid-stride loop
+// only for shards beyond 2^31 tiles) and a cap on resident workgroups per CU, enforced by requesting dynamic
+// LDS that the kernel never touches.  HBM sustains the most bandwidth when the number of address streams
+// times the wavefronts in flight stays moderate: a kernel that walks 14 arrays at once (8 gradients, w/m/v in,
+// w/m/v out) loses ~10% of bandwidth at full occupancy against 2-3 workgroups per CU, while a 2-stream copy
+// wants all the occupancy it can get.  `streams` = arrays read + arrays written by the kernel.
+struct StreamLaunch { unsigned grid; unsigned lds_bytes; };
+StreamLaunch stream_launch(size_t units, size_t tile, int streams);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -31,7 +31,7 @@ struct SumF32 {
 };
 
 struct ReduceMath : SumF32 {
-  static constexpr int NS = 0, UNROLL = 2;
+  static constexpr int NS = 0, UNROLL = 1;
   static constexpr bool OUT16 = false, OUTF = true, FLAG = false;
   struct Prm {};
   static __device__ __forceinline__ bool apply(Acc gs, float*, uint16_t&, float& of, const Prm&) {
@@ -42,7 +42,7 @@ struct ReduceMath : SumF32 {
 
 // examples/test-sgd.cu:17-18
 struct SgdMath : SumF32 {
-  static constexpr int NS = 1, UNROLL = 2;
+  static constexpr int NS = 1, UNROLL = 1;
   static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
   struct Prm { float lr; };
   static __device__ __forceinline__ bool apply(Acc gs, float* st, uint16_t&, float&, const Prm& k) {
@@ -53,7 +53,7 @@ struct SgdMath : SumF32 {
 
 // nccl-overlap/samples/single-process-wX.cu:141
 struct AxpbyMath : SumF32 {
-  static constexpr int NS = 1, UNROLL = 2;
+  static constexpr int NS = 1, UNROLL = 1;
   static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
   struct Prm { float alpha, beta; };
   static __device__ __forceinline__ bool apply(Acc gs, float* st, uint16_t&, float&, const Prm& k) {
@@ -64,7 +64,7 @@ struct AxpbyMath : SumF32 {
 
 // examples/test-adam.cu:14-38
 struct PseudoAdamMath : SumF32 {
-  static constexpr int NS = 3, UNROLL = 2;
+  static constexpr int NS = 3, UNROLL = 1;
   static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
   struct Prm { float lr, b1, omb1, b2, omb2; };
   static __device__ __forceinline__ bool apply(Acc S0, float* st, uint16_t&, float&, const Prm& k) {
@@ -96,7 +96,7 @@ __device__ __forceinline__ void adam_step(float gs, float* st, const AdamPrm& k)
 }
 
 struct AdamMath : SumF32 {
-  static constexpr int NS = 3, UNROLL = 2;
+  static constexpr int NS = 3, UNROLL = 1;
   static constexpr bool OUT16 = false, OUTF = false, FLAG = false;
   using Prm = AdamPrm;
   static __device__ __forceinline__ bool apply(Acc gs, float* st, uint16_t&, float&, const Prm& k) {
@@ -129,7 +129,7 @@ struct Adam16Math {
 struct Overflow16Math {
   using G = uint16_t;
   using Acc = bool;
-  static constexpr int NS = 0, UNROLL = 2;
+  static constexpr int NS = 0, UNROLL = 1;
   static constexpr bool OUT16 = false, OUTF = false, FLAG = true;
   struct Prm {};
   static __device__ __forceinline__ Acc first(G h, const Prm&) { return (h & 0x7c00u) == 0x7c00u; }
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(kBlock) void fused_stream_kernel(
           for (int p = 0; p < P; p++) gv[u][p] = load_stream<G, VEC>(g.p[p] + e0);
         }
 #pragma unroll
-        for (int k = 0; k < M::NS; k++) sv[u][k] = load_keep<float, VEC>(st.p[k] + e0);
+        for (int k = 0; k < M::NS; k++) sv[u][k] = load_stream<float, VEC>(st.p[k] + e0);
         if constexpr (P == 0) {
           for (int p = 0; p < nP; p++) {
             const Pack<G, VEC> x = load_stream<G, VEC>(g.p[p] + e0);
@@ -253,9 +253,9 @@ __global__ __launch_bounds__(kBlock) void fused_stream_kernel(
           ofv.d[e] = of;
         }
 #pragma unroll
-        for (int k = 0; k < M::NS; k++) store_pack<float, VEC>(st.p[k] + e0, sv[u][k]);
-        if constexpr (M::OUT16) store_pack<uint16_t, VEC>(out16 + e0, o16v);
-        if constexpr (M::OUTF) store_pack<float, VEC>(outf + e0, ofv);
+        for (int k = 0; k < M::NS; k++) store_stream<float, VEC>(st.p[k] + e0, sv[u][k]);
+        if constexpr (M::OUT16) store_stream<uint16_t, VEC>(out16 + e0, o16v);
+        if constexpr (M::OUTF) store_stream<float, VEC>(outf + e0, ofv);
       }
     }
   }
@@ -286,9 +286,10 @@ static int launch_one(const typename M::G* const* g, int nP, const StateTable<M:
   SrcTable<typename M::G, (P ? P : CCN_MAX_RANKS)> tbl;
   for (int p = 0; p < (P ? P : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < nP ? p : 0];
   const size_t nvec = n / VEC;
-  const unsigned grid = stream_grid(nvec, (size_t)kBlock * UNROLL);
-  hipLaunchKernelGGL((fused_stream_kernel<M, P, VEC, UNROLL>), dim3(grid), dim3(kBlock), 0, s, tbl, nP, st, out16, outf,
-                     flag, n, prm);
+  const int streams = nP + 2 * M::NS + (M::OUT16 ? 1 : 0) + (M::OUTF ? 1 : 0);
+  const StreamLaunch L = stream_launch(nvec, (size_t)kBlock * UNROLL, streams);
+  hipLaunchKernelGGL((fused_stream_kernel<M, P, VEC, UNROLL>), dim3(L.grid), dim3(kBlock), L.lds_bytes, s, tbl, nP, st,
+                     out16, outf, flag, n, prm);
   CCN_HIP(hipGetLastError());
   return CCN_OK;
 }

@@ -67,6 +67,32 @@ unsigned stream_grid(size_t units, size_t tile) {
   return (unsigned)(need < cap ? need : cap);
 }
 
+StreamLaunch stream_launch(size_t units, size_t tile, int streams) {
+  // CCN_BLOCKS_PER_CU overrides the cap (0 = no cap); meant for tuning runs.
+  static const int forced = [] {
+    const char* e = std::getenv("CCN_BLOCKS_PER_CU");
+    return e ? std::atoi(e) : -1;
+  }();
+  int cap = forced;
+  if (cap < 0) {
+    if (streams <= 2) cap = 0;                          // copy-like: full occupancy
+    else cap = (16 + streams - 1) / streams;            // 3-4 streams: 4-6, 6-8 streams: 2-3, more: 2
+    if (cap != 0 && cap < 2) cap = 2;
+  }
+  StreamLaunch L;
+  size_t need = (units + tile - 1) / tile;
+  if (need < 1) need = 1;
+  L.grid = (unsigned)(need < 0x7fffffffull ? need : 0x7fffffffull);
+  constexpr unsigned kLdsPerCu = 160 * 1024;
+  unsigned lds = 0;
+  if (cap >= 2 && cap <= 16) {
+    lds = (kLdsPerCu / (unsigned)cap) & ~1023u;
+    if (lds > 64 * 1024) lds = 64 * 1024;               // two per CU; larger requests need an opt-in attribute
+  }
+  L.lds_bytes = lds;
+  return L;
+}
+
 }  // namespace ccn
 
 using namespace ccn;
