@@ -36,27 +36,29 @@ def parse():
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--stagger", type=int, default=0, help="extra bytes between consecutive buffers of one arena")
+    ap.add_argument("--allocator", default="ccn", choices=["ccn", "torch"],
+                    help="ccn: buffers from ccn_malloc (channel-staggered); torch: plain torch allocations")
     return ap.parse_args()
 
 
-class Arena:
-    """Carves equally sized buffers out of one torch allocation, optionally staggered by a few KiB so that the
-    P streams do not start on the same HBM channel."""
+class Buffers:
+    """Device buffers from the library's own allocator (ccn_malloc), the one the generated driver uses.  It
+    staggers buffer starts so that the P+3 arrays walked in lock step do not collide on HBM channels;
+    --allocator torch uses plain torch allocations (same-sized blocks, starts a power of two apart) instead."""
 
-    def __init__(self, torch, nbytes_each, count, stagger):
-        self.step = nbytes_each + stagger
-        assert self.step % 256 == 0
-        self.buf = torch.empty(self.step * count + 256, dtype=torch.uint8, device="cuda")
-        base = self.buf.data_ptr()
-        self.off0 = (-base) % 256
-        self.k = 0
-        self.nbytes = nbytes_each
+    def __init__(self, capi, torch, use_torch):
+        self.capi, self.torch, self.use_torch, self.keep = capi, torch, use_torch, []
 
-    def take(self, torch, dtype):
-        lo = self.off0 + self.k * self.step
-        self.k += 1
-        return self.buf[lo:lo + self.nbytes].view(dtype)
+    def from_tensor(self, t):
+        if self.use_torch:
+            self.keep.append(t)
+            return t
+        nbytes = t.numel() * t.element_size()
+        a = self.capi.malloc(nbytes)
+        self.capi.memcpy_d2d(a, t, nbytes)
+        self.torch.cuda.synchronize()
+        self.keep.append(a)
+        return a
 
 
 def traffic_from_profiles(name):
@@ -128,20 +130,20 @@ def main():
         P = a.ranks or (4 if wl == "sgd_f32" else 8)
         N = 1 << (a.log2n or (20 if wl == "sgd_f32" else 28))
         gbytes = 2 if wl == "adam_f16g" else 4
-        ar = Arena(torch, N * gbytes, P, a.stagger)
+        bufs = Buffers(capi, torch, a.allocator == "torch")
         g = []
         for p in range(P):
-            t = ar.take(torch, torch.float16 if gbytes == 2 else torch.float32)
             if gbytes == 2:
-                t.copy_((torch.randn(N, device="cuda", generator=gen) * (1e-3 * 65536.0)).to(torch.float16))
+                t = (torch.randn(N, device="cuda", generator=gen) * (1e-3 * 65536.0)).to(torch.float16)
+                if p == 0:
+                    t[::1 << 20] = float("inf")        # BASELINE config 3: one entry in 2^20 overflows
             else:
-                t.normal_(0.0, 1e-3 if wl != "sgd_f32" else 1e-2, generator=gen)
-            g.append(t)
-        ar2 = Arena(torch, N * 4, 3, a.stagger)
-        w, m, v = (ar2.take(torch, torch.float32) for _ in range(3))
-        w.uniform_(-0.05, 0.05, generator=gen)
-        m.zero_()
-        v.zero_()
+                t = torch.empty(N, device="cuda").normal_(0.0, 1e-3 if wl != "sgd_f32" else 1e-2, generator=gen)
+            g.append(bufs.from_tensor(t))
+            del t
+        w = bufs.from_tensor(torch.empty(N, device="cuda").uniform_(-0.05, 0.05, generator=gen))
+        m = bufs.from_tensor(torch.zeros(N, device="cuda"))
+        v = bufs.from_tensor(torch.zeros(N, device="cuda"))
         if wl == "adam_f32":
             per_param = (P + 3) * 4 + 3 * 4
             step = lambda t: capi.adam_f32(g, w, m, v, N, 1e-3, 0.9, 0.999, 1e-6, t, stream)
@@ -151,9 +153,8 @@ def main():
             step = lambda t: capi.sgd_f32(g, w, N, 0.01, stream)
             kernel = "fused_stream_kernel<SgdMath>"
         elif wl == "adam_f16g":
-            w16 = torch.empty(N, dtype=torch.float16, device="cuda")
+            w16 = bufs.from_tensor(torch.empty(N, dtype=torch.float16, device="cuda"))
             flag = torch.zeros(1, dtype=torch.int32, device="cuda")
-            g[0][::1 << 20] = float("inf")
             per_param = P * 2 + 12 + 12 + 2
             step = lambda t: capi.adam_f16g(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, t, 2.0 ** -16, flag, stream)
             kernel = "fused_stream_kernel<Adam16Math,8,8,1>"
@@ -166,7 +167,7 @@ def main():
         alg_bytes = float(per_param) * N
         units = N
         config = {"workload": f"{wl} fused reduce+update, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,
-                  "algorithmic_bytes_per_param": per_param, "stagger_bytes": a.stagger}
+                  "algorithmic_bytes_per_param": per_param, "allocator": a.allocator}
     elif wl == "mlp_outproj":
         M = Nn = 8192
         Kd = 1024

@@ -146,6 +146,33 @@ def device_info():
     return {"cu_count": cu.value, "hbm_bytes": hbm.value, "arch": arch.value.decode()}
 
 
+def malloc(nbytes):
+    """ccn_malloc: device memory whose start is staggered against HBM channel conflicts.  Returns the address."""
+    h = C.c_void_p()
+    _check(load().ccn_malloc(C.byref(h), nbytes), "ccn_malloc")
+    return h.value or 0
+
+
+def free(address):
+    _check(load().ccn_free(address), "ccn_free")
+
+
+def memcpy_d2d(dst, src, nbytes, stream=None):
+    _check(load().ccn_memcpy_d2d(addr(dst), addr(src), nbytes, stream), "ccn_memcpy_d2d")
+
+
+def memcpy_h2d(dst, src_host, nbytes, stream=None):
+    _check(load().ccn_memcpy_h2d(addr(dst), src_host, nbytes, stream), "ccn_memcpy_h2d")
+
+
+def memcpy_d2h(dst_host, src, nbytes, stream=None):
+    _check(load().ccn_memcpy_d2h(dst_host, addr(src), nbytes, stream), "ccn_memcpy_d2h")
+
+
+def fill_f32(dst, value, n, stream=None):
+    _check(load().ccn_fill_f32(addr(dst), value, n, stream), "ccn_fill_f32")
+
+
 class Event:
     def __init__(self):
         h = C.c_void_p()

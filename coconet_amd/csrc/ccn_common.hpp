@@ -39,66 +39,59 @@ template <typename T, int N> struct Pack {
   T d[N];
 };
 
-// Gradients and partial sums are touched once per step: stream them past the caches (nontemporal).
-template <typename T, int N> __device__ __forceinline__ Pack<T, N> load_stream(const T* p) {
-  Pack<T, N> r;
-  if constexpr (N == 1) {
-    r.d[0] = __builtin_nontemporal_load(p);
-  } else {
-    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
-    constexpr int C = (N * (int)sizeof(T)) / 16;
+// A pack moves as one scalar (N == 1), one 8-byte piece, or whole 16-byte pieces.
+template <typename T, int N> struct PackIo {
+  static constexpr int kBytes = N * (int)sizeof(T);
+  static_assert(N == 1 || kBytes == 8 || kBytes % 16 == 0, "unsupported pack size");
+  template <bool NT> static __device__ __forceinline__ Pack<T, N> load(const T* p) {
+    Pack<T, N> r;
+    if constexpr (N == 1) {
+      r.d[0] = NT ? __builtin_nontemporal_load(p) : *p;
+    } else if constexpr (kBytes == 8) {
+      const u32x2 x = NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p)) : *reinterpret_cast<const u32x2*>(p);
+      __builtin_memcpy(r.d, &x, 8);
+    } else {
 #pragma unroll
-    for (int c = 0; c < C; c++) {
-      const u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p) + c);
-      __builtin_memcpy(reinterpret_cast<char*>(r.d) + 16 * c, &x, 16);
+      for (int c = 0; c < kBytes / 16; c++) {
+        const u32x4 x = NT ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p) + c)
+                           : *(reinterpret_cast<const u32x4*>(p) + c);
+        __builtin_memcpy(reinterpret_cast<char*>(r.d) + 16 * c, &x, 16);
+      }
+    }
+    return r;
+  }
+  template <bool NT> static __device__ __forceinline__ void store(T* p, const Pack<T, N>& v) {
+    if constexpr (N == 1) {
+      if constexpr (NT) __builtin_nontemporal_store(v.d[0], p); else *p = v.d[0];
+    } else if constexpr (kBytes == 8) {
+      u32x2 x;
+      __builtin_memcpy(&x, v.d, 8);
+      if constexpr (NT) __builtin_nontemporal_store(x, reinterpret_cast<u32x2*>(p)); else *reinterpret_cast<u32x2*>(p) = x;
+    } else {
+#pragma unroll
+      for (int c = 0; c < kBytes / 16; c++) {
+        u32x4 x;
+        __builtin_memcpy(&x, reinterpret_cast<const char*>(v.d) + 16 * c, 16);
+        if constexpr (NT) __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(p) + c);
+        else *(reinterpret_cast<u32x4*>(p) + c) = x;
+      }
     }
   }
-  return r;
+};
+
+// Streaming (nontemporal) accesses: gradients, partial sums and the optimizer state are touched once per step,
+// and a step streams gigabytes past them, so nothing here is worth keeping in the caches.
+template <typename T, int N> __device__ __forceinline__ Pack<T, N> load_stream(const T* p) {
+  return PackIo<T, N>::template load<true>(p);
 }
 template <typename T, int N> __device__ __forceinline__ Pack<T, N> load_keep(const T* p) {
-  Pack<T, N> r;
-  if constexpr (N == 1) {
-    r.d[0] = *p;
-  } else {
-    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
-    constexpr int C = (N * (int)sizeof(T)) / 16;
-#pragma unroll
-    for (int c = 0; c < C; c++) {
-      const u32x4 x = *(reinterpret_cast<const u32x4*>(p) + c);
-      __builtin_memcpy(reinterpret_cast<char*>(r.d) + 16 * c, &x, 16);
-    }
-  }
-  return r;
+  return PackIo<T, N>::template load<false>(p);
+}
+template <typename T, int N> __device__ __forceinline__ void store_stream(T* p, const Pack<T, N>& v) {
+  PackIo<T, N>::template store<true>(p, v);
 }
 template <typename T, int N> __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& v) {
-  if constexpr (N == 1) {
-    *p = v.d[0];
-  } else {
-    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
-    constexpr int C = (N * (int)sizeof(T)) / 16;
-#pragma unroll
-    for (int c = 0; c < C; c++) {
-      u32x4 x;
-      __builtin_memcpy(&x, reinterpret_cast<const char*>(v.d) + 16 * c, 16);
-      *(reinterpret_cast<u32x4*>(p) + c) = x;
-    }
-  }
-}
-
-// Streaming store: the updated state is not read again before the next step has streamed ~15 GB past it.
-template <typename T, int N> __device__ __forceinline__ void store_stream(T* p, const Pack<T, N>& v) {
-  if constexpr (N == 1) {
-    __builtin_nontemporal_store(v.d[0], p);
-  } else {
-    static_assert((N * sizeof(T)) % 16 == 0, "packs move as whole 16-byte pieces");
-    constexpr int C = (N * (int)sizeof(T)) / 16;
-#pragma unroll
-    for (int c = 0; c < C; c++) {
-      u32x4 x;
-      __builtin_memcpy(&x, reinterpret_cast<const char*>(v.d) + 16 * c, 16);
-      __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(p) + c);
-    }
-  }
+  PackIo<T, N>::template store<false>(p, v);
 }
 
 // ---- table of P source pointers, passed by value in the kernel argument segment ----------------------------------
@@ -177,7 +170,11 @@ unsigned stream_grid(size_t units, size_t tile);
 // w/m/v out) loses ~10% of bandwidth at full occupancy against 2-3 workgroups per CU, while a 2-stream copy
 // wants all the occupancy it can get.  `streams` = arrays read + arrays written by the kernel.
 struct StreamLaunch { unsigned grid; unsigned lds_bytes; };
-StreamLaunch stream_launch(size_t units, size_t tile, int streams);
+StreamLaunch stream_launch(size_t units, size_t tile, int blocks_per_cu);
+
+// Measured on MI355X with 256-thread workgroups moving one 16-byte pack per stream and thread: kernels with six
+// or more streams peak at 2 workgroups per CU, four or five streams at 4, fewer want full occupancy.
+inline int blocks_per_cu_for(int streams) { return streams >= 6 ? 2 : (streams >= 4 ? 4 : 0); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -1,20 +1,23 @@
 // LAMB with per-segment trust ratio: two streaming passes and a tiny finalize kernel, no atomics.
 //
 // A plan cuts [0,N) into tiles of at most kLambTile elements that never straddle a segment boundary.
-//   pass 1   one workgroup per tile: P-way gradient reduce, m/v update, r, and the tile's sums of w^2
-//            and r^2 in float64 (lane partials -> wavefront shuffle reduction -> LDS -> one pair per tile)
+//   pass 1   one workgroup per tile, one 4-element pack per thread: P-way gradient reduce, m/v update, r, and the
+//            tile's sums of w^2 and r^2 in float64 (lane values -> wavefront shuffle reduction -> LDS -> one pair
+//            per tile)
 //   finalize one workgroup per segment: fixed-order sum of the segment's tile pairs, norms, scale
 //   pass 2   one workgroup per tile: r recomputed from the stored m, v and the old w; w updated
+// Both passes use the launch shape of the other fused kernels (one pack per thread, capped residency).
 // Arithmetic follows nccl-overlap/samples/multi-process-adam-scattered.cpp:402-449 statement by statement.
 #include "ccn_common.hpp"
 
 #include <cmath>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 namespace ccn {
 
-constexpr int kLambTile = 8192;   // elements per tile: 256 threads x float4 x 8
+constexpr int kLambTile = kBlock * 4;   // 1024 elements: one float4 per thread
 
 struct LambTile {
   uint64_t start;   // first element
@@ -24,6 +27,25 @@ struct LambTile {
   uint32_t pad[3];
 };
 static_assert(sizeof(LambTile) == 32, "tile record is 32 bytes");
+
+// Segments of one common length that is a multiple of the tile need no table: tile -> segment by division.
+struct LambLayout {
+  const LambTile* tiles;    // used when seg_len == 0
+  uint64_t seg_len;         // common segment length, or 0 for a ragged layout
+  float seg_len_f;
+};
+
+__device__ __forceinline__ LambTile lamb_tile_of(const LambLayout& L, unsigned b) {
+  if (L.seg_len != 0) {
+    LambTile t;
+    t.start = (uint64_t)b * kLambTile;
+    t.count = kLambTile;
+    t.seg = (uint32_t)(t.start / L.seg_len);
+    t.nf = L.seg_len_f;
+    return t;
+  }
+  return L.tiles[b];
+}
 
 struct LambPrm {
   float b1, omb1, b2, omb2, eps, wd, lr;
@@ -37,72 +59,70 @@ __device__ __forceinline__ float lamb_r(float mi, float vi, float w, const LambP
   return m_ / (sqrtf(v_) + k.eps) + k.wd * w;
 }
 
+// One pack of VEC elements starting at element e0.
 template <int P, int VEC>
-__device__ __forceinline__ void lamb_pass1_range(const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, int nP, const float* w,
-                                                 float* m, float* v, size_t start, uint32_t count, float nf,
-                                                 const LambPrm& k, double& accW, double& accR) {
+__device__ __forceinline__ void lamb_pass1_pack(const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, int nP, const float* w,
+                                                float* m, float* v, size_t e0, float nf, const LambPrm& k, double& accW,
+                                                double& accR) {
   const int np = P ? P : nP;
   constexpr int PX = P > 0 ? P : 1;
-  const uint32_t nvec = count / VEC;
-  for (uint32_t j = threadIdx.x; j < nvec; j += kBlock) {
-    const size_t e0 = start + (size_t)j * VEC;   // 16-byte aligned on the VEC == 4 path
-    Pack<float, VEC> gv[PX];
-    if constexpr (P > 0) {
+  Pack<float, VEC> gv[PX];
+  if constexpr (P > 0) {
 #pragma unroll
-      for (int p = 0; p < P; p++) gv[p] = load_stream<float, VEC>(g.p[p] + e0);
-    }
-    const Pack<float, VEC> wv = load_keep<float, VEC>(w + e0);
-    Pack<float, VEC> mv = load_keep<float, VEC>(m + e0);
-    Pack<float, VEC> vv = load_keep<float, VEC>(v + e0);
-    Pack<float, VEC> gs;
-    if constexpr (P > 0) {
-#pragma unroll
-      for (int e = 0; e < VEC; e++) {
-        float a = gv[0].d[e];
-#pragma unroll
-        for (int p = 1; p < P; p++) a = a + gv[p].d[e];
-        gs.d[e] = a;
-      }
-    } else {
-      gs = load_stream<float, VEC>(g.p[0] + e0);
-      for (int p = 1; p < np; p++) {
-        const Pack<float, VEC> x = load_stream<float, VEC>(g.p[p] + e0);
-#pragma unroll
-        for (int e = 0; e < VEC; e++) gs.d[e] = gs.d[e] + x.d[e];
-      }
-    }
+    for (int p = 0; p < P; p++) gv[p] = load_stream<float, VEC>(g.p[p] + e0);
+  }
+  const Pack<float, VEC> wv = load_stream<float, VEC>(w + e0);   // w is read again by pass 2, 12 GB later
+  Pack<float, VEC> mv = load_stream<float, VEC>(m + e0);
+  Pack<float, VEC> vv = load_stream<float, VEC>(v + e0);
+  Pack<float, VEC> gs;
+  if constexpr (P > 0) {
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-      const float ge = gs.d[e];
-      const float we = wv.d[e];
-      const float mi = k.b1 * mv.d[e] + k.omb1 * ge;
-      const float vi = k.b2 * vv.d[e] + k.omb2 * ge * ge;
-      const float r = lamb_r(mi, vi, we, k);
-      accR += (double)((r * r) / nf);
-      accW += (double)(we * we);
-      mv.d[e] = mi;
-      vv.d[e] = vi;
+      float a = gv[0].d[e];
+#pragma unroll
+      for (int p = 1; p < P; p++) a = a + gv[p].d[e];
+      gs.d[e] = a;
     }
-    store_pack<float, VEC>(m + e0, mv);
-    store_pack<float, VEC>(v + e0, vv);
+  } else {
+    gs = load_stream<float, VEC>(g.p[0] + e0);
+    for (int p = 1; p < np; p++) {
+      const Pack<float, VEC> x = load_stream<float, VEC>(g.p[p] + e0);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) gs.d[e] = gs.d[e] + x.d[e];
+    }
   }
+#pragma unroll
+  for (int e = 0; e < VEC; e++) {
+    const float ge = gs.d[e];
+    const float we = wv.d[e];
+    const float mi = k.b1 * mv.d[e] + k.omb1 * ge;
+    const float vi = k.b2 * vv.d[e] + k.omb2 * ge * ge;
+    const float r = lamb_r(mi, vi, we, k);
+    accR += (double)((r * r) / nf);
+    accW += (double)(we * we);
+    mv.d[e] = mi;
+    vv.d[e] = vi;
+  }
+  store_stream<float, VEC>(m + e0, mv);
+  store_stream<float, VEC>(v + e0, vv);
 }
 
 template <int P>
 __global__ __launch_bounds__(kBlock) void lamb_pass1_kernel(const SrcTable<float, (P ? P : CCN_MAX_RANKS)> g, const int nP,
-                                                            const float* w, float* m, float* v,
-                                                            const LambTile* __restrict__ tiles,
+                                                            const float* w, float* m, float* v, const LambLayout lay,
                                                             double* __restrict__ partials, const int vec_ok,
                                                             const LambPrm k) {
   __shared__ double lds[2 * kBlock / kWave];
-  const LambTile t = tiles[blockIdx.x];
+  const LambTile t = lamb_tile_of(lay, blockIdx.x);
   double accW = 0.0, accR = 0.0;
-  if (vec_ok && (t.start & 3u) == 0) {
-    const uint32_t body = t.count & ~3u;
-    lamb_pass1_range<P, 4>(g, nP, w, m, v, t.start, body, t.nf, k, accW, accR);
-    lamb_pass1_range<P, 1>(g, nP, w, m, v, t.start + body, t.count - body, t.nf, k, accW, accR);
-  } else {
-    lamb_pass1_range<P, 1>(g, nP, w, m, v, t.start, t.count, t.nf, k, accW, accR);
+  const uint32_t j0 = threadIdx.x * 4;          // this thread's elements of the tile: [j0, j0+4) clipped to count
+  if (j0 < t.count) {
+    if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+      lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR);
+    } else {
+      const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
+      for (uint32_t j = j0; j < j1; j++) lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j, t.nf, k, accW, accR);
+    }
   }
   const double sW = block_sum(accW, lds);
   const double sR = block_sum(accR, lds + kBlock / kWave);
@@ -140,37 +160,33 @@ __global__ __launch_bounds__(kBlock) void lamb_finalize_kernel(const double* __r
 }
 
 template <int VEC>
-__device__ __forceinline__ void lamb_pass2_range(float* w, const float* m, const float* v, size_t start, uint32_t count,
-                                                 float step_scale, const LambPrm& k) {
-  const uint32_t nvec = count / VEC;
-  for (uint32_t j = threadIdx.x; j < nvec; j += kBlock) {
-    const size_t e0 = start + (size_t)j * VEC;
-    Pack<float, VEC> wv = load_keep<float, VEC>(w + e0);
-    const Pack<float, VEC> mv = load_keep<float, VEC>(m + e0);
-    const Pack<float, VEC> vv = load_keep<float, VEC>(v + e0);
+__device__ __forceinline__ void lamb_pass2_pack(float* w, const float* m, const float* v, size_t e0, float step_scale,
+                                                const LambPrm& k) {
+  Pack<float, VEC> wv = load_stream<float, VEC>(w + e0);
+  const Pack<float, VEC> mv = load_stream<float, VEC>(m + e0);
+  const Pack<float, VEC> vv = load_stream<float, VEC>(v + e0);
 #pragma unroll
-    for (int e = 0; e < VEC; e++) {
-      const float we = wv.d[e];
-      const float r = lamb_r(mv.d[e], vv.d[e], we, k);
-      const float x = step_scale * r;
-      wv.d[e] = we - x;
-    }
-    store_pack<float, VEC>(w + e0, wv);
+  for (int e = 0; e < VEC; e++) {
+    const float we = wv.d[e];
+    const float r = lamb_r(mv.d[e], vv.d[e], we, k);
+    const float x = step_scale * r;
+    wv.d[e] = we - x;
   }
+  store_stream<float, VEC>(w + e0, wv);
 }
 
-__global__ __launch_bounds__(kBlock) void lamb_pass2_kernel(float* w, const float* m, const float* v,
-                                                            const LambTile* __restrict__ tiles,
+__global__ __launch_bounds__(kBlock) void lamb_pass2_kernel(float* w, const float* m, const float* v, const LambLayout lay,
                                                             const float* __restrict__ scale, const int vec_ok,
                                                             const LambPrm k) {
-  const LambTile t = tiles[blockIdx.x];
+  const LambTile t = lamb_tile_of(lay, blockIdx.x);
   const float step_scale = k.lr * scale[t.seg];   // stepsize * scale, then times r
-  if (vec_ok && (t.start & 3u) == 0) {
-    const uint32_t body = t.count & ~3u;
-    lamb_pass2_range<4>(w, m, v, t.start, body, step_scale, k);
-    lamb_pass2_range<1>(w, m, v, t.start + body, t.count - body, step_scale, k);
+  const uint32_t j0 = threadIdx.x * 4;
+  if (j0 >= t.count) return;
+  if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+    lamb_pass2_pack<4>(w, m, v, t.start + j0, step_scale, k);
   } else {
-    lamb_pass2_range<1>(w, m, v, t.start, t.count, step_scale, k);
+    const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
+    for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(w, m, v, t.start + j, step_scale, k);
   }
 }
 
@@ -183,6 +199,7 @@ struct ccn_lamb_plan {
   int nseg = 0;
   size_t N = 0;
   size_t ntiles = 0;
+  uint64_t uniform_seg_len = 0;   // non-zero: all segments have this length and it is a multiple of the tile
   LambTile* tiles = nullptr;
   uint32_t* seg_tile_begin = nullptr;
   uint64_t* seg_len = nullptr;
@@ -233,6 +250,9 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
     if (tiles.size() > 0x7fffffffu) return CCN_ERANGE;
   }
   begin[nseg] = (uint32_t)tiles.size();
+  uint64_t uniform = len[0];
+  for (int b = 1; b < nseg; b++) if (len[b] != uniform) uniform = 0;
+  if (uniform % kLambTile) uniform = 0;
 
   ccn_lamb_plan* p = new (std::nothrow) ccn_lamb_plan();
   if (!p) return CCN_ENOMEM;
@@ -240,6 +260,7 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   p->nseg = nseg;
   p->N = seg_offsets[nseg];
   p->ntiles = tiles.size();
+  p->uniform_seg_len = uniform;
   hipError_t e = hipSuccess;
   auto alloc = [&](void** ptr, size_t bytes) { if (e == hipSuccess) e = hipMalloc(ptr, bytes); };
   alloc((void**)&p->tiles, tiles.size() * sizeof(LambTile));
@@ -286,13 +307,19 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
   const int vec_ok = al ? 1 : 0;
   hipStream_t s = as_stream(stream);
   const dim3 grid((unsigned)plan->ntiles), block(kBlock);
+  LambLayout lay;
+  lay.tiles = plan->tiles;
+  lay.seg_len = vec_ok ? plan->uniform_seg_len : 0;
+  lay.seg_len_f = (float)plan->uniform_seg_len;
+  const unsigned lds1 = stream_launch(1, 1, blocks_per_cu_for(P + 5)).lds_bytes;   // P gradients + w,m,v in, m,v out
+  const unsigned lds2 = stream_launch(1, 1, blocks_per_cu_for(4)).lds_bytes;       // w,m,v in, w out
 
   auto pass1 = [&](auto ptag) {
     constexpr int PP = decltype(ptag)::value;
     SrcTable<float, (PP ? PP : CCN_MAX_RANKS)> tbl;
     for (int p = 0; p < (PP ? PP : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < P ? p : 0];
-    hipLaunchKernelGGL((lamb_pass1_kernel<PP>), grid, block, 0, s, tbl, P, (const float*)w, m, v,
-                       (const LambTile*)plan->tiles, plan->partials, vec_ok, k);
+    hipLaunchKernelGGL((lamb_pass1_kernel<PP>), grid, block, lds1, s, tbl, P, (const float*)w, m, v, lay, plan->partials,
+                       vec_ok, k);
   };
   switch (P) {
 #define CCN_CASE(K) case K: pass1(std::integral_constant<int, K>{}); break;
@@ -304,8 +331,8 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
   hipLaunchKernelGGL(lamb_finalize_kernel, dim3((unsigned)plan->nseg), block, 0, s, (const double*)plan->partials,
                      (const uint32_t*)plan->seg_tile_begin, (const uint64_t*)plan->seg_len, plan->norms, plan->scale, mode);
   CCN_HIP(hipGetLastError());
-  hipLaunchKernelGGL(lamb_pass2_kernel, grid, block, 0, s, w, (const float*)m, (const float*)v,
-                     (const LambTile*)plan->tiles, (const float*)plan->scale, vec_ok, k);
+  hipLaunchKernelGGL(lamb_pass2_kernel, grid, block, lds2, s, w, (const float*)m, (const float*)v, lay,
+                     (const float*)plan->scale, vec_ok, k);
   CCN_HIP(hipGetLastError());
   return CCN_OK;
 }
