@@ -147,7 +147,7 @@ def main():
         if wl == "adam_f32":
             per_param = (P + 3) * 4 + 3 * 4
             step = lambda t: capi.adam_f32(g, w, m, v, N, 1e-3, 0.9, 0.999, 1e-6, t, stream)
-            kernel = "fused_stream_kernel<AdamMath,8,4,2>"
+            kernel = "fused_stream_kernel<AdamMath,8,4,1>"
         elif wl == "sgd_f32":
             per_param = (P + 1) * 4 + 4
             step = lambda t: capi.sgd_f32(g, w, N, 0.01, stream)
@@ -157,7 +157,7 @@ def main():
             flag = torch.zeros(1, dtype=torch.int32, device="cuda")
             per_param = P * 2 + 12 + 12 + 2
             step = lambda t: capi.adam_f16g(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, t, 2.0 ** -16, flag, stream)
-            kernel = "fused_stream_kernel<Adam16Math,8,8,1>"
+            kernel = "fused_stream_kernel<Adam16Math,8,4,1>"
         else:
             nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
             plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
