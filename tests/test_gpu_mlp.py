@@ -1,0 +1,151 @@
+"""GPU parity tests of the model-parallel MLP out-projection (bf16 MFMA GEMM + fused epilogue) and of the
+standalone bias/dropout/residual epilogue, against the CPU oracle.
+
+Bars: dropout masks exact; the standalone epilogue is fp32 elementwise work and is bit-exact; the fused GEMM
+accumulates K bf16 products in fp32 inside the MFMA (order differs from the oracle's float64 sum), so its
+pre-rounding value is bounded by K*2^-24*sum|x||w| and the bf16 output may differ by one bf16 ulp where that
+error straddles a rounding boundary.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from util import rng
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def bf16_dev(bits):
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(DEV)
+
+
+def bf16_host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy().view(np.uint16)
+
+
+def make_case(seed, M, N, K, nP):
+    r = rng(seed)
+    X = orc.f32_to_bf16(r.standard_normal((M, K), dtype=np.float32))
+    W = orc.f32_to_bf16(r.standard_normal((K, N), dtype=np.float32) * np.float32(0.02))
+    parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N, dtype=np.float32)
+    resid = orc.f32_to_bf16(r.standard_normal((M, N), dtype=np.float32))
+    return X, W, parts, bias, resid
+
+
+def bf16_ulp_distance(a, b):
+    def key(x):
+        x = x.astype(np.int32)
+        return np.where(x & 0x8000, -(x & 0x7fff), x)
+    return np.abs(key(a) - key(b))
+
+
+@pytest.mark.parametrize("M,N,K,nP,p", [(128, 128, 64, 7, 0.1), (256, 384, 192, 7, 0.1), (128, 256, 1024, 3, 0.5),
+                                         (384, 128, 128, 0, 0.0), (128, 128, 64, 1, 0.0)])
+def test_outproj_against_oracle(ccn, M, N, K, nP, p):
+    X, W, parts, bias, resid = make_case(30 + nP, M, N, K, nP)
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(bf16_dev(X), bf16_dev(W), [torch.from_numpy(q).to(DEV) for q in parts], torch.from_numpy(bias).to(DEV),
+                         bf16_dev(resid), out, M, N, K, p, 0)
+    got = bf16_host(out).reshape(M, N)
+    want, want_f32 = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, p, 0)
+    # dropout mask: a dropped element is exactly the residual
+    keep = orc.dropout_mask(0, 0, M * N, p).reshape(M, N).astype(bool)
+    assert np.array_equal(got[~keep], resid[~keep])
+    d = bf16_ulp_distance(got, want)
+    assert d.max() <= 1, f"max bf16 ulp distance {d.max()}"
+    assert (d > 0).mean() < 0.02, f"{(d > 0).mean():.4f} of the outputs differ by one ulp"
+    gf = orc.bf16_to_f32(got)
+    assert np.max(np.abs(gf - want_f32) / (np.abs(want_f32) + 1.0)) < 2.0 ** -7
+
+
+def test_outproj_all_ones_known_answer(ccn):
+    # the reference's own check at this boundary: all-ones operands give C == K*ranks
+    # (nccl-overlap/samples/matmul-allreduce-bias-dropout-layernorm.cu:520-526)
+    M, N, K = 256, 256, 128
+    ones = lambda shape: orc.f32_to_bf16(np.ones(shape, np.float32))
+    parts = [torch.full((M, N), float(K), device=DEV) for _ in range(7)]
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(bf16_dev(ones((M, K))), bf16_dev(ones((K, N))), parts, torch.zeros(N, device=DEV), None, out,
+                         M, N, K, 0.0, 0)
+    assert np.all(orc.bf16_to_f32(bf16_host(out)) == K * 8)
+
+
+def test_outproj_tile_order_and_indexing(ccn):
+    # X = one-hot rows, W = distinct small integers: C[m][n] = W[k(m)][n] exactly, so any transposed or
+    # swizzled index in the tile loads shows up as a wrong integer
+    M, N, K = 256, 256, 128
+    r = rng(40)
+    sel = r.integers(0, K, M)
+    Xf = np.zeros((M, K), np.float32)
+    Xf[np.arange(M), sel] = 1.0
+    Wf = r.integers(-64, 64, (K, N)).astype(np.float32)
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(bf16_dev(orc.f32_to_bf16(Xf)), bf16_dev(orc.f32_to_bf16(Wf)), [], torch.zeros(N, device=DEV), None,
+                         out, M, N, K, 0.0, 0)
+    assert np.array_equal(orc.bf16_to_f32(bf16_host(out)).reshape(M, N), Wf[sel])
+
+
+@pytest.mark.parametrize("M,N,nP,p", [(64, 128, 7, 0.1), (3, 20, 2, 0.3), (1000, 36, 0, 0.0), (17, 4, 7, 0.9)])
+def test_standalone_epilogue_bit_exact(ccn, M, N, nP, p):
+    r = rng(50 + nP)
+    acc = r.standard_normal((M, N), dtype=np.float32)
+    parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N, dtype=np.float32)
+    resid = orc.f32_to_bf16(r.standard_normal((M, N), dtype=np.float32))
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.bias_dropout_residual(torch.from_numpy(acc).to(DEV), [torch.from_numpy(q).to(DEV) for q in parts],
+                              torch.from_numpy(bias).to(DEV), bf16_dev(resid), out, M, N, p, 7)
+    # oracle: the same epilogue with the product replaced by acc (K = 0 GEMM + acc as the first partial)
+    s = acc.copy()
+    for q in parts:
+        s = s + q
+    t = s + bias[None, :]
+    keep = orc.dropout_mask(7, 0, M * N, p).reshape(M, N).astype(bool)
+    scale = np.float32(1.0) / (np.float32(1.0) - np.float32(p))
+    y = np.where(keep, t * scale, np.float32(0)) + orc.bf16_to_f32(resid)
+    assert np.array_equal(bf16_host(out).reshape(M, N), orc.f32_to_bf16(y.astype(np.float32)))
+
+
+def test_outproj_config5_full_size(ccn):
+    """BASELINE config 5 at full size (8192 x 1024 x 8192, 7 partials, p = 0.1, seed 0).  Checked by:
+    the exact dropout mask over all 2^26 outputs (torch recomputes nothing: dropped outputs equal the
+    residual, kept ones almost never do), and the oracle on sampled rows."""
+    M = N = 8192
+    K = 1024
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(5)
+    X = torch.randn(M, K, device=DEV, generator=gen).to(torch.bfloat16)
+    W = (torch.randn(K, N, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+    parts = [torch.randn(M, N, device=DEV, generator=gen) for _ in range(7)]
+    bias = torch.randn(N, device=DEV, generator=gen)
+    resid = torch.randn(M, N, device=DEV, generator=gen).to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ccn.mlp_outproj_bf16(X, W, parts, bias, resid, out, M, N, K, 0.1, 0)
+    torch.cuda.synchronize()
+    rows = [0, 1, 127, 128, 4095, 4096, 8191]
+    keep_rows = np.stack([orc.dropout_mask(0, r * N, N, 0.1) for r in rows]).astype(bool)
+    Xh = X[rows].view(torch.int16).cpu().numpy().view(np.uint16)
+    Wh = W.view(torch.int16).cpu().numpy().view(np.uint16)
+    ph = [q[rows].cpu().numpy() for q in parts]
+    rh = resid[rows].view(torch.int16).cpu().numpy().view(np.uint16)
+    got = out[rows].view(torch.int16).cpu().numpy().view(np.uint16)
+    # oracle on the sampled rows: numpy float64 GEMM for the product, then the oracle's epilogue order
+    acc = (orc.bf16_to_f32(Xh).astype(np.float64) @ orc.bf16_to_f32(Wh).astype(np.float64)).astype(np.float32)
+    s = acc
+    for q in ph:
+        s = s + q
+    t = s + bias.cpu().numpy()[None, :]
+    scale = np.float32(1.0) / (np.float32(1.0) - np.float32(0.1))
+    y = np.where(keep_rows, t * scale, np.float32(0)) + orc.bf16_to_f32(rh)
+    want = orc.f32_to_bf16(y.astype(np.float32))
+    assert np.array_equal(got[~keep_rows], rh[~keep_rows])                 # mask exact on the sampled rows
+    d = bf16_ulp_distance(got, want)
+    assert d.max() <= 1 and (d > 0).mean() < 0.02
+    # over the whole output: the fraction of outputs equal to the residual is the drop rate (kept outputs equal
+    # the residual only when the scaled sum rounds away, which is rare)
+    dropped = float((out == resid).float().mean())
+    assert abs(dropped - 0.1) < 2e-3
