@@ -74,8 +74,15 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
                                                              const float* __restrict__ bias,
                                                              const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
                                                              const int M, const int N, const int K, const EpiPrm ep) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds_x[BM * BK * 2];   // [m][k] swizzled
-  __shared__ __attribute__((aligned(16))) uint8_t lds_w[BN * BK * 2];   // [n][k] swizzled (W tile transposed)
+  // main loop: X tile [m][k] and transposed W tile [n][k], 16 KiB each, chunk-swizzled.
+  // epilogue: half of the fp32 C tile, 64 rows x (128 + 4 pad) floats, to turn the MFMA register layout
+  // into whole 512-byte row segments per wavefront.
+  constexpr int kCStride = BN + 4;
+  constexpr int kLdsBytes = (BM / 2) * kCStride * 4 > 2 * BM * BK * 2 ? (BM / 2) * kCStride * 4 : 2 * BM * BK * 2;
+  __shared__ __attribute__((aligned(16))) uint8_t lds_all[kLdsBytes];
+  uint8_t* const lds_x = lds_all;
+  uint8_t* const lds_w = lds_all + BM * BK * 2;
+  float* const lds_c = reinterpret_cast<float*>(lds_all);
 
   // ---- workgroup -> tile.  Workgroups are dealt round-robin to the 8 XCDs; give each XCD a band of tile rows and
   //      walk it column by column so that the tiles resident on one XCD share X and W panels in its L2.
@@ -171,23 +178,38 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
     }
   }
 
-  // ---- epilogue: accumulator register 4*i4+e of block (bn,bm) is C[m][n+e] with
-  //      n = n0 + wn*64 + bn*32 + i4*8 + (lane/32)*4,  m = m0 + wm*64 + bm*32 + lane%32
+  // ---- epilogue.  Accumulator register 4*i4+e of block (bn,bm) is C[m][n+e] with
+  //      n = wn*64 + bn*32 + i4*8 + (lane/32)*4,  m = wm*64 + bm*32 + lane%32  (tile-local).
+  //      Read straight from HBM in that layout, a wavefront instruction would touch 32 rows x 32 bytes of every
+  //      partial buffer; going through LDS makes it 2 rows x 512 contiguous bytes.
+  for (int half = 0; half < 2; half++) {
+    __syncthreads();   // main-loop tiles (half 0) or the previous half's C rows are no longer needed
+    if (wm == half) {
 #pragma unroll
-  for (int bm = 0; bm < 2; bm++) {
-    const size_t m = m0 + wm * 64 + bm * 32 + (lane & 31);
+      for (int bm = 0; bm < 2; bm++) {
+        const int row = bm * 32 + (lane & 31);
 #pragma unroll
-    for (int bn = 0; bn < 2; bn++) {
+        for (int bn = 0; bn < 2; bn++) {
 #pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const size_t n = n0 + wn * 64 + bn * 32 + i4 * 8 + (lane >> 5) * 4;
-        f32x4 a;
-        a[0] = acc[bn][bm][i4 * 4 + 0];
-        a[1] = acc[bn][bm][i4 * 4 + 1];
-        a[2] = acc[bn][bm][i4 * 4 + 2];
-        a[3] = acc[bn][bm][i4 * 4 + 3];
-        epilogue_quad<NP>(a, parts, nPartials, bias, resid, out, m, n, (size_t)N, ep);
+          for (int i4 = 0; i4 < 4; i4++) {
+            const int col = wn * 64 + bn * 32 + i4 * 8 + (lane >> 5) * 4;
+            f32x4 a;
+            a[0] = acc[bn][bm][i4 * 4 + 0];
+            a[1] = acc[bn][bm][i4 * 4 + 1];
+            a[2] = acc[bn][bm][i4 * 4 + 2];
+            a[3] = acc[bn][bm][i4 * 4 + 3];
+            *reinterpret_cast<f32x4*>(lds_c + row * kCStride + col) = a;
+          }
+        }
       }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < (BM / 2) * (BN / 4) / kBlock; it++) {
+      const int q = it * kBlock + t;
+      const int row = q / (BN / 4), colq = q % (BN / 4);
+      const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
+      epilogue_quad<NP>(a, parts, nPartials, bias, resid, out, m0 + half * 64 + row, n0 + colq * 4, (size_t)N, ep);
     }
   }
 }
