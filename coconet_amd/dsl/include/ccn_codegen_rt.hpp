@@ -1,0 +1,339 @@
+// Runtime part of programs emitted by the HIP code-generation target.
+//
+// The code generator writes, per fused group of pipeline stages, a small "body" struct holding the user's
+// expressions as straight-line per-element code.  Everything that decides performance is hand-written here and
+// shared by all generated programs: the streaming kernel (16-byte packs, every load of a thread issued before the
+// first use, P-way gradient fold in ascending rank order, capped workgroup residency), the workgroup reductions
+// for norms, and the launch logic.  Generated programs talk to the device only through the C ABI of
+// libcoconet_hip (memory, events, the stock reduce) and hipLaunchKernelGGL for their own kernels.
+#ifndef CCN_CODEGEN_RT_HPP
+#define CCN_CODEGEN_RT_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "coconet_hip.h"
+
+#define CCNCHECK(cmd)                                                                              \
+  do {                                                                                             \
+    int _rc = (cmd);                                                                               \
+    if (_rc != CCN_OK) {                                                                           \
+      printf("Failed, coconet_hip error %s:%d '%s'\n", __FILE__, __LINE__, ccn_strerror(_rc));     \
+      exit(EXIT_FAILURE);                                                                          \
+    }                                                                                              \
+  } while (0)
+
+#define HIPCHECK(cmd)                                                                              \
+  do {                                                                                             \
+    hipError_t _e = (cmd);                                                                         \
+    if (_e != hipSuccess) {                                                                        \
+      printf("Failed: HIP error %s:%d '%s'\n", __FILE__, __LINE__, hipGetErrorString(_e));         \
+      exit(EXIT_FAILURE);                                                                          \
+    }                                                                                              \
+  } while (0)
+
+#define DIVUP(x, y) (((x) + (y)-1) / (y))
+
+namespace ccn_gen {
+
+constexpr int kBlock = 256;
+constexpr int kWave = 64;
+constexpr int kMaxRanks = CCN_MAX_RANKS;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int N> struct Vals { float d[N]; };
+
+template <int VEC> __device__ __forceinline__ Vals<VEC> load_vals(const float* p) {
+  Vals<VEC> r;
+  if constexpr (VEC == 1) {
+    r.d[0] = __builtin_nontemporal_load(p);
+  } else {
+    const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+    r.d[0] = x[0]; r.d[1] = x[1]; r.d[2] = x[2]; r.d[3] = x[3];
+  }
+  return r;
+}
+template <int VEC> __device__ __forceinline__ void store_vals(float* p, const Vals<VEC>& v) {
+  if constexpr (VEC == 1) {
+    __builtin_nontemporal_store(v.d[0], p);
+  } else {
+    f32x4 x;
+    x[0] = v.d[0]; x[1] = v.d[1]; x[2] = v.d[2]; x[3] = v.d[3];
+    __builtin_nontemporal_store(x, reinterpret_cast<f32x4*>(p));
+  }
+}
+
+// ---- counter-based dropout mask: Philox-4x32-10 on (seed, element index / 4), word index % 4 ---------------------
+__host__ __device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t k0, uint32_t k1, uint32_t out[4]) {
+  uint32_t c2 = 0, c3 = 0;
+  for (int r = 0; r < 10; r++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+__host__ __device__ inline bool dropout_keep(uint64_t seed, uint64_t idx, float p_drop) {
+  uint32_t w[4];
+  const uint64_t blk = idx >> 2;
+  philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)seed, (uint32_t)(seed >> 32), w);
+  const float u = (float)(w[idx & 3] >> 8) * 5.9604644775390625e-08f;
+  return u >= p_drop;
+}
+// Dropout as the emitted expressions use it: drop with probability p, scale survivors by 1/(1-p).
+__host__ __device__ inline float dropout(float x, float p_drop, uint64_t seed, uint64_t idx) {
+  return dropout_keep(seed, idx, p_drop) ? x * (1.0f / (1.0f - p_drop)) : 0.0f;
+}
+
+// ---- reductions ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ double wave_sum(double x) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, kWave);
+  return x;
+}
+__device__ __forceinline__ double block_sum(double x, double* lds) {
+  x = wave_sum(x);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = x;
+  __syncthreads();
+  double r = 0.0;
+  if (threadIdx.x == 0)
+    for (int k = 0; k < kBlock / kWave; k++) r += lds[k];
+  __syncthreads();
+  return r;
+}
+
+// ---- kernel arguments ---------------------------------------------------------------------------------------------
+// A generated Body declares:
+//   NIN        plain fp32 input arrays, read at the element index
+//   NOUT       fp32 output arrays (an in-place update lists the array under both)
+//   HAS_RED    the body's first operand is the sum over rank buffers (the lowered AllReduce / ReduceScatter)
+//   NACC       sums of squares the body accumulates (inputs of Norm stages), float64
+//   NNORM      finished norms the body reads
+//   struct Scalars
+//   static void apply(float red, const float* in, float* out, const Scalars&, double* acc, const float* norms, uint64_t idx)
+template <class Body> struct KernelArgs {
+  const float* red[kMaxRanks];
+  int nranks;
+  const float* in[Body::NIN > 0 ? Body::NIN : 1];
+  float* out[Body::NOUT > 0 ? Body::NOUT : 1];
+  double* partials;      // NACC values per workgroup
+  const float* norms;    // NNORM values
+  size_t n;
+  typename Body::Scalars s;
+};
+
+template <class Body, int P, int VEC>
+__global__ __launch_bounds__(kBlock) void fused_pointwise_kernel(const KernelArgs<Body> a) {
+  constexpr int NINX = Body::NIN > 0 ? Body::NIN : 1;
+  constexpr int NOUTX = Body::NOUT > 0 ? Body::NOUT : 1;
+  constexpr int NACCX = Body::NACC > 0 ? Body::NACC : 1;
+  constexpr int PX = P > 0 ? P : 1;
+  __shared__ double lds[kBlock / kWave];
+  const size_t nvec = a.n / VEC;
+  double acc[NACCX];
+#pragma unroll
+  for (int k = 0; k < NACCX; k++) acc[k] = 0.0;
+  float nrm[Body::NNORM > 0 ? Body::NNORM : 1];
+#pragma unroll
+  for (int k = 0; k < Body::NNORM; k++) nrm[k] = a.norms[k];
+
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (size_t)gridDim.x * kBlock) {
+    const size_t e0 = i * VEC;
+    Vals<VEC> rv[PX];
+    Vals<VEC> iv[NINX];
+    Vals<VEC> red;
+    if constexpr (Body::HAS_RED && P > 0) {
+#pragma unroll
+      for (int p = 0; p < P; p++) rv[p] = load_vals<VEC>(a.red[p] + e0);
+    }
+#pragma unroll
+    for (int k = 0; k < Body::NIN; k++) iv[k] = load_vals<VEC>(a.in[k] + e0);
+    if constexpr (Body::HAS_RED) {
+      if constexpr (P > 0) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          float s = rv[0].d[e];
+#pragma unroll
+          for (int p = 1; p < P; p++) s = s + rv[p].d[e];
+          red.d[e] = s;
+        }
+      } else {
+        red = load_vals<VEC>(a.red[0] + e0);
+        for (int p = 1; p < a.nranks; p++) {
+          const Vals<VEC> x = load_vals<VEC>(a.red[p] + e0);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) red.d[e] = red.d[e] + x.d[e];
+        }
+      }
+    }
+    Vals<VEC> ov[NOUTX];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      float in1[NINX], out1[NOUTX];
+#pragma unroll
+      for (int k = 0; k < Body::NIN; k++) in1[k] = iv[k].d[e];
+      Body::apply(Body::HAS_RED ? red.d[e] : 0.0f, in1, out1, a.s, acc, nrm, (uint64_t)(e0 + e));
+#pragma unroll
+      for (int k = 0; k < Body::NOUT; k++) ov[k].d[e] = out1[k];
+    }
+#pragma unroll
+    for (int k = 0; k < Body::NOUT; k++) store_vals<VEC>(a.out[k] + e0, ov[k]);
+  }
+
+  if constexpr (VEC > 1) {   // the last n % VEC elements, scalar, by the first lanes of workgroup 0
+    const size_t rem = a.n - nvec * VEC;
+    if (blockIdx.x == 0 && threadIdx.x < rem) {
+      const size_t i = nvec * VEC + threadIdx.x;
+      float red = 0.0f;
+      if constexpr (Body::HAS_RED) {
+        red = a.red[0][i];
+        for (int p = 1; p < a.nranks; p++) red = red + a.red[p][i];
+      }
+      float in1[NINX], out1[NOUTX];
+      for (int k = 0; k < Body::NIN; k++) in1[k] = a.in[k][i];
+      Body::apply(red, in1, out1, a.s, acc, nrm, (uint64_t)i);
+      for (int k = 0; k < Body::NOUT; k++) a.out[k][i] = out1[k];
+    }
+  }
+
+  if constexpr (Body::NACC > 0) {
+#pragma unroll
+    for (int k = 0; k < Body::NACC; k++) {
+      const double s = block_sum(acc[k], lds);
+      if (threadIdx.x == 0) a.partials[(size_t)blockIdx.x * Body::NACC + k] = s;
+    }
+  }
+}
+
+// norms[k] = sqrt(sum over workgroups of partials[b*nacc + k]); one workgroup, fixed order: deterministic.
+__global__ __launch_bounds__(kBlock) void finalize_norms_kernel(const double* partials, unsigned nblocks, int nacc, float* norms) {
+  __shared__ double lds[kBlock / kWave];
+  for (int k = 0; k < nacc; k++) {
+    double s = 0.0;
+    for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) s += partials[(size_t)b * nacc + k];
+    const double t = block_sum(s, lds);
+    if (threadIdx.x == 0) norms[k] = (float)sqrt(t);
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------------------------
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Resident workgroups per CU for a kernel that walks `streams` arrays (measured on MI355X: many-stream kernels
+// reach the most HBM bandwidth with few wavefronts in flight), as unused dynamic LDS.
+inline unsigned lds_cap_bytes(int streams) {
+  const int cap = streams >= 6 ? 2 : (streams >= 4 ? 4 : 0);
+  if (cap == 0) return 0;
+  unsigned lds = (160u * 1024u / (unsigned)cap) & ~1023u;
+  return lds > 64u * 1024u ? 64u * 1024u : lds;
+}
+
+inline unsigned grid_for(size_t n, int vec) {
+  size_t need = DIVUP(n / vec > 0 ? n / vec : 1, (size_t)kBlock);
+  return (unsigned)(need < 0x7fffffffull ? need : 0x7fffffffull);
+}
+
+template <class Body, int VEC> void launch_vec(const KernelArgs<Body>& a, hipStream_t s) {
+  const unsigned grid = grid_for(a.n, VEC);
+  const int streams = (Body::HAS_RED ? a.nranks : 0) + Body::NIN + Body::NOUT;
+  const unsigned lds = lds_cap_bytes(streams);
+  const int P = Body::HAS_RED ? a.nranks : 1;
+  switch (P) {
+#define CCN_GEN_CASE(K) \
+  case K: hipLaunchKernelGGL((fused_pointwise_kernel<Body, K, VEC>), dim3(grid), dim3(kBlock), lds, s, a); break;
+    CCN_GEN_CASE(1) CCN_GEN_CASE(2) CCN_GEN_CASE(3) CCN_GEN_CASE(4) CCN_GEN_CASE(5) CCN_GEN_CASE(6) CCN_GEN_CASE(7)
+    CCN_GEN_CASE(8)
+#undef CCN_GEN_CASE
+    default: hipLaunchKernelGGL((fused_pointwise_kernel<Body, 0, VEC>), dim3(grid), dim3(kBlock), lds, s, a); break;
+  }
+  HIPCHECK(hipGetLastError());
+}
+
+// Number of workgroups launch() will use (the size of the partials array is NACC times this).
+inline unsigned blocks_for(size_t n) { return grid_for(n, 1); }
+
+template <class Body> void launch(const KernelArgs<Body>& a, void* stream) {
+  if (a.n == 0) return;
+  bool al = true;
+  if (Body::HAS_RED)
+    for (int p = 0; p < a.nranks; p++) al = al && aligned16(a.red[p]);
+  for (int k = 0; k < Body::NIN; k++) al = al && aligned16(a.in[k]);
+  for (int k = 0; k < Body::NOUT; k++) al = al && aligned16(a.out[k]);
+  if (al) launch_vec<Body, 4>(a, (hipStream_t)stream);
+  else launch_vec<Body, 1>(a, (hipStream_t)stream);
+}
+
+inline void finalize_norms(const double* partials, size_t n, bool vec, int nacc, float* norms, void* stream) {
+  const unsigned nblocks = grid_for(n, vec ? 4 : 1);
+  hipLaunchKernelGGL(finalize_norms_kernel, dim3(1), dim3(kBlock), 0, (hipStream_t)stream, partials, nblocks, nacc, norms);
+  HIPCHECK(hipGetLastError());
+}
+
+// ---- input generation and checking (host) ----------------------------------------------------------------------------
+// The reference fills inputs with cuRAND uniform(0,1), seed 1234 (examples/header.h:64-76); cuRAND is not
+// available, so a splitmix64 stream with the same seed and range takes its place.
+inline float uniform01(uint64_t seed, uint64_t i) {
+  uint64_t z = seed + 0x9E3779B97F4A7C15ull * (i + 1);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return (float)((z >> 40) + 1) * 5.9604644775390625e-08f;   // (0, 1]
+}
+
+inline void fill_uniform(float* dev, size_t n, uint64_t seed, std::vector<float>* keep = nullptr) {
+  std::vector<float> h(n);
+  for (size_t i = 0; i < n; i++) h[i] = uniform01(seed, i);
+  CCNCHECK(ccn_memcpy_h2d(dev, h.data(), n * sizeof(float), nullptr));
+  CCNCHECK(ccn_stream_sync(nullptr));
+  if (keep) keep->swap(h);
+}
+
+// relative comparison in the spirit of the reference's eqFloat (examples/header.h:55-62), with a tighter bound:
+// the emitted kernels round exactly like the emitted host loops except for the association of norm sums.
+inline bool eqFloat(float ref, float got, float tol = 1e-5f) {
+  if (ref == got) return true;
+  if (std::isnan(ref) || std::isnan(got)) return std::isnan(ref) && std::isnan(got);
+  const float den = std::fabs(ref) > 1e-30f ? std::fabs(ref) : 1e-30f;
+  return std::fabs(ref - got) / den <= tol;
+}
+
+inline bool compare(const char* what, const std::vector<float>& ref, const float* dev, size_t n, float tol = 1e-5f) {
+  std::vector<float> got(n);
+  CCNCHECK(ccn_memcpy_d2h(got.data(), dev, n * sizeof(float), nullptr));
+  for (size_t i = 0; i < n; i++) {
+    if (!eqFloat(ref[i], got[i], tol)) {
+      printf("Mismatch in %s at %zu : ref '%.9g', computed '%.9g'\n", what, i, ref[i], got[i]);
+      return false;
+    }
+  }
+  return true;
+}
+
+// ---- bf16 on the host (round-to-nearest-even), for programs that feed the MFMA GEMM ---------------------------------
+inline uint16_t f32_to_bf16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return (uint16_t)(x >> 16);
+}
+inline float bf16_to_f32(uint16_t h) {
+  const uint32_t x = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &x, 4);
+  return f;
+}
+
+}  // namespace ccn_gen
+
+#endif

@@ -1,0 +1,106 @@
+// Small pipelines exercising the front end's rules, one per command-line case; driven by tests/test_dsl.py.
+// A case either prints the pipeline (Pipeline::print) and exits 0, or is expected to abort through ASSERT.
+#include <dsl.hpp>
+#include <pipeline.hpp>
+
+#include <sstream>
+
+using namespace ACCCDSL;
+
+struct AdamParts {
+  Variable N{Int32, "N"};
+  Variable lr{Float32, "lr"}, beta1{Float32, "beta1"}, beta2{Float32, "beta2"};
+  Tensor g{Float32, N, Local, "g"};
+  Tensor w{Float32, N, Replicated, "w"}, m{Float32, N, Replicated, "m"}, v{Float32, N, Replicated, "v"};
+  Stage g1 = AllReduce(Summation, g);
+  Stage m1 = Update(m, beta1 * m + (1 - beta1) * g1);
+  Stage v1 = Update(v, beta2 * v + (1 - beta2) * g1 * g1);
+  Stage m_ = m1 / beta1;
+  Stage v_ = v1 / beta2;
+  Stage w1 = Update(w, w - lr * (m_ / v_));
+};
+
+int main(int argc, char** argv) {
+  const std::string c = argc > 1 ? argv[1] : "";
+  if (c == "print_unfused" || c == "print_fused" || c == "print_all_fused") {
+    AdamParts a;
+    Pipeline pl("adam", {a.g, a.w, a.m, a.v, a.lr, a.beta1, a.beta2}, {a.m1, a.v1, a.w1});
+    if (c == "print_fused") pl.fuse({a.m1, a.v1, a.m_, a.v_, a.w1});
+    if (c == "print_all_fused") pl.fuse({a.g1, a.m1, a.v1, a.m_, a.v_, a.w1});
+    pl.print(std::cout);
+    return 0;
+  }
+  if (c == "fuse_skips_consumer") {
+    // g1 -> m1 -> m_ ; fusing {g1, m_} while m1 stays outside makes the fused kernel both feed m1 and read it
+    AdamParts a;
+    Pipeline pl("adam", {a.g, a.w, a.m, a.v, a.lr, a.beta1, a.beta2}, {a.m1, a.v1, a.w1});
+    pl.fuse({a.g1, a.m_});
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "fuse_unreachable") {
+    AdamParts a;
+    Stage stray = a.w * a.lr;
+    Pipeline pl("adam", {a.g, a.w, a.m, a.v, a.lr, a.beta1, a.beta2}, {a.m1, a.v1, a.w1});
+    pl.fuse({a.m1, stray});
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "allreduce_of_replicated") {
+    Variable N(Int32, "N");
+    Tensor w(Float32, N, Replicated, "w");
+    Stage s = AllReduce(Summation, w);
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "allgather_of_replicated") {
+    Variable N(Int32, "N");
+    Tensor w(Float32, N, Replicated, "w");
+    Stage s = AllGather(w);
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "local_read_without_collective") {
+    Variable N(Int32, "N");
+    Variable lr(Float32, "lr");
+    Tensor g(Float32, N, Local, "g");
+    Tensor w(Float32, N, Replicated, "w");
+    Stage g1 = AllReduce(Summation, g);
+    Stage w1 = Update(w, w - lr * g1 + g);
+    Pipeline pl("bad", {g, w, lr}, {w1});
+    std::cout << generateHIP(pl, {});
+    return 0;
+  }
+  if (c == "missing_argument") {
+    Variable N(Int32, "N");
+    Variable lr(Float32, "lr");
+    Tensor g(Float32, N, Local, "g");
+    Tensor w(Float32, N, Replicated, "w");
+    Stage g1 = AllReduce(Summation, g);
+    Stage w1 = Update(w, w - lr * g1);
+    Pipeline pl("bad", {g, w}, {w1});   // lr not listed
+    std::cout << generateHIP(pl, {});
+    return 0;
+  }
+  if (c == "sliced_layouts") {
+    // the RS_C_AG shape: slices flow through the pointwise stages and are gathered at the end
+    Variable N(Int32, "N");
+    Variable lr(Float32, "lr");
+    Tensor g(Float32, N, Local, "g");
+    Tensor w(Float32, N, Replicated, "w");
+    Stage g1 = ReduceScatter(Summation, g);
+    Stage w1 = Scatter(w) - lr * g1;
+    Stage w2 = Update(w, AllGather(w1));
+    Pipeline pl("sgd", {g, w, lr}, {w2});
+    pl.print(std::cout);
+    return 0;
+  }
+  if (c == "bad_file") {
+    AdamParts a;
+    Pipeline pl("adam", {a.g, a.w, a.m, a.v, a.lr, a.beta1, a.beta2}, {a.m1, a.v1, a.w1});
+    pl.codegen("/nonexistent-dir/x.cu");
+    return 0;
+  }
+  std::cout << "unknown case" << std::endl;
+  return 64;
+}

@@ -1,0 +1,78 @@
+// DSL programs for the BASELINE configurations, written against the CoCoNet API.
+//   ccn-programs <program> <schedule> [output.hip]
+// program: sgd | adam | lamb     schedule: unfused | fused
+#include <dsl.hpp>
+#include <pipeline.hpp>
+
+#include <cstring>
+
+using namespace ACCCDSL;
+
+// w <- w - lr * sum_p g_p   (BASELINE config 1)
+static void sgd(bool fused, const std::string& out) {
+  Variable N(Int32, "N");
+  Variable lr(Float32, "lr");
+  Tensor w(Float32, N, Replicated, "w");
+  Tensor g(Float32, N, Local, "g");
+  Stage gsum = AllReduce(Summation, g);
+  Stage wnew = Update(w, w - lr * gsum);
+  Pipeline pl("sgd", {g, w, lr}, {wnew});
+  if (fused) pl.fuse({gsum, wnew});
+  pl.codegen(out);
+}
+
+// bias-corrected Adam (BASELINE config 2).  The DSL has no pow(), so the caller passes the two bias
+// corrections 1-beta^t as scalars; eps as well.
+static void adam(bool fused, const std::string& out) {
+  Variable N(Int32, "N");
+  Variable lr(Float32, "lr"), b1(Float32, "beta1"), b2(Float32, "beta2"), eps(Float32, "eps");
+  Variable c1(Float32, "bias1"), c2(Float32, "bias2");
+  Tensor g(Float32, N, Local, "g");
+  Tensor w(Float32, N, Replicated, "w"), m(Float32, N, Replicated, "m"), v(Float32, N, Replicated, "v");
+  Stage gs = AllReduce(Summation, g);
+  Stage mn = Update(m, b1 * m + (1 - b1) * gs);
+  Stage vn = Update(v, b2 * v + (1 - b2) * gs * gs);
+  Stage mhat = mn / c1;
+  Stage vhat = vn / c2;
+  Stage wn = Update(w, w - lr * mhat / (Sqrt(vhat) + eps));
+  Pipeline pl("adam", {g, w, m, v, lr, b1, b2, eps, c1, c2}, {mn, vn, wn});
+  if (fused) pl.fuse({gs, mn, vn, mhat, vhat, wn});
+  else pl.fuse({mn, vn, mhat, vhat, wn});
+  pl.codegen(out);
+}
+
+// LAMB with one global trust ratio (the DSL's Norm is over the whole tensor)
+static void lamb(bool fused, const std::string& out) {
+  Variable N(Int32, "N");
+  Variable lr(Float32, "lr"), b1(Float32, "beta1"), b2(Float32, "beta2"), eps(Float32, "eps"), wd(Float32, "wd");
+  Variable c1(Float32, "bias1"), c2(Float32, "bias2");
+  Tensor g(Float32, N, Local, "g");
+  Tensor w(Float32, N, Replicated, "w"), m(Float32, N, Replicated, "m"), v(Float32, N, Replicated, "v");
+  Stage gs = AllReduce(Summation, g);
+  Stage mn = Update(m, b1 * m + (1 - b1) * gs);
+  Stage vn = Update(v, b2 * v + (1 - b2) * gs * gs);
+  Stage r = (mn / c1) / (Sqrt(vn / c2) + eps) + wd * w;
+  Stage rn = Norm(r);
+  Stage wnorm = Norm(w);
+  Stage wn = Update(w, w - lr * (wnorm / rn) * r);
+  Pipeline pl("lamb", {g, w, m, v, lr, b1, b2, eps, wd, c1, c2}, {wn});
+  if (fused) pl.fuse({gs, mn, vn, r, rn, wnorm, wn});
+  else pl.fuse({mn, vn, r, rn, wnorm, wn});
+  pl.codegen(out);
+}
+
+int main(int argc, char** argv) {
+  if (argc < 3) {
+    std::cout << "usage: " << argv[0] << " <sgd|adam|lamb> <unfused|fused> [output.hip]" << std::endl;
+    return 1;
+  }
+  const std::string prog = argv[1], sched = argv[2];
+  const bool fused = sched == "fused";
+  if (!fused && sched != "unfused") { std::cout << "Invalid schedule" << std::endl; return 1; }
+  const std::string out = argc > 3 ? argv[3] : prog + "-" + sched + ".hip";
+  if (prog == "sgd") sgd(fused, out);
+  else if (prog == "adam") adam(fused, out);
+  else if (prog == "lamb") lamb(fused, out);
+  else { std::cout << "Invalid program" << std::endl; return 1; }
+  return 0;
+}

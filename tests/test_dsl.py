@@ -1,0 +1,174 @@
+"""The C++ DSL front end and the HIP code-generation target (CPU side): API conformance with the reference's
+example programs, fusion legality, storage classes, the error convention, and the text of emitted kernels."""
+import ast
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DSL = os.path.join(ROOT, "coconet_amd", "dsl")
+BUILD = os.path.join(DSL, "build")
+REF = "/root/reference"
+
+
+@pytest.fixture(scope="module")
+def dsl_build():
+    subprocess.check_call(["make", "-C", DSL, "-s", "-j8", "all"])
+    return BUILD
+
+
+def run(exe, *args, cwd=None):
+    return subprocess.run([exe, *args], capture_output=True, text=True, cwd=cwd)
+
+
+def test_storage_classes_and_fusion_groups(dsl_build):
+    chk = os.path.join(dsl_build, "ccn-dsl-check")
+    unf = run(chk, "print_unfused").stdout
+    assert unf.count("kernel ") == 6 and "register" not in unf          # every stage is its own kernel, all in memory
+    fused = run(chk, "print_fused").stdout
+    assert fused.count("kernel ") == 2
+    # reference rule (src/pipeline.hpp:360-387): values consumed only inside the fused kernel stay in registers,
+    # Update targets and outputs are memory
+    assert "S3 [Replicated, register]" in fused and "S4 [Replicated, register]" in fused
+    assert "S0 [Replicated, memory] = AllReduce(g)" in fused
+    assert "S5 [Replicated, memory, output] = Update(w" in fused
+    allf = run(chk, "print_all_fused").stdout
+    assert allf.count("kernel ") == 1 and "S0 [Replicated, register] = AllReduce(g)" in allf
+    sl = run(chk, "sliced_layouts").stdout
+    assert "S0 [Sliced" in sl and "S1 [Sliced" in sl and "S2 [Replicated, memory, output] = Update(w, AllGather(S1))" in sl
+
+
+@pytest.mark.parametrize("case,needle", [
+    ("fuse_skips_consumer", "fuse:"),               # reference spec hint: tests/fusion-test.cpp:68-83
+    ("fuse_unreachable", "not reachable"),          # tests/fusion-test.cpp:34-49
+    ("allreduce_of_replicated", "must be Local"),
+    ("allgather_of_replicated", "must be Sliced"),
+    ("local_read_without_collective", "is Local"),
+    ("missing_argument", "not a pipeline argument"),
+])
+def test_invalid_programs_abort_with_a_message(dsl_build, case, needle):
+    """Error convention of the reference (src/ast.hpp:33-44): message on stderr, then std::terminate()."""
+    r = run(os.path.join(dsl_build, "ccn-dsl-check"), case)
+    assert r.returncode != 0 and "not rejected" not in r.stdout
+    assert "ASSERT failed" in r.stderr and needle in r.stderr
+
+
+def test_unwritable_output_reports_and_returns(dsl_build):
+    r = run(os.path.join(dsl_build, "ccn-dsl-check"), "bad_file")       # src/pipeline.hpp:656-663
+    assert r.returncode == 0 and "Error opening file" in r.stdout
+
+
+# ---- emitted text --------------------------------------------------------------------------------------------------------
+def canon(expr, rename):
+    """Expression tree with identifiers renamed and the operands of + and * sorted: equal canon() means equal
+    grouping, i.e. the same floating-point result (commuting a single + or * does not change it)."""
+    def go(n):
+        if isinstance(n, ast.BinOp):
+            op = type(n.op).__name__
+            a, b = go(n.left), go(n.right)
+            if op in ("Add", "Mult"):
+                a, b = sorted([a, b], key=repr)
+            return (op, a, b)
+        if isinstance(n, ast.Call):
+            return ("call", go(n.func), tuple(go(a) for a in n.args))
+        if isinstance(n, ast.Name):
+            return rename.get(n.id, n.id)
+        if isinstance(n, ast.Constant):
+            return float(n.value)
+        if isinstance(n, ast.UnaryOp):
+            return ("neg", go(n.operand))
+        raise AssertionError(ast.dump(n))
+    return go(ast.parse(expr, mode="eval").body)
+
+
+def emitted_statements(text):
+    text = re.sub(r"\bs\.", "", text)
+    return dict(re.findall(r"const float (v_S\d+) = (.*);", text))
+
+
+def test_emitted_expressions_keep_the_users_grouping(dsl_build, tmp_path):
+    exe = os.path.join(dsl_build, "ccn-programs")
+    out = tmp_path / "adam.hip"
+    assert run(exe, "adam", "fused", str(out)).returncode == 0
+    st = emitted_statements(out.read_text())
+    ren = {"in_m": "m", "in_v": "v", "in_w": "w", "v_S0": "gs", "red": "gs", "v_S1": "m1", "v_S2": "v1", "v_S3": "mh", "v_S4": "vh"}
+    assert canon(st["v_S1"], ren) == canon("beta1*m + (1 - beta1)*gs", ren)
+    assert canon(st["v_S2"], ren) == canon("beta2*v + ((1 - beta2)*gs)*gs", ren)          # left to right, as the checker
+    assert canon(st["v_S2"], ren) != canon("beta2*v + (1 - beta2)*(gs*gs)", ren)
+    assert canon(st["v_S5"], ren) == canon("w - (lr*mh)/(sqrtf(vh) + eps)", ren)
+    text = out.read_text()
+    assert "HAS_RED = true" in text and "ccn_reduce_f32" not in text                       # reduce fused into the kernel
+    unf = tmp_path / "adam-u.hip"
+    assert run(exe, "adam", "unfused", str(unf)).returncode == 0
+    t2 = unf.read_text()
+    assert "ccn_reduce_f32(g, comm_size, g[0]" in t2 and "HAS_RED = false" in t2
+    assert re.search(r'printf\("\{SZ: %ld, Epochs: %d, AllReduce: %f, kernel0: %f, Total: %f\}', t2)   # reference line format
+
+
+def test_two_pass_lowering_of_norms(dsl_build, tmp_path):
+    exe = os.path.join(dsl_build, "ccn-programs")
+    out = tmp_path / "lamb.hip"
+    assert run(exe, "lamb", "fused", str(out)).returncode == 0
+    text = out.read_text()
+    assert "lamb_body0_pass1" in text and "lamb_body0_pass2" in text and "finalize_norms" in text
+    p1 = text[text.index("struct lamb_body0_pass1"):text.index("struct lamb_body0_pass2")]
+    p2 = text[text.index("struct lamb_body0_pass2"):text.index("void lamb(")]
+    assert "NACC = 2" in p1 and p1.count("acc[") == 2 and "out[2]" not in p1       # pass 1 stores m, v only
+    assert "NNORM = 2" in p2 and "HAS_RED = false" in p2                            # pass 2 does not re-read gradients
+    assert "nrm[1] / nrm[0]" in p2                                                   # wNorm / rNorm
+
+
+@pytest.mark.skipif(not os.path.isdir(REF), reason="reference tree not present")
+def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path):
+    """API conformance: the reference's own DSL programs build against these headers from where they lie and every
+    schedule produces a program."""
+    for ex, schedules in [("sgd", ["AR_C", "RS_C_AG", "fuse_RS_C_AG"]), ("adam", ["AR_C", "RS_C_AG", "fuse_RS_C_AG"]),
+                          ("lamb", ["AR_C", "RS_C_AG", "fuse_RS_C_AG"]),
+                          ("model-parallel", ["MM_AR_C", "MM_RS_C_AG", "ol_MM_fuse_RS_C_AG"])]:
+        exe = os.path.join(dsl_build, "ex-" + ex)
+        assert os.path.exists(exe), exe
+        for s in schedules:
+            r = run(exe, s, cwd=tmp_path)
+            assert r.returncode == 0, r.stderr
+    made = sorted(f for f in os.listdir(tmp_path) if f.endswith(".hip"))
+    assert len(made) == 12 and "adam-fuse-rs-c-ag.hip" in made
+    fused = (tmp_path / "adam-fuse-rs-c-ag.hip").read_text()
+    assert "HAS_RED = true" in fused and "ccn_memcpy_d2d" not in fused       # RS + compute + AG in one kernel
+    unf = (tmp_path / "adam-rs-c-ag.hip").read_text()
+    assert "ccn_reduce_f32" in unf and "ccn_memcpy_d2d(w, S5" in unf         # ReduceScatter, kernel, AllGather
+    mlp = (tmp_path / "model-parallel-mm-ar-c.hip").read_text()
+    assert "ccn_mlp_outproj_bf16" in mlp and "p_drop = 0.5f" in mlp
+
+
+@pytest.mark.skipif(not os.path.exists(os.path.join(ROOT, "oracle", "_ref", "ref-adam")), reason="oracle/_ref not built")
+def test_expression_grouping_matches_the_reference_generator(dsl_build, tmp_path):
+    """Text oracle: the reference's own generator (built from its sources into oracle/_ref) and this target must
+    emit expressions with the same grouping for the reference's adam program."""
+    ref_dir = tmp_path / "ref"
+    ref_dir.mkdir()
+    assert run(os.path.join(ROOT, "oracle", "_ref", "ref-adam"), "AR_C", cwd=ref_dir).returncode == 0
+    cu = (ref_dir / "adam-ar-c.cu").read_text()
+    cu = cu.replace("[i0]", "")
+    ref_stmt = dict(re.findall(r"^\s*(\w+) = (.*);$", cu[:cu.index("void adam(")], flags=re.M))
+    mine_dir = tmp_path / "mine"
+    mine_dir.mkdir()
+    assert run(os.path.join(dsl_build, "ex-adam"), "AR_C", cwd=mine_dir).returncode == 0
+    st = emitted_statements((mine_dir / "adam-ar-c.hip").read_text())
+    mine_ren = {"in_m": "m", "in_v": "v", "in_w": "w", "in_S0": "g", "v_S1": "m", "v_S2": "v", "v_S3": "S3", "v_S4": "S4"}
+    assert canon(st["v_S1"], mine_ren) == canon(ref_stmt["m"], {})
+    assert canon(st["v_S2"], mine_ren) == canon(ref_stmt["v"], {})
+    assert canon(st["v_S3"], mine_ren) == canon(ref_stmt["S3"], {})
+    assert canon(st["v_S5"], mine_ren) == canon(ref_stmt["w"], {})
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="no hipcc")
+def test_emitted_programs_were_cross_compiled(dsl_build):
+    """__graft_entry__.build() runs `make gen`; the binaries are what the GPU tests execute."""
+    gen = os.path.join(dsl_build, "gen")
+    if not os.path.isdir(gen):
+        subprocess.check_call(["make", "-C", DSL, "-s", "-j8", "gen"])
+    for name in ("sgd-fused", "adam-fused", "adam-unfused", "lamb-fused"):
+        assert os.access(os.path.join(gen, name), os.X_OK), name

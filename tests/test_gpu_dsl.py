@@ -1,0 +1,83 @@
+"""GPU tests of the programs the HIP code-generation target emits: each binary (cross-compiled in-tree by
+`make -C coconet_amd/dsl gen`) runs its pipeline on the GPU, re-executes it on the CPU stage by stage with the
+fixed-order P-way sum, compares, and prints the reference's "{SZ: ..., Epochs: ..., <step>: ms, Total: ms}" lines."""
+import os
+import re
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GEN = os.path.join(ROOT, "coconet_amd", "dsl", "build", "gen")
+LINE = re.compile(r"^\{SZ: (\d+), Epochs: (\d+)((?:, \w+: [0-9.eE+-]+)+)\}$")
+
+OWN = ["sgd-fused", "sgd-unfused", "adam-fused", "adam-unfused", "lamb-fused", "lamb-unfused"]
+REF = ["ref-sgd-ar-c", "ref-sgd-rs-c-ag", "ref-sgd-fuse-rs-c-ag", "ref-adam-ar-c", "ref-adam-rs-c-ag",
+       "ref-adam-fuse-rs-c-ag", "ref-lamb-ar-c", "ref-lamb-rs-c-ag", "ref-lamb-fuse-rs-c-ag"]
+
+
+def run_program(name, *args):
+    exe = os.path.join(GEN, name)
+    if not os.path.exists(exe):
+        pytest.skip(f"{name} was not built (make -C coconet_amd/dsl gen)")
+    r = subprocess.run([exe, *map(str, args)], capture_output=True, text=True, timeout=240)
+    assert "do not match" not in r.stdout and "Mismatch" not in r.stdout, r.stdout[-2000:]
+    assert r.returncode == 0, (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
+    rows = []
+    for line in r.stdout.splitlines():
+        m = LINE.match(line.strip())
+        if m:
+            fields = dict(re.findall(r"(\w+): ([0-9.eE+-]+)", m.group(3)))
+            rows.append((int(m.group(1)), int(m.group(2)), {k: float(v) for k, v in fields.items()}))
+    return rows
+
+
+@pytest.mark.parametrize("name", OWN)
+@pytest.mark.parametrize("ranks", [1, 4, 8, 11])
+def test_own_programs_check_themselves(name, ranks):
+    # sizes 2^10 .. 2^21 with the CPU re-execution switched on
+    rows = run_program(name, 2, ranks, 10, 21, 1)
+    assert [r[0] for r in rows] == [1 << k for k in range(10, 22)]
+    for size, epochs, f in rows:
+        assert epochs == 2 and abs(sum(v for k, v in f.items() if k != "Total") - f["Total"]) < 1e-3
+    steps = set(rows[0][2]) - {"Total"}
+    assert steps == ({"kernel0"} if name.endswith("-fused") else {"AllReduce", "kernel0"})
+
+
+@pytest.mark.parametrize("name", REF)
+def test_programs_emitted_from_the_reference_examples(name):
+    """The reference's examples/{sgd,adam,lamb}/*.cpp, compiled unmodified against this front end, every schedule."""
+    rows = run_program(name, 2, 4, 10, 20, 1)
+    assert len(rows) == 11
+    steps = set(rows[0][2]) - {"Total"}
+    if "fuse" in name:
+        assert steps == {"kernel0"}
+    elif "rs-c-ag" in name:
+        assert steps == {"ReduceScatter", "kernel0", "AllGather"}
+    else:
+        assert steps == {"AllReduce", "kernel0"}
+
+
+def test_unaligned_size_takes_scalar_tail():
+    # 2^k sizes never leave a tail; an odd size comes from the explicit bounds path of another program, so run the
+    # smallest sweep point with 3 ranks instead: the kernel's n % 4 tail code is covered by N = 2^10 only when
+    # buffers are unaligned -- here we simply make sure tiny sizes work
+    rows = run_program("adam-fused", 1, 3, 1, 9, 1)
+    assert [r[0] for r in rows] == [1 << k for k in range(1, 10)]
+
+
+def test_model_parallel_program():
+    rows = run_program("ref-model-parallel-mm-ar-c", 2, 8, 1)
+    # B in {8, 16}, S = 1024, H = 3072: M = B*S rows, N = 3072
+    assert [r[0] for r in rows] == [8 * 1024 * 3072, 16 * 1024 * 3072]
+    assert all("MatMulFused" in r[2] for r in rows)
+
+
+def test_fusion_pays_off_at_config2_size():
+    """The point of CoCoNet's fusion, measured: at N = 2^28, P = 8 the fused schedule must beat
+    all-reduce-then-update by a clear margin (one pass over the gradients instead of two)."""
+    fused = run_program("adam-fused", 5, 8, 28, 28, 0)[0][2]["Total"]
+    unfused = run_program("adam-unfused", 5, 8, 28, 28, 0)[0][2]["Total"]
+    assert fused < 0.85 * unfused, (fused, unfused)
