@@ -311,9 +311,10 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
   lay.tiles = plan->tiles;
   lay.seg_len = vec_ok ? plan->uniform_seg_len : 0;
   lay.seg_len_f = (float)plan->uniform_seg_len;
-  const unsigned lds1 = stream_launch(1, 1, blocks_per_cu_for(P + 5)).lds_bytes;   // P gradients + w,m,v in, m,v out
-  const unsigned lds2 = stream_launch(1, 1, blocks_per_cu_for(4)).lds_bytes;       // w,m,v in, w out
-
+  // Residency caps measured for config 4 (N = 2^28, P = 8): pass 1 is fastest at 4 workgroups per CU (its float64
+  // sums and the workgroup reduction need more wavefronts to hide than the plain Adam kernel), pass 2 uncapped.
+  const unsigned lds1 = stream_launch(1, 1, P >= 2 ? 4 : 0).lds_bytes;
+  const unsigned lds2 = 0;
   auto pass1 = [&](auto ptag) {
     constexpr int PP = decltype(ptag)::value;
     SrcTable<float, (PP ? PP : CCN_MAX_RANKS)> tbl;
