@@ -21,6 +21,7 @@ CCN_ERANGE = -34
 CCN_MAX_RANKS = 16
 LAMB_TRUST_RATIO = 0
 LAMB_REFERENCE = 1
+LAMB_NCCL_GLOBAL = 2
 
 # every symbol include/coconet_hip.h declares
 SYMBOLS = [

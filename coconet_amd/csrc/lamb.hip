@@ -54,6 +54,7 @@ struct LambPrm {
 };
 
 __device__ __forceinline__ float lamb_r(float mi, float vi, float w, const LambPrm& k) {
+  if (k.mode == CCN_LAMB_NCCL_GLOBAL) return ((mi / k.b1)) / sqrtf((vi / k.b2)) + k.wd * w;
   const float m_ = (float)((double)mi / k.bc1);
   const float v_ = (float)((double)vi / k.bc2);
   return m_ / (sqrtf(v_) + k.eps) + k.wd * w;
@@ -95,10 +96,16 @@ __device__ __forceinline__ void lamb_pass1_pack(const SrcTable<float, (P ? P : C
   for (int e = 0; e < VEC; e++) {
     const float ge = gs.d[e];
     const float we = wv.d[e];
-    const float mi = k.b1 * mv.d[e] + k.omb1 * ge;
-    const float vi = k.b2 * vv.d[e] + k.omb2 * ge * ge;
+    float mi, vi;
+    if (k.mode == CCN_LAMB_NCCL_GLOBAL) {
+      vi = ((vv.d[e] * k.b2) + ((ge * ge) * k.omb2));
+      mi = ((mv.d[e] * k.b1) + (ge * k.omb1));
+    } else {
+      mi = k.b1 * mv.d[e] + k.omb1 * ge;
+      vi = k.b2 * vv.d[e] + k.omb2 * ge * ge;
+    }
     const float r = lamb_r(mi, vi, we, k);
-    accR += (double)((r * r) / nf);
+    accR += k.mode == CCN_LAMB_NCCL_GLOBAL ? (double)(r * r) : (double)((r * r) / nf);
     accW += (double)(we * we);
     mv.d[e] = mi;
     vv.d[e] = vi;
@@ -149,7 +156,12 @@ __global__ __launch_bounds__(kBlock) void lamb_finalize_kernel(const double* __r
   }
   const double sW = block_sum(aW, lds);
   const double sR = block_sum(aR, lds + kBlock / kWave);
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0 && mode == CCN_LAMB_NCCL_GLOBAL) {
+    const float wNorm = sqrtf((float)sW), rNorm = sqrtf((float)sR);
+    norms[2 * b] = wNorm;
+    norms[2 * b + 1] = rNorm;
+    scale[b] = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f) / rNorm;
+  } else if (threadIdx.x == 0) {
     const double rNorm = sqrt(sR);
     const double wNorm = sqrt(sW / (double)seg_len[b]);
     const double ratio = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f);
@@ -283,7 +295,7 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
 int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, float* m, float* v, float lr, float beta1,
                  float beta2, float eps, float wd, int step, int mode, void* stream) {
   if (!plan || !g || !w || !m || !v || P < 1 || P > CCN_MAX_RANKS || step < 1) return CCN_EINVAL;
-  if (mode != CCN_LAMB_TRUST_RATIO && mode != CCN_LAMB_REFERENCE) return CCN_EINVAL;
+  if (mode != CCN_LAMB_TRUST_RATIO && mode != CCN_LAMB_REFERENCE && mode != CCN_LAMB_NCCL_GLOBAL) return CCN_EINVAL;
   for (int p = 0; p < P; p++) if (!g[p]) return CCN_EINVAL;
   const DeviceInfo* di = nullptr;
   int rc = current_device_info(&di);

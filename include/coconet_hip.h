@@ -39,6 +39,10 @@ extern "C" {
 
 #define CCN_LAMB_TRUST_RATIO 0  /* scale = W/R                         (textbook)                      */
 #define CCN_LAMB_REFERENCE   1  /* scale = (W/R)/R  as the reference's kernel and checker compute it   */
+#define CCN_LAMB_NCCL_GLOBAL 2  /* the modified NCCL's global-norm LAMB: m/beta1, v/beta2 in place of bias correction,
+                                   r = S3/sqrtf(S4) + wd*w, L2 norms, scale = (W/R)/R in fp32; eps and step unused
+                                   (nccl/src/collectives/device/reduce_kernel.h:391-452, common_kernel.h:2211-2273,
+                                   2687-2726).  One segment covering [0,N) reproduces its single global norm. */
 
 /* ---- runtime glue: what the generated driver needs instead of cudaMalloc / events
  *      (reference: emitted main(), src/codegen.cpp:4583-4784; examples/header.h:36-53) ---- */

@@ -256,9 +256,50 @@ uint32_t orc_overflow_f16(const uint16_t* const* g, int P, size_t N) {
  * The hard-coded 1.0f is the weight-decay factor wd here (wd = 1.0f reproduces the reference bit for bit).
  * mode 1 keeps the reference's second division by rNorm; mode 0 drops it (textbook trust ratio).
  * ---------------------------------------------------------------------------------------------- */
+/* mode 2: the modified NCCL's LAMB (global-norm variant), per segment:
+ *   functors nccl/src/collectives/device/reduce_kernel.h:391-452 (binOp1, binOp2, binOp3, binOp4, rOp, delta,
+ *   weightUpdate) in the call order of common_kernel.h:2211-2273 (phase 1) and :2687-2726 (phase 2);
+ *   norms all_reduce_computation.h:931-978.
+ *   v = (v*b2) + ((gs*gs)*(1-b2));  S4 = v/b2;  m = (m*b1) + (gs*(1-b1));  S3 = m/b1;
+ *   r = S3/sqrtf(S4) + 1.0f*w;  wNorm = sqrtf(sum w^2), rNorm = sqrtf(sum r^2)   (L2 norms, no division by n)
+ *   scale = ((wNorm>0) ? (rNorm>0 ? wNorm/rNorm : 1) : 1)/rNorm  in fp32;  w = w - (lr*scale)*r
+ * The kernel accumulates the two sums in fp32 through shuffles and atomics, i.e. in no fixed order; the oracle
+ * accumulates in float64 and rounds once, which every fp32 order approximates.  eps and step are not used;
+ * wd takes the place of the hard-coded 1.0f. */
+static void lamb_nccl_segment(const float* const* g, int P, float* w, float* m, float* v, size_t lo, size_t hi,
+                              float lr, float beta1, float beta2, float wd, double* norms_out) {
+  double rr = 0.0, ww = 0.0;
+  for (size_t i = lo; i < hi; i++) {
+    float gs = reduce_at(g, P, i);
+    float vi = ((v[i] * beta2) + ((gs * gs) * (1 - beta2)));
+    float S4 = (vi / beta2);
+    float mi = ((m[i] * beta1) + (gs * (1 - beta1)));
+    float S3 = (mi / beta1);
+    float r = (S3) / sqrtf(S4) + wd * w[i];
+    ww += (double)(w[i] * w[i]);
+    rr += (double)(r * r);
+    v[i] = vi;
+    m[i] = mi;
+  }
+  const float wNorm = sqrtf((float)ww), rNorm = sqrtf((float)rr);
+  if (norms_out) { norms_out[0] = wNorm; norms_out[1] = rNorm; }
+  const float scale = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f) / rNorm;
+  for (size_t i = lo; i < hi; i++) {
+    float r = ((m[i] / beta1)) / sqrtf((v[i] / beta2)) + wd * w[i];
+    float delta = (lr * scale) * r;
+    w[i] = w[i] - delta;
+  }
+}
+
 void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
                   const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2,
                   float eps, float wd, int step, int mode, double* norms_out) {
+  if (mode == 2) {
+    for (int b = 0; b < nseg; b++)
+      lamb_nccl_segment(g, P, w, m, v, seg_offsets[b], seg_offsets[b + 1], lr, beta1, beta2, wd,
+                        norms_out ? norms_out + 2 * b : NULL);
+    return;
+  }
   const double bc1 = 1 - pow((double)beta1, (double)step);
   const double bc2 = 1 - pow((double)beta2, (double)step);
   const float stepsize = lr;

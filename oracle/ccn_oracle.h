@@ -22,6 +22,8 @@
  *   orc_adam_f32          nccl-overlap/samples/multi-process-adam-scattered.cpp:112-136;
  *                         reference integer fixture, torch.optim.Adam (CPU) cross-check, step-1 closed form   pinned
  *   orc_lamb_f32          same file :402-449; single-segment/w==0 special cases, float64 brute force  pinned
+ *                         (mode 2: nccl/.../reduce_kernel.h:391-452; all-ones closed form, float64 brute force;
+ *                          the reference sums its norms in fp32 in no fixed order: norm rounding parity unpinned)
  *   orc_adam_f16g         no counterpart in the reference (it has no loss scaling / overflow detection):
  *                         build-defined, pinned by closed forms only; parity with Apex "parity unpinned"
  *   orc_philox4x32_10     Random123 known-answer vectors                         pinned
@@ -78,7 +80,8 @@ uint32_t orc_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, floa
 uint32_t orc_overflow_f16(const uint16_t* const* g, int P, size_t N);
 
 /* ---- LAMB with per-segment norms.  seg_offsets has nseg+1 entries, seg_offsets[nseg] == N.
- *      mode 0: scale = trust ratio W/R;  mode 1 (reference): scale = (W/R)/R.
+ *      mode 0: scale = trust ratio W/R;  mode 1 (reference): scale = (W/R)/R;
+ *      mode 2: the modified NCCL's global-norm LAMB arithmetic (divide by beta, L2 norms, no eps).
  *      norms_out (optional, 2*nseg doubles): W_b, R_b after the square root. ---- */
 void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
                   const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2,

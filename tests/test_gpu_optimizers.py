@@ -415,3 +415,31 @@ def test_lamb_full_size_segments(ccn):
     del g
     plan.close()
     assert norms.shape == (nseg, 2) and np.all(norms > 0)
+
+
+def test_lamb_nccl_global_variant(ccn):
+    """The modified NCCL's global-norm LAMB arithmetic (mode 2): its all-ones known answer and parity on random data.
+    m, v bit-exact; the norms are rounded to fp32 from float64 sums on both sides; w within 1e-6."""
+    for P in (2, 8):
+        N = 4096
+        ones = [torch.ones(N, device=DEV) for _ in range(P)]
+        w, m, v = (torch.zeros(N, device=DEV) for _ in range(3))
+        plan = ccn.LambPlan([0, N])
+        plan.step(ones, w, m, v, 1.0, 0.5, 0.5, 0.0, 1.0, 1, ccn.LAMB_NCCL_GLOBAL)
+        assert np.all(host(w) == np.float32(-1.0 / 64.0)) and np.all(host(m) == P / 2)
+        plan.close()
+    P, N = 8, 200003
+    g = grads_f32(61, P, N, 1e-2)
+    w0 = weights_f32(61, N, 0.05)
+    m0 = weights_f32(62, N, 0.01)
+    v0 = np.abs(weights_f32(63, N, 1e-3)) + np.float32(1e-5)
+    wd, md, vd = dev(w0), dev(m0), dev(v0)
+    plan = ccn.LambPlan([0, N])
+    plan.step([dev(x) for x in g], wd, md, vd, 1e-3, 0.9, 0.999, 0.0, 1.0, 1, ccn.LAMB_NCCL_GLOBAL)
+    w, m, v = w0.copy(), m0.copy(), v0.copy()
+    norms = orc.lamb_f32(g, w, m, v, [0, N], 1e-3, 0.9, 0.999, 0.0, 1.0, 1, 2)
+    assert_f32_parity(host(md), m, "nccl-lamb m")
+    assert_f32_parity(host(vd), v, "nccl-lamb v")
+    assert rel_err(plan.norms(), norms) < 1e-6
+    assert np.max(np.abs(host(wd).astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
+    plan.close()

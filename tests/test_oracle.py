@@ -395,3 +395,39 @@ def test_mlp_outproj_float64_brute_force_and_all_ones():
     parts1 = [np.full((M, N), K, np.float32) for _ in range(7)]
     _, outf = orc.mlp_outproj(X1, W1, parts1, np.zeros(N, np.float32), None, M, N, K, 0.0, 0)
     assert np.all(outf == K * 8)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the modified NCCL's global-norm LAMB arithmetic (mode 2)
+# ---------------------------------------------------------------------------------------------------------------------
+def test_lamb_nccl_global_all_ones_closed_form():
+    # all-ones gradients on P ranks, w = m = v = 0, beta = .5, lr = 1 (the inputs of examples/test-adam.cu:73-88):
+    # v = P^2/2, S4 = P^2, m = P/2, S3 = P, r = P/P + 0 = 1, W = 0, R = sqrt(N), scale = 1/R, w = -1/sqrt(N)
+    for P in (2, 8):
+        N = 4096
+        g = [np.ones(N, np.float32) for _ in range(P)]
+        w, m, v = (np.zeros(N, np.float32) for _ in range(3))
+        norms = orc.lamb_f32(g, w, m, v, [0, N], 1.0, 0.5, 0.5, 0.0, 1.0, 1, 2)
+        assert np.all(m == P / 2) and np.all(v == P * P / 2)
+        assert norms[0, 0] == 0.0 and norms[0, 1] == 64.0
+        assert np.all(w == np.float32(-1.0 / 64.0))
+
+
+def test_lamb_nccl_global_float64_brute_force():
+    P, N = 4, 5000
+    g = grads_f32(60, P, N, 1e-2)
+    w0 = weights_f32(60, N, 0.05)
+    m0 = (rng(60, 50).standard_normal(N) * 1e-2).astype(np.float32)
+    v0 = (rng(60, 51).uniform(1e-5, 1e-3, N)).astype(np.float32)
+    w, m, v = w0.copy(), m0.copy(), v0.copy()
+    b1, b2, lr = float(np.float32(0.9)), float(np.float32(0.999)), float(np.float32(1e-3))
+    norms = orc.lamb_f32(g, w, m, v, [0, N], lr, b1, b2, 0.0, 1.0, 1, 2)
+    gs = np.sum(np.stack(g).astype(np.float64), axis=0)
+    vv = v0 * b2 + gs * gs * (1 - b2)
+    mm = m0 * b1 + gs * (1 - b1)
+    r = (mm / b1) / np.sqrt(vv / b2) + w0
+    W, R = np.sqrt(np.sum(w0.astype(np.float64) ** 2)), np.sqrt(np.sum(r ** 2))
+    assert abs(norms[0, 0] / W - 1) < 1e-6 and abs(norms[0, 1] / R - 1) < 1e-6
+    expect = w0 - lr * (W / R / R) * r
+    assert np.max(np.abs(w - expect)) < 1e-6 * np.max(np.abs(expect))
+    assert np.max(np.abs(m - mm)) < 1e-6 * np.max(np.abs(mm)) and np.max(np.abs(v - vv)) < 1e-6 * np.max(np.abs(vv))
