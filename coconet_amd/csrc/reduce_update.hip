@@ -2,7 +2,7 @@
 //
 // One streaming skeleton (fused_stream_kernel) is instantiated with a math policy per optimizer.
 // The skeleton owns the memory behaviour: 128-bit loads of every operand, all loads of a tile issued
-// before the first use, grid-stride over the shard, in-place 128-bit stores.  The policy owns the
+// before the first use, one tile per workgroup, in-place 128-bit stores.  The policy owns the
 // arithmetic, written operation by operation in the order of the reference's checker loops so that
 // every fp32 rounding happens where the checker's does (the library is compiled with
 // -ffp-contract=off; division and square root are the correctly rounded ones).
@@ -28,7 +28,6 @@ struct SumF32 {
   using G = float;
   using Acc = float;
   static constexpr int PACK_BYTES = 16;
-  static int blocks_per_cu(int streams) { return blocks_per_cu_for(streams); }
   template <class Prm> static __device__ __forceinline__ Acc first(G x, const Prm&) { return x; }
   template <class Prm> static __device__ __forceinline__ void next(Acc& a, G x, const Prm&) { a = a + x; }
 };
@@ -111,10 +110,7 @@ struct AdamMath : SumF32 {
 // fp16 gradients with a loss scale; overflow = any rank's element has exponent 0x1F.
 struct Adam16Math {
   using G = uint16_t;
-  // fp16 gradients move as 8-byte packs (4 elements per thread): measured 76% of HBM peak at 4 workgroups per CU
-  // against 70% with 16-byte packs of 8 elements at 2.
-  static constexpr int PACK_BYTES = 8;
-  static int blocks_per_cu(int streams) { return streams >= 6 ? 4 : 0; }
+  static constexpr int PACK_BYTES = 8;   // fp16 gradients move as 8-byte packs: 76% of HBM peak against 70% with 16-byte packs
   struct Acc { float s; bool bad; };
   static constexpr int NS = 3, UNROLL = 1;
   static constexpr bool OUT16 = true, OUTF = false, FLAG = true;
@@ -135,10 +131,7 @@ struct Adam16Math {
 
 struct Overflow16Math {
   using G = uint16_t;
-  // fp16 gradients move as 8-byte packs (4 elements per thread): measured 76% of HBM peak at 4 workgroups per CU
-  // against 70% with 16-byte packs of 8 elements at 2.
-  static constexpr int PACK_BYTES = 8;
-  static int blocks_per_cu(int streams) { return streams >= 6 ? 4 : 0; }
+  static constexpr int PACK_BYTES = 8;   // fp16 gradients move as 8-byte packs: 76% of HBM peak against 70% with 16-byte packs
   using Acc = bool;
   static constexpr int NS = 0, UNROLL = 1;
   static constexpr bool OUT16 = false, OUTF = false, FLAG = true;
@@ -151,10 +144,7 @@ struct Overflow16Math {
 // nccl/src/collectives/device/reduce_kernel.h:36-68 in the call order of common_kernel.h:875-921
 struct FusedAdamRefMath {
   using G = uint16_t;
-  // fp16 gradients move as 8-byte packs (4 elements per thread): measured 76% of HBM peak at 4 workgroups per CU
-  // against 70% with 16-byte packs of 8 elements at 2.
-  static constexpr int PACK_BYTES = 8;
-  static int blocks_per_cu(int streams) { return streams >= 6 ? 4 : 0; }
+  static constexpr int PACK_BYTES = 8;   // fp16 gradients move as 8-byte packs: 76% of HBM peak against 70% with 16-byte packs
   using Acc = uint16_t;   // the ring carries the running sum in fp16
   static constexpr int NS = 3, UNROLL = 1;
   static constexpr bool OUT16 = true, OUTF = false, FLAG = false;
@@ -180,8 +170,9 @@ struct FusedAdamRefMath {
 };
 
 // ------------------------------------------------------------------------------------------------------------------
-// The streaming skeleton.  P > 0: rank count known at compile time (all P loads in flight together).
-// P == 0: rank count nP read at run time (ranks 9..16), loads folded one rank at a time.
+// The streaming skeleton.  P > 0: rank count known at compile time.  P == 0: rank count nP (9..16) read at run
+// time; the loads of ranks >= nP are skipped by wavefront-uniform branches.  Either way all loads of a thread
+// are in flight together before the first use.
 // VEC elements per thread per access; n counts elements.  Elements [ (n/VEC)*VEC, n ) are finished
 // by the first lanes of workgroup 0 with scalar accesses.
 // ------------------------------------------------------------------------------------------------------------------
@@ -204,58 +195,49 @@ __device__ __forceinline__ void one_element(const SrcTable<typename M::G, (P ? P
   if constexpr (M::OUTF) outf[i] = of;
 }
 
-template <class M, int P, int VEC, int UNROLL>
-__global__ __launch_bounds__(kBlock) void fused_stream_kernel(
+template <class M, int P, int VEC, int UNROLL, int BS>
+__global__ __launch_bounds__(BS) void fused_stream_kernel(
     const SrcTable<typename M::G, (P ? P : CCN_MAX_RANKS)> g, const int nP, const StateTable<M::NS> st,
     uint16_t* out16, float* outf, uint32_t* flag, const size_t n, const typename M::Prm prm) {
   using G = typename M::G;
   constexpr int NSX = M::NS > 0 ? M::NS : 1;
-  constexpr int PX = P > 0 ? P : 1;
+  constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;   // P == 0: rank count nP (9..16) known at run time only
   const size_t nvec = n / VEC;
-  const size_t tile = (size_t)kBlock * UNROLL;
   bool bad = false;
-
-  for (size_t t0 = (size_t)blockIdx.x * tile; t0 < nvec; t0 += (size_t)gridDim.x * tile) {
+  // One tile per workgroup, no loop: wavefronts here live for a single pack per array, so every instruction
+  // ahead of the first load is exposed latency (a grid-stride loop's bookkeeping costs ~3% of bandwidth).
+  // The y dimension of the grid only comes into play beyond 2^31 tiles.
+  const size_t blk = (size_t)blockIdx.x + (size_t)blockIdx.y * gridDim.x;
+  const size_t t0 = blk * ((size_t)BS * UNROLL);
+  {
     Pack<G, VEC> gv[UNROLL][PX];
     Pack<float, VEC> sv[UNROLL][NSX];
     typename M::Acc acc[UNROLL][VEC];
     // ---- issue every load of the tile -------------------------------------------------------------------------
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
-      const size_t e0 = (t0 + (size_t)u * kBlock + threadIdx.x) * VEC;   // first element of this thread's pack
+      const size_t e0 = (t0 + (size_t)u * BS + threadIdx.x) * VEC;   // first element of this thread's pack
       if (e0 < nvec * VEC) {
-        if constexpr (P > 0) {
 #pragma unroll
-          for (int p = 0; p < P; p++) gv[u][p] = load_stream<G, VEC>(g.p[p] + e0);
-        }
+        for (int p = 0; p < PX; p++)
+          if (P > 0 || p < nP) gv[u][p] = load_stream<G, VEC>(g.p[p] + e0);
 #pragma unroll
         for (int k = 0; k < M::NS; k++) sv[u][k] = load_stream<float, VEC>(st.p[k] + e0);
-        if constexpr (P == 0) {
-          for (int p = 0; p < nP; p++) {
-            const Pack<G, VEC> x = load_stream<G, VEC>(g.p[p] + e0);
-#pragma unroll
-            for (int e = 0; e < VEC; e++) {
-              if (p == 0) acc[u][e] = M::first(x.d[e], prm);
-              else M::next(acc[u][e], x.d[e], prm);
-            }
-          }
-        }
       }
     }
     // ---- fold, update, store ---------------------------------------------------------------------------------
 #pragma unroll
     for (int u = 0; u < UNROLL; u++) {
-      const size_t e0 = (t0 + (size_t)u * kBlock + threadIdx.x) * VEC;
+      const size_t e0 = (t0 + (size_t)u * BS + threadIdx.x) * VEC;
       if (e0 < nvec * VEC) {
         Pack<uint16_t, VEC> o16v;
         Pack<float, VEC> ofv;
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
-          if constexpr (P > 0) {
-            acc[u][e] = M::first(gv[u][0].d[e], prm);
+          acc[u][e] = M::first(gv[u][0].d[e], prm);
 #pragma unroll
-            for (int p = 1; p < P; p++) M::next(acc[u][e], gv[u][p].d[e], prm);
-          }
+          for (int p = 1; p < PX; p++)
+            if (P > 0 || p < nP) M::next(acc[u][e], gv[u][p].d[e], prm);
           float s[NSX];
 #pragma unroll
           for (int k = 0; k < M::NS; k++) s[k] = sv[u][k].d[e];
@@ -277,7 +259,7 @@ __global__ __launch_bounds__(kBlock) void fused_stream_kernel(
 
   if constexpr (VEC > 1) {
     const size_t rem = n - nvec * VEC;
-    if (blockIdx.x == 0 && threadIdx.x < rem) one_element<M, P>(g, nP, st, out16, outf, nvec * VEC + threadIdx.x, prm, bad);
+    if (blk == 0 && threadIdx.x < rem) one_element<M, P>(g, nP, st, out16, outf, nvec * VEC + threadIdx.x, prm, bad);
   }
 
   if constexpr (M::FLAG) {
@@ -302,9 +284,17 @@ static int launch_one(const typename M::G* const* g, int nP, const StateTable<M:
   for (int p = 0; p < (P ? P : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < nP ? p : 0];
   const size_t nvec = n / VEC;
   const int streams = nP + 2 * M::NS + (M::OUT16 ? 1 : 0) + (M::OUTF ? 1 : 0);
-  const StreamLaunch L = stream_launch(nvec, (size_t)kBlock * UNROLL, M::blocks_per_cu(streams));
-  hipLaunchKernelGGL((fused_stream_kernel<M, P, VEC, UNROLL>), dim3(L.grid), dim3(kBlock), L.lds_bytes, s, tbl, nP, st,
-                     out16, outf, flag, n, prm);
+  const StreamShape sh = stream_shape(streams, VEC * (int)sizeof(typename M::G));
+  size_t tiles = (nvec + (size_t)sh.block * UNROLL - 1) / ((size_t)sh.block * UNROLL);
+  if (tiles < 1) tiles = 1;                                     // the n % VEC tail still needs workgroup 0
+  const size_t gx = tiles < 0x40000000ull ? tiles : 0x40000000ull;
+  const dim3 grid((unsigned)gx, (unsigned)((tiles + gx - 1) / gx));
+  if (sh.block == 64)
+    hipLaunchKernelGGL((fused_stream_kernel<M, P, VEC, UNROLL, 64>), grid, dim3(64), sh.lds_bytes, s, tbl, nP, st, out16,
+                       outf, flag, n, prm);
+  else
+    hipLaunchKernelGGL((fused_stream_kernel<M, P, VEC, UNROLL, 256>), grid, dim3(256), sh.lds_bytes, s, tbl, nP, st,
+                       out16, outf, flag, n, prm);
   CCN_HIP(hipGetLastError());
   return CCN_OK;
 }

@@ -90,6 +90,31 @@ StreamLaunch stream_launch(size_t units, size_t tile, int streams /* requested w
   return L;
 }
 
+StreamShape stream_shape(int streams, int pack_bytes) {
+  // CCN_BLOCK / CCN_LDS_KB override the shape; meant for tuning runs.
+  static const int f_block = [] { const char* e = std::getenv("CCN_BLOCK"); return e ? std::atoi(e) : 0; }();
+  static const int f_lds = [] { const char* e = std::getenv("CCN_LDS_KB"); return e ? std::atoi(e) : -1; }();
+  StreamShape sh;
+  // Single-wavefront workgroups, and as many of them per CU as keeps (16-byte streams x wavefronts) near 100:
+  // measured optima on MI355X at N = 2^28 are 7 wavefronts per CU for the 14-stream fp32 Adam kernel (85% of HBM
+  // peak; 6 or 8 give 82-83%), 13 for the 6-stream SGD kernel (84%) and 12-13 for the fp16-gradient Adam kernel,
+  // whose 15 streams move 8-byte packs (80%).
+  const int eq_streams = (streams * pack_bytes + 15) / 16;
+  if (eq_streams <= 3) {
+    sh.block = 256;                 // copy-like kernels want all the occupancy they can get
+    sh.lds_bytes = 0;
+  } else {
+    int waves = (98 + eq_streams / 2) / eq_streams;
+    if (waves < 6) waves = 6;
+    if (waves > 13) waves = 13;
+    sh.block = 64;
+    sh.lds_bytes = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
+  }
+  if (f_block == 64 || f_block == 256) sh.block = f_block;
+  if (f_lds >= 0 && f_lds <= 64) sh.lds_bytes = (unsigned)f_lds * 1024u;
+  return sh;
+}
+
 }  // namespace ccn
 
 using namespace ccn;
