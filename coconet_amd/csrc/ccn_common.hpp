@@ -9,6 +9,7 @@ namespace ccn {
 
 constexpr int kBlock = 256;        // 4 wavefronts of 64 lanes
 constexpr int kWave = 64;
+constexpr size_t kLdsPerCu = 160 * 1024;   // LDS bytes of one gfx950 compute unit
 
 // ---- host-side error plumbing -----------------------------------------------------------------------------------
 extern thread_local int g_last_hip_error;

@@ -1,16 +1,21 @@
-// LAMB with per-segment trust ratio: two streaming passes and a tiny finalize kernel, no atomics.
+// LAMB with per-segment trust ratio.  The update of a segment needs the segment's two norms, which need every element
+// of the segment first, so each element is visited twice.  A plan sorts the segments into two groups:
 //
-// A plan cuts [0,N) into tiles of at most kLambTile elements that never straddle a segment boundary.
-//   pass 1   one workgroup per tile, one 4-element pack per thread: P-way gradient reduce, m/v update, r, and the
-//            tile's sums of w^2 and r^2 in float64 (lane values -> wavefront shuffle reduction -> LDS -> one pair
-//            per tile)
+// resident segments (short enough for the chip to hold between the visits: 2 tiles per workgroup of a grid that fills
+//   the GPU once, 4 M elements at the default shape) go through one persistent kernel.  A workgroup runs pass 1 on a
+//   tile (P-way gradient reduce, m/v update, r, the tile's float64 sums of w^2 and r^2), parks r and the old w in
+//   LDS, and one round later, when the workgroup that finished the segment's last tile has published the scale,
+//   writes w from what it parked: 56 bytes per element instead of 68.  No sum is an atomic accumulation: tile sums
+//   are stored one by one and added in a fixed order, so results do not depend on scheduling.
+// the other segments take two streaming passes with a finalize kernel between them:
+//   pass 1   one workgroup per tile of kLambTile elements, one 4-element pack per thread
 //   finalize one workgroup per segment: fixed-order sum of the segment's tile pairs, norms, scale
 //   pass 2   one workgroup per tile: r recomputed from the stored m, v and the old w; w updated
-// Both passes use the launch shape of the other fused kernels (one pack per thread, capped residency).
 // Arithmetic follows nccl-overlap/samples/multi-process-adam-scattered.cpp:402-449 statement by statement.
 #include "ccn_common.hpp"
 
 #include <cmath>
+#include <cstdlib>
 #include <new>
 #include <type_traits>
 #include <vector>
@@ -33,13 +38,14 @@ struct LambLayout {
   const LambTile* tiles;    // used when seg_len == 0
   uint64_t seg_len;         // common segment length, or 0 for a ragged layout
   float seg_len_f;
+  uint32_t tile;            // elements per full tile
 };
 
 __device__ __forceinline__ LambTile lamb_tile_of(const LambLayout& L, unsigned b) {
   if (L.seg_len != 0) {
     LambTile t;
-    t.start = (uint64_t)b * kLambTile;
-    t.count = kLambTile;
+    t.start = (uint64_t)b * L.tile;
+    t.count = L.tile;
     t.seg = (uint32_t)(t.start / L.seg_len);
     t.nf = L.seg_len_f;
     return t;
@@ -61,57 +67,69 @@ __device__ __forceinline__ float lamb_r(float mi, float vi, float w, const LambP
 }
 
 // One pack of VEC elements starting at element e0.
+// Everything pass 1 reads for one pack of VEC elements.
 template <int P, int VEC>
-__device__ __forceinline__ void lamb_pass1_pack(const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, int nP, const float* w,
-                                                float* m, float* v, size_t e0, float nf, const LambPrm& k, double& accW,
-                                                double& accR) {
-  const int np = P ? P : nP;
-  constexpr int PX = P > 0 ? P : 1;
-  Pack<float, VEC> gv[PX];
-  if constexpr (P > 0) {
+struct LambIn {
+  Pack<float, VEC> g[P > 0 ? P : CCN_MAX_RANKS];
+  Pack<float, VEC> w, m, v;
+};
+
+// Issues the pack's loads, all of them before anything waits (P = 0: the first nP of CCN_MAX_RANKS, wave-uniform).
+template <int P, int VEC>
+__device__ __forceinline__ void lamb_pass1_load(LambIn<P, VEC>& in, const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, int nP,
+                                                const float* w, const float* m, const float* v, size_t e0) {
+  constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
 #pragma unroll
-    for (int p = 0; p < P; p++) gv[p] = load_stream<float, VEC>(g.p[p] + e0);
+  for (int p = 0; p < PX; p++) {
+    if (P > 0 || p < nP) in.g[p] = load_stream<float, VEC>(g.p[p] + e0);
   }
-  const Pack<float, VEC> wv = load_stream<float, VEC>(w + e0);   // w is read again by pass 2, 12 GB later
-  Pack<float, VEC> mv = load_stream<float, VEC>(m + e0);
-  Pack<float, VEC> vv = load_stream<float, VEC>(v + e0);
-  Pack<float, VEC> gs;
-  if constexpr (P > 0) {
-#pragma unroll
-    for (int e = 0; e < VEC; e++) {
-      float a = gv[0].d[e];
-#pragma unroll
-      for (int p = 1; p < P; p++) a = a + gv[p].d[e];
-      gs.d[e] = a;
-    }
-  } else {
-    gs = load_stream<float, VEC>(g.p[0] + e0);
-    for (int p = 1; p < np; p++) {
-      const Pack<float, VEC> x = load_stream<float, VEC>(g.p[p] + e0);
-#pragma unroll
-      for (int e = 0; e < VEC; e++) gs.d[e] = gs.d[e] + x.d[e];
-    }
-  }
+  in.w = load_stream<float, VEC>(w + e0);   // w is read again by pass 2, 12 GB later
+  in.m = load_stream<float, VEC>(m + e0);
+  in.v = load_stream<float, VEC>(v + e0);
+}
+
+template <int P, int VEC>
+__device__ __forceinline__ void lamb_pass1_math(const LambIn<P, VEC>& in, int nP, float* m, float* v, size_t e0, float nf,
+                                                const LambPrm& k, double& accW, double& accR, Pack<float, VEC>& r_out,
+                                                Pack<float, VEC>& w_out) {
+  constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
+  Pack<float, VEC> mv, vv;
 #pragma unroll
   for (int e = 0; e < VEC; e++) {
-    const float ge = gs.d[e];
-    const float we = wv.d[e];
+    float ge = in.g[0].d[e];
+#pragma unroll
+    for (int p = 1; p < PX; p++) {
+      if (P > 0 || p < nP) ge = ge + in.g[p].d[e];
+    }
+    const float we = in.w.d[e];
     float mi, vi;
     if (k.mode == CCN_LAMB_NCCL_GLOBAL) {
-      vi = ((vv.d[e] * k.b2) + ((ge * ge) * k.omb2));
-      mi = ((mv.d[e] * k.b1) + (ge * k.omb1));
+      vi = ((in.v.d[e] * k.b2) + ((ge * ge) * k.omb2));
+      mi = ((in.m.d[e] * k.b1) + (ge * k.omb1));
     } else {
-      mi = k.b1 * mv.d[e] + k.omb1 * ge;
-      vi = k.b2 * vv.d[e] + k.omb2 * ge * ge;
+      mi = k.b1 * in.m.d[e] + k.omb1 * ge;
+      vi = k.b2 * in.v.d[e] + k.omb2 * ge * ge;
     }
     const float r = lamb_r(mi, vi, we, k);
     accR += k.mode == CCN_LAMB_NCCL_GLOBAL ? (double)(r * r) : (double)((r * r) / nf);
     accW += (double)(we * we);
     mv.d[e] = mi;
     vv.d[e] = vi;
+    r_out.d[e] = r;
+    w_out.d[e] = we;
   }
   store_stream<float, VEC>(m + e0, mv);
   store_stream<float, VEC>(v + e0, vv);
+}
+
+// One pack of VEC elements starting at element e0.
+template <int P, int VEC>
+__device__ __forceinline__ void lamb_pass1_pack(const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, int nP, const float* w,
+                                                float* m, float* v, size_t e0, float nf, const LambPrm& k, double& accW,
+                                                double& accR, Pack<float, VEC>& r_out, Pack<float, VEC>& w_out) {
+  LambIn<P, VEC> in;
+  lamb_pass1_load<P, VEC>(in, g, nP, w, m, v, e0);
+  lamb_pass1_math<P, VEC>(in, nP, m, v, e0, nf, k, accW, accR, r_out, w_out);
 }
 
 template <int P>
@@ -125,10 +143,12 @@ __global__ __launch_bounds__(kBlock) void lamb_pass1_kernel(const SrcTable<float
   const uint32_t j0 = threadIdx.x * 4;          // this thread's elements of the tile: [j0, j0+4) clipped to count
   if (j0 < t.count) {
     if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-      lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR);
+      Pack<float, 4> r4, w4;
+      lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
     } else {
       const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
-      for (uint32_t j = j0; j < j1; j++) lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j, t.nf, k, accW, accR);
+      Pack<float, 1> r1, w1;
+      for (uint32_t j = j0; j < j1; j++) lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j, t.nf, k, accW, accR, r1, w1);
     }
   }
   const double sW = block_sum(accW, lds);
@@ -139,8 +159,84 @@ __global__ __launch_bounds__(kBlock) void lamb_pass1_kernel(const SrcTable<float
   }
 }
 
-// One workgroup per segment.  Thread t adds tiles t, t+256, ... in ascending order, then the fixed
-// shuffle/LDS tree: the result does not depend on scheduling.
+// ---- communication between workgroups of one launch ---------------------------------------------------------------------
+// Device-scope release/acquire fences write back and invalidate the XCD's whole L2; with one per tile they serialise
+// the kernel (measured: 7 to 40 ms for a 2.8 ms step).  The few words that workgroups exchange therefore go through
+// relaxed device-scope atomics only, which are performed at the point where the XCDs' L2s are coherent and cost no
+// cache maintenance, and the order "data, then the word that announces it" is kept by waiting for the data's
+// acknowledgement (vmcnt = 0) before the announcing atomic is issued.
+__device__ __forceinline__ double peek_f64(const double* p) {
+  return __longlong_as_double((long long)__hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT));
+}
+// All vector-memory operations this wavefront has issued are acknowledged before anything after this is issued.
+__device__ __forceinline__ void drain_vector_memory() {
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0); expcnt and lgkmcnt left at their maxima
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
+// Sum of `x` over a BS-thread workgroup (BS = 64: one wavefront, no LDS); result valid in thread 0.
+// lds must hold BS / kWave doubles.
+template <int BS>
+__device__ __forceinline__ double group_sum(double x, double* lds) {
+  static_assert(BS % kWave == 0 && BS <= kBlock, "whole wavefronts, at most kBlock threads");
+  x = wave_sum(x);
+  if constexpr (BS == kWave) {
+    return x;
+  } else {
+    const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+    if (lane == 0) lds[wv] = x;
+    __syncthreads();
+    double r = 0.0;
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int i = 0; i < BS / kWave; i++) r += lds[i];
+    }
+    __syncthreads();
+    return r;
+  }
+}
+
+// Norms and scale of segment b from its tiles' partial sums [lo, hi).  Thread t adds tiles lo+t, lo+t+BS, ... in
+// ascending order, then the fixed shuffle/LDS tree: the result does not depend on scheduling.
+// SHARED: the partial sums were published by other workgroups of this launch.
+// Returns the scale (valid in thread 0).
+template <int BS, bool SHARED>
+__device__ __forceinline__ float lamb_finalize_segment(const double* partials, uint32_t lo, uint32_t hi, uint64_t seg_len,
+                                                      int b, double* norms, float* scale, int mode, double* lds) {
+  double aW = 0.0, aR = 0.0;
+  for (uint32_t t = lo + threadIdx.x; t < hi; t += BS) {
+    if constexpr (SHARED) {
+      aW += peek_f64(partials + 2 * (size_t)t);
+      aR += peek_f64(partials + 2 * (size_t)t + 1);
+    } else {
+      aW += partials[2 * (size_t)t];
+      aR += partials[2 * (size_t)t + 1];
+    }
+  }
+  const double sW = group_sum<BS>(aW, lds);
+  const double sR = group_sum<BS>(aR, lds + kBlock / kWave);
+  float sc = 0.0f;
+  if (threadIdx.x == 0 && mode == CCN_LAMB_NCCL_GLOBAL) {
+    const float wNorm = sqrtf((float)sW), rNorm = sqrtf((float)sR);
+    norms[2 * b] = wNorm;
+    norms[2 * b + 1] = rNorm;
+    sc = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f) / rNorm;
+    scale[b] = sc;
+  } else if (threadIdx.x == 0) {
+    const double rNorm = sqrt(sR);
+    const double wNorm = sqrt(sW / (double)seg_len);
+    const double ratio = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f);
+    norms[2 * b] = wNorm;
+    norms[2 * b + 1] = rNorm;
+    sc = (float)(mode == CCN_LAMB_REFERENCE ? ratio / rNorm : ratio);
+    scale[b] = sc;
+  }
+  return sc;
+}
+
+// One workgroup per segment that has tiles in this table.
 __global__ __launch_bounds__(kBlock) void lamb_finalize_kernel(const double* __restrict__ partials,
                                                                const uint32_t* __restrict__ seg_tile_begin,
                                                                const uint64_t* __restrict__ seg_len,
@@ -149,26 +245,8 @@ __global__ __launch_bounds__(kBlock) void lamb_finalize_kernel(const double* __r
   __shared__ double lds[2 * kBlock / kWave];
   const int b = blockIdx.x;
   const uint32_t lo = seg_tile_begin[b], hi = seg_tile_begin[b + 1];
-  double aW = 0.0, aR = 0.0;
-  for (uint32_t t = lo + threadIdx.x; t < hi; t += kBlock) {
-    aW += partials[2 * (size_t)t];
-    aR += partials[2 * (size_t)t + 1];
-  }
-  const double sW = block_sum(aW, lds);
-  const double sR = block_sum(aR, lds + kBlock / kWave);
-  if (threadIdx.x == 0 && mode == CCN_LAMB_NCCL_GLOBAL) {
-    const float wNorm = sqrtf((float)sW), rNorm = sqrtf((float)sR);
-    norms[2 * b] = wNorm;
-    norms[2 * b + 1] = rNorm;
-    scale[b] = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f) / rNorm;
-  } else if (threadIdx.x == 0) {
-    const double rNorm = sqrt(sR);
-    const double wNorm = sqrt(sW / (double)seg_len[b]);
-    const double ratio = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f);
-    norms[2 * b] = wNorm;
-    norms[2 * b + 1] = rNorm;
-    scale[b] = (float)(mode == CCN_LAMB_REFERENCE ? ratio / rNorm : ratio);
-  }
+  if (lo == hi) return;   // the segment is handled by the resident kernel
+  lamb_finalize_segment<kBlock, false>(partials, lo, hi, seg_len[b], b, norms, scale, mode, lds);
 }
 
 template <int VEC>
@@ -202,6 +280,256 @@ __global__ __launch_bounds__(kBlock) void lamb_pass2_kernel(float* w, const floa
   }
 }
 
+// ---- segment-resident variant ----------------------------------------------------------------------------------------
+// A persistent grid that is resident as a whole walks the tiles of the "resident" segments round-robin.  A workgroup
+// runs pass 1 on a tile, parks the tile's r and old w in LDS, and retires the tile one round later, when the
+// segment's scale is known: pass 2 then reads nothing from memory.  The workgroup that finishes a segment's last tile
+// computes its norms and scale and publishes them through a flag.  Every wait is bounded: a tile whose segment is not
+// ready within the spin limit goes onto a deferred list, and a trailing kernel finishes it from the stored m and v
+// (w is still the old one), so the result is the same whatever the scheduling and every workgroup exits.
+// A segment may hold at most kResDepth * gridDim.x tiles: with more, a workgroup's parking slots would fill up
+// with tiles of a segment whose other tiles it has yet to start.
+constexpr int kResDepth = 2;   // parking slots per workgroup
+constexpr int kResSub = 4;     // packs per thread per tile
+// Arrival counters.  Device-scope atomics on one address are served one after the other (some 15 ns each, measured),
+// so a segment's tiles count into kResFan counters, each on a cache line of its own, and the tile that completes one
+// of them counts into the segment's top counter.
+constexpr int kResFan = 8;
+constexpr int kResCntLine = 16;                              // uint32 per 64-byte line
+constexpr int kResCntStride = (kResFan + 1) * kResCntLine;   // uint32 per segment: top counter, then the fan
+
+struct LambResident {
+  uint32_t* cnt;                    // [nseg * kResCntStride] arrival counters (zero at kernel start)
+  unsigned long long* ready;        // [nseg] (1 << 32 | scale bits) once the segment's scale is known (zero at kernel start)
+  const uint32_t* seg_tile_begin;   // [nseg+1] resident-tile numbering
+  uint32_t* deferred;               // [ntiles]
+  uint32_t* ndeferred;              // zero at kernel start
+  uint32_t ntiles;
+  uint32_t spin_limit;
+};
+
+__global__ void lamb_reset_kernel(uint32_t* cnt, unsigned long long* ready, int nseg, uint32_t* ndeferred) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < nseg) {
+    ready[i] = 0;
+#pragma unroll
+    for (int f = 0; f <= kResFan; f++) cnt[(size_t)i * kResCntStride + f * kResCntLine] = 0;
+  }
+  if (i == 0) *ndeferred = 0;
+}
+
+template <int BS, int SUB>
+__device__ __forceinline__ void lamb_retire_tile(float* w, const LambTile& t, const Pack<float, 4>* park, float step_scale,
+                                                 int vec_ok) {
+#pragma unroll
+  for (int u = 0; u < SUB; u++) {
+    const uint32_t j0 = (u * BS + threadIdx.x) * 4;
+    if (j0 >= t.count) continue;
+    const Pack<float, 4> rv = park[(u * 2) * BS + threadIdx.x];
+    Pack<float, 4> wv = park[(u * 2 + 1) * BS + threadIdx.x];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float x = step_scale * rv.d[e];
+      wv.d[e] = wv.d[e] - x;
+    }
+    if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+      store_stream<float, 4>(w + t.start + j0, wv);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (j0 + e < t.count) w[t.start + j0 + e] = wv.d[e];
+      }
+    }
+  }
+}
+
+// BS threads per workgroup, SUB packs per thread per tile: a tile is BS * 4 * SUB elements.
+template <int P, int BS, int SUB>
+__global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float, (P ? P : CCN_MAX_RANKS)> g, const int nP,
+                                                           float* w, float* m, float* v, const LambLayout lay,
+                                                           double* partials, const uint64_t* __restrict__ seg_len,
+                                                           double* norms, float* scale, const LambResident rs,
+                                                           const int vec_ok, const LambPrm k) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int kSlotPacks = SUB * 2 * BS;
+  Pack<float, 4>* park = reinterpret_cast<Pack<float, 4>*>(smem);
+  double* red = reinterpret_cast<double*>(smem + (size_t)kResDepth * kSlotPacks * sizeof(Pack<float, 4>));
+  uint32_t* bc = reinterpret_cast<uint32_t*>(red + 2 * kBlock / kWave);   // [0] last tile of its segment, [1] ready, [2] scale
+  const unsigned G = gridDim.x;
+  const unsigned rounds = (rs.ntiles + G - 1) / G;
+  bool degraded = false;   // thread 0: a wait ran out before; later waits poll once
+  LambTile prev{};         // the tile parked in the previous round
+  bool have_prev = false;
+  // A whole, aligned tile takes the pipelined path: the loads of a pack are issued before the pack before it is
+  // worked on, and those of the next tile's first pack before this tile's sums and counters are dealt with, so that
+  // the workgroup has memory traffic in flight while it synchronises.
+  // (Not for 9..CCN_MAX_RANKS ranks: two packs of up to 19 loads each do not fit the registers of two wavefronts per SIMD.)
+  auto is_fast = [&](const LambTile& x) {
+    return P > 0 && vec_ok && (x.start & 3u) == 0 && x.count == (uint32_t)(BS * 4 * SUB);
+  };
+  LambTile next{};
+  LambIn<P, 4> pre;
+  if (blockIdx.x < rs.ntiles) {
+    next = lamb_tile_of(lay, blockIdx.x);
+    if (is_fast(next)) lamb_pass1_load<P, 4>(pre, g, nP, w, m, v, next.start + threadIdx.x * 4);
+  }
+  for (unsigned it = 0; it < rounds + (kResDepth - 1); it++) {
+    const unsigned tile = blockIdx.x + it * G;
+    const bool have_tile = it < rounds && tile < rs.ntiles;
+    // Thread 0 asks for the previous tile's scale now; the answer is looked at after this round's pass 1.
+    unsigned long long early = 0;
+    if (threadIdx.x == 0 && have_prev)
+      early = __hip_atomic_load(&rs.ready[prev.seg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    LambTile t{};
+    uint32_t arrived = 0, fan_target = 0, seg_tiles = 0;
+    if (have_tile) {
+      t = next;
+      Pack<float, 4>* slot = park + (size_t)(it % kResDepth) * kSlotPacks;
+      double accW = 0.0, accR = 0.0;
+      if (is_fast(t)) {
+        LambIn<P, 4> cur = pre;
+#pragma unroll
+        for (int u = 0; u < SUB; u++) {
+          const size_t e0 = t.start + (size_t)(u * BS + threadIdx.x) * 4;
+          LambIn<P, 4> nxt;
+          if (u + 1 < SUB) lamb_pass1_load<P, 4>(nxt, g, nP, w, m, v, e0 + BS * 4);
+          Pack<float, 4> r4, w4;
+          lamb_pass1_math<P, 4>(cur, nP, m, v, e0, t.nf, k, accW, accR, r4, w4);
+          slot[(u * 2) * BS + threadIdx.x] = r4;
+          slot[(u * 2 + 1) * BS + threadIdx.x] = w4;
+          if (u + 1 < SUB) cur = nxt;
+        }
+      } else
+#pragma unroll
+      for (int u = 0; u < SUB; u++) {
+        const uint32_t j0 = (u * BS + threadIdx.x) * 4;
+        Pack<float, 4> r4 = {}, w4 = {};
+        if (j0 < t.count) {
+          if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+            lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              if (j0 + e < t.count) {
+                Pack<float, 1> r1, w1;
+                lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
+                r4.d[e] = r1.d[0];
+                w4.d[e] = w1.d[0];
+              }
+            }
+          }
+        }
+        slot[(u * 2) * BS + threadIdx.x] = r4;
+        slot[(u * 2 + 1) * BS + threadIdx.x] = w4;
+      }
+      if (it + 1 < rounds && tile + G < rs.ntiles) {
+        next = lamb_tile_of(lay, tile + G);
+        if (is_fast(next)) lamb_pass1_load<P, 4>(pre, g, nP, w, m, v, next.start + threadIdx.x * 4);
+      }
+      const double sW = group_sum<BS>(accW, red);
+      const double sR = group_sum<BS>(accR, red + kBlock / kWave);
+      if (threadIdx.x == 0) {
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile,
+                           (unsigned long long)__double_as_longlong(sW), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile + 1,
+                           (unsigned long long)__double_as_longlong(sR), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        drain_vector_memory();   // the sums are in place before the count says so
+        const uint32_t seg_lo = rs.seg_tile_begin[t.seg];
+        seg_tiles = rs.seg_tile_begin[t.seg + 1] - seg_lo;
+        const uint32_t f = (tile - seg_lo) % kResFan;
+        fan_target = (seg_tiles - f + kResFan - 1) / kResFan;   // tiles of the segment that count into counter f
+        arrived = __hip_atomic_fetch_add(&rs.cnt[(size_t)t.seg * kResCntStride + (1 + f) * kResCntLine], 1u, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT) + 1;
+      }
+    }
+    // Previous tile, if its scale was already known at the top of the round: retire it while the count comes back.
+    bool retired = !have_prev;
+    if (have_prev) {
+      if (threadIdx.x == 0) {
+        bc[1] = (uint32_t)(early >> 32);
+        bc[2] = (uint32_t)early;
+      }
+      __syncthreads();
+      if (bc[1]) {
+        lamb_retire_tile<BS, SUB>(w, prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks, k.lr * __uint_as_float(bc[2]),
+                                  vec_ok);
+        retired = true;
+      }
+    }
+    // The workgroup that finishes a segment's last tile computes the segment's norms and scale.
+    if (have_tile) {
+      if (threadIdx.x == 0) {
+        uint32_t last = 0;
+        if (arrived == fan_target) {   // this tile completed its fan counter
+          const uint32_t fans = seg_tiles < (uint32_t)kResFan ? seg_tiles : (uint32_t)kResFan;
+          last = __hip_atomic_fetch_add(&rs.cnt[(size_t)t.seg * kResCntStride], 1u, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT) + 1 == fans;
+        }
+        bc[0] = last;
+      }
+      __syncthreads();
+      if (bc[0]) {
+        const float sc = lamb_finalize_segment<BS, true>(partials, rs.seg_tile_begin[t.seg], rs.seg_tile_begin[t.seg + 1],
+                                                         seg_len[t.seg], (int)t.seg, norms, scale, k.mode, red);
+        if (threadIdx.x == 0)
+          __hip_atomic_store(&rs.ready[t.seg], (1ull << 32) | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    // Previous tile, otherwise: wait for its scale, within the spin limit.  This comes after the finalize step above
+    // because the segment waited for may be the one this workgroup has just finished.
+    if (!retired) {
+      __syncthreads();   // bc[1], bc[2] were read above
+      if (threadIdx.x == 0) {
+        uint32_t budget = degraded ? 0u : rs.spin_limit;
+        unsigned long long word;
+        while (((word = __hip_atomic_load(&rs.ready[prev.seg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
+          if (budget == 0) break;
+          budget--;
+          __builtin_amdgcn_s_sleep(4);
+        }
+        if ((word >> 32) == 0) {
+          degraded = true;
+          const uint32_t at = __hip_atomic_fetch_add(rs.ndeferred, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          rs.deferred[at] = blockIdx.x + (it - 1) * G;
+        }
+        bc[1] = (uint32_t)(word >> 32);
+        bc[2] = (uint32_t)word;
+      }
+      __syncthreads();
+      if (bc[1])
+        lamb_retire_tile<BS, SUB>(w, prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks, k.lr * __uint_as_float(bc[2]),
+                                  vec_ok);
+    }
+    __syncthreads();   // bc and the retired slot are reused by the next round
+    prev = t;
+    have_prev = have_tile;
+  }
+}
+
+// Finishes the deferred tiles: pass 2 from the stored m and v, as the two-pass path does.
+template <int BS, int SUB>
+__global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, const float* m, const float* v, const LambLayout lay,
+                                                           const float* __restrict__ scale,
+                                                           const uint32_t* __restrict__ deferred,
+                                                           const uint32_t* __restrict__ ndeferred, const int vec_ok,
+                                                           const LambPrm k) {
+  const uint32_t n = *ndeferred;
+  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
+    const LambTile t = lamb_tile_of(lay, deferred[i]);
+    const float step_scale = k.lr * scale[t.seg];
+    for (int u = 0; u < SUB; u++) {
+      const uint32_t j0 = (u * BS + threadIdx.x) * 4;
+      if (j0 >= t.count) continue;
+      if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+        lamb_pass2_pack<4>(w, m, v, t.start + j0, step_scale, k);
+      } else {
+        const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
+        for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(w, m, v, t.start + j, step_scale, k);
+      }
+    }
+  }
+}
+
 }  // namespace ccn
 
 using namespace ccn;
@@ -210,22 +538,106 @@ struct ccn_lamb_plan {
   int device = -1;
   int nseg = 0;
   size_t N = 0;
+  // common per-segment state
+  uint64_t* seg_len = nullptr;
+  double* norms = nullptr;
+  float* scale = nullptr;
+  // two-pass part: tiles of kLambTile elements of the segments too long to stay on chip
   size_t ntiles = 0;
   uint64_t uniform_seg_len = 0;   // non-zero: all segments have this length and it is a multiple of the tile
   LambTile* tiles = nullptr;
   uint32_t* seg_tile_begin = nullptr;
-  uint64_t* seg_len = nullptr;
   double* partials = nullptr;
-  double* norms = nullptr;
-  float* scale = nullptr;
+  // resident part: tiles of res_block * 4 * res_sub elements of the other segments
+  int res_block = 0;              // 64 or kBlock
+  unsigned res_grid = 0, res_lds = 0;
+  uint32_t res_ntiles = 0;
+  uint64_t res_uniform_seg_len = 0;
+  uint32_t spin_limit = 0;
+  LambTile* rtiles = nullptr;
+  uint32_t* seg_rtile_begin = nullptr;
+  double* rpartials = nullptr;
+  int res_sub = 0;                // packs per thread per tile
+  uint32_t* sync = nullptr;       // cnt[nseg], ndeferred
+  unsigned long long* ready = nullptr;
+  uint32_t* deferred = nullptr;
+  int occupancy[CCN_MAX_RANKS + 1] = {0};   // resident workgroups per CU by rank count, 0 = not asked yet
 };
+
+namespace {
+
+long env_long(const char* name, long dflt) {
+  const char* e = std::getenv(name);
+  if (!e || !*e) return dflt;
+  char* end = nullptr;
+  const long x = std::strtol(e, &end, 10);
+  return end && *end == 0 ? x : dflt;
+}
+
+// Calls body(integral_constant<BS>, integral_constant<SUB>) for a supported resident-kernel shape; false otherwise.
+template <class Body>
+bool with_resident_shape(int block, int sub, Body body) {
+  switch (block * 10 + sub) {
+#define CCN_SHAPE(B, S) case B * 10 + S: body(std::integral_constant<int, B>{}, std::integral_constant<int, S>{}); return true;
+    CCN_SHAPE(64, 4) CCN_SHAPE(256, 4)
+#undef CCN_SHAPE
+    default: return false;
+  }
+}
+
+// Calls body(integral_constant<P>) with the rank count as a compile-time constant (0 = 9..CCN_MAX_RANKS, looped).
+template <class Body>
+void with_rank_count(int P, Body body) {
+  switch (P) {
+#define CCN_CASE(K) case K: body(std::integral_constant<int, K>{}); break;
+    CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
+#undef CCN_CASE
+    default: body(std::integral_constant<int, 0>{}); break;
+  }
+}
+
+// Workgroups of the resident kernel for P ranks that one CU holds at once with `lds` bytes of LDS each (0 on error).
+int resident_occupancy(int P, int block, int sub, unsigned lds) {
+  int occ = 0;
+  with_rank_count(P, [&](auto ptag) {
+    with_resident_shape(block, sub, [&](auto bstag, auto subtag) {
+      auto* fn = lamb_resident_kernel<decltype(ptag)::value, decltype(bstag)::value, decltype(subtag)::value>;
+      if (lds > 64 * 1024 &&
+          hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+      }
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, block, lds) != hipSuccess) {
+        (void)hipGetLastError();
+        occ = 0;
+      }
+    });
+  });
+  return occ;
+}
+
+// Cuts segment b into tiles of `tile` elements appended to `out`.
+void cut_segment(std::vector<LambTile>& out, const size_t* seg_offsets, int b, uint64_t tile) {
+  const uint64_t n = seg_offsets[b + 1] - seg_offsets[b];
+  for (uint64_t off = 0; off < n; off += tile) {
+    LambTile t{};
+    t.start = seg_offsets[b] + off;
+    t.count = (uint32_t)((n - off) < tile ? (n - off) : tile);
+    t.seg = (uint32_t)b;
+    t.nf = (float)n;
+    out.push_back(t);
+  }
+}
+
+}  // namespace
 
 extern "C" {
 
 int ccn_lamb_plan_destroy(ccn_lamb_plan* plan) {
   if (!plan) return CCN_OK;
   int rc = CCN_OK;
-  void* bufs[] = {plan->tiles, plan->seg_tile_begin, plan->seg_len, plan->partials, plan->norms, plan->scale};
+  void* bufs[] = {plan->tiles,  plan->seg_tile_begin,  plan->seg_len,   plan->partials, plan->norms,   plan->scale,
+                  plan->rtiles, plan->seg_rtile_begin, plan->rpartials, plan->sync,     plan->deferred, plan->ready};
   for (void* b : bufs) {
     if (b && hipFree(b) != hipSuccess) rc = CCN_EHIP;
   }
@@ -244,27 +656,65 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
 
-  std::vector<LambTile> tiles;
-  std::vector<uint32_t> begin((size_t)nseg + 1);
+  // Shape of the resident kernel.  CCN_LAMB_RESIDENT=0 sends every segment down the two-pass path;
+  // CCN_LAMB_RES_BLOCK (64 | 256), CCN_LAMB_RES_WGS (workgroups per CU) and CCN_LAMB_SPIN are for tuning and tests.
+  const bool resident_wanted = env_long("CCN_LAMB_RESIDENT", 1) != 0;
+  int res_block = (int)env_long("CCN_LAMB_RES_BLOCK", kBlock);
+  if (res_block != kWave && res_block != kBlock) res_block = kBlock;
+  const int res_sub = kResSub;
+  int lds_limit = 0;
+  if (hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, di->device) != hipSuccess) lds_limit = 65536;
+  auto lds_need = [&](int bs) {
+    return (size_t)kResDepth * bs * 4 * res_sub * 8 + 2 * (kBlock / kWave) * sizeof(double) + 16;
+  };
+  if (lds_need(res_block) > (size_t)lds_limit) res_block = kWave;
+  const uint64_t res_tile = (uint64_t)res_block * 4 * res_sub;
+  const size_t res_need = lds_need(res_block);
+  long res_wgs = env_long("CCN_LAMB_RES_WGS", (long)(kLdsPerCu / res_need));
+  const long wgs_max = (long)(kLdsPerCu / res_need);
+  if (res_wgs < 1) res_wgs = 1;
+  if (res_wgs > wgs_max) res_wgs = wgs_max;
+  // Keep to even counts: with 3 workgroups of 52 KiB per CU the kernel ran into its spin limit (measured), as it
+  // does when part of the grid is not resident, although the occupancy query below reports 3; 2, 4, 6 and 8 are fine.
+  if (res_wgs > 1) res_wgs &= ~1L;
+  // LDS request that lets res_wgs workgroups, and no more where the device's limits allow, share a CU: the whole grid
+  // is then resident at once and evenly spread.  The runtime's occupancy figure has the last word (LDS is handed out
+  // in blocks): shrink the request until res_wgs fit, or settle for the workgroups that do.
+  unsigned res_lds = (unsigned)((kLdsPerCu / (size_t)res_wgs) & ~(size_t)1023);
+  if (res_lds > (unsigned)lds_limit) res_lds = (unsigned)lds_limit;
+  int occ = resident_occupancy(8, res_block, res_sub, res_lds);
+  while (occ > 0 && occ < res_wgs && res_lds >= res_need + 1024) {
+    res_lds -= 1024;
+    occ = resident_occupancy(8, res_block, res_sub, res_lds);
+  }
+  if (occ > 0 && occ < res_wgs) res_wgs = occ;
+  const bool resident_ok = occ > 0;
+  const unsigned res_grid_full = (unsigned)di->cu_count * (unsigned)res_wgs;
+  const uint64_t res_cap_tiles = (uint64_t)kResDepth * res_grid_full;
+
+  std::vector<LambTile> tiles, rtiles;
+  std::vector<uint32_t> begin((size_t)nseg + 1), rbegin((size_t)nseg + 1);
   std::vector<uint64_t> len((size_t)nseg);
+  bool all_two_pass = true, all_resident = true;
   for (int b = 0; b < nseg; b++) {
     begin[b] = (uint32_t)tiles.size();
+    rbegin[b] = (uint32_t)rtiles.size();
     const uint64_t n = seg_offsets[b + 1] - seg_offsets[b];
     len[b] = n;
-    for (uint64_t off = 0; off < n; off += kLambTile) {
-      LambTile t{};
-      t.start = seg_offsets[b] + off;
-      t.count = (uint32_t)((n - off) < (uint64_t)kLambTile ? (n - off) : (uint64_t)kLambTile);
-      t.seg = (uint32_t)b;
-      t.nf = (float)n;
-      tiles.push_back(t);
+    const bool resident = resident_wanted && resident_ok && (n + res_tile - 1) / res_tile <= res_cap_tiles;
+    if (resident) {
+      cut_segment(rtiles, seg_offsets, b, res_tile);
+      all_two_pass = false;
+    } else {
+      cut_segment(tiles, seg_offsets, b, kLambTile);
+      all_resident = false;
     }
-    if (tiles.size() > 0x7fffffffu) return CCN_ERANGE;
+    if (tiles.size() > 0x7fffffffu || rtiles.size() > 0x7fffffffu) return CCN_ERANGE;
   }
   begin[nseg] = (uint32_t)tiles.size();
+  rbegin[nseg] = (uint32_t)rtiles.size();
   uint64_t uniform = len[0];
   for (int b = 1; b < nseg; b++) if (len[b] != uniform) uniform = 0;
-  if (uniform % kLambTile) uniform = 0;
 
   ccn_lamb_plan* p = new (std::nothrow) ccn_lamb_plan();
   if (!p) return CCN_ENOMEM;
@@ -272,18 +722,36 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   p->nseg = nseg;
   p->N = seg_offsets[nseg];
   p->ntiles = tiles.size();
-  p->uniform_seg_len = uniform;
+  p->uniform_seg_len = (all_two_pass && uniform % kLambTile == 0) ? uniform : 0;
+  p->res_block = res_block;
+  p->res_sub = res_sub;
+  p->res_ntiles = (uint32_t)rtiles.size();
+  p->res_uniform_seg_len = (all_resident && uniform % res_tile == 0) ? uniform : 0;
+  p->res_grid = p->res_ntiles < res_grid_full ? p->res_ntiles : res_grid_full;
+  p->res_lds = res_lds;
+  p->spin_limit = (uint32_t)env_long("CCN_LAMB_SPIN", 1 << 15);
   hipError_t e = hipSuccess;
-  auto alloc = [&](void** ptr, size_t bytes) { if (e == hipSuccess) e = hipMalloc(ptr, bytes); };
+  auto alloc = [&](void** ptr, size_t bytes) { if (e == hipSuccess) e = hipMalloc(ptr, bytes ? bytes : 16); };
+  auto upload = [&](void* dst, const void* src, size_t bytes) {
+    if (e == hipSuccess && bytes) e = hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice);
+  };
   alloc((void**)&p->tiles, tiles.size() * sizeof(LambTile));
   alloc((void**)&p->seg_tile_begin, begin.size() * sizeof(uint32_t));
   alloc((void**)&p->seg_len, len.size() * sizeof(uint64_t));
   alloc((void**)&p->partials, 2 * tiles.size() * sizeof(double));
   alloc((void**)&p->norms, 2 * (size_t)nseg * sizeof(double));
   alloc((void**)&p->scale, (size_t)nseg * sizeof(float));
-  if (e == hipSuccess) e = hipMemcpy(p->tiles, tiles.data(), tiles.size() * sizeof(LambTile), hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemcpy(p->seg_tile_begin, begin.data(), begin.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
-  if (e == hipSuccess) e = hipMemcpy(p->seg_len, len.data(), len.size() * sizeof(uint64_t), hipMemcpyHostToDevice);
+  alloc((void**)&p->rtiles, rtiles.size() * sizeof(LambTile));
+  alloc((void**)&p->seg_rtile_begin, rbegin.size() * sizeof(uint32_t));
+  alloc((void**)&p->rpartials, 2 * rtiles.size() * sizeof(double));
+  alloc((void**)&p->sync, ((size_t)nseg * kResCntStride + 1) * sizeof(uint32_t));
+  alloc((void**)&p->ready, (size_t)nseg * sizeof(unsigned long long));
+  alloc((void**)&p->deferred, rtiles.size() * sizeof(uint32_t));
+  upload(p->tiles, tiles.data(), tiles.size() * sizeof(LambTile));
+  upload(p->seg_tile_begin, begin.data(), begin.size() * sizeof(uint32_t));
+  upload(p->seg_len, len.data(), len.size() * sizeof(uint64_t));
+  upload(p->rtiles, rtiles.data(), rtiles.size() * sizeof(LambTile));
+  upload(p->seg_rtile_begin, rbegin.data(), rbegin.size() * sizeof(uint32_t));
   if (e != hipSuccess) {
     ccn_lamb_plan_destroy(p);
     return hip_fail(e);
@@ -318,35 +786,85 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
   for (int p = 0; p < P; p++) al = al && aligned16(g[p]);
   const int vec_ok = al ? 1 : 0;
   hipStream_t s = as_stream(stream);
-  const dim3 grid((unsigned)plan->ntiles), block(kBlock);
-  LambLayout lay;
-  lay.tiles = plan->tiles;
-  lay.seg_len = vec_ok ? plan->uniform_seg_len : 0;
-  lay.seg_len_f = (float)plan->uniform_seg_len;
-  // Residency caps measured for config 4 (N = 2^28, P = 8): pass 1 is fastest at 4 workgroups per CU (its float64
-  // sums and the workgroup reduction need more wavefronts to hide than the plain Adam kernel), pass 2 uncapped.
-  const unsigned lds1 = stream_launch(1, 1, P >= 2 ? 4 : 0).lds_bytes;
-  const unsigned lds2 = 0;
-  auto pass1 = [&](auto ptag) {
+  const dim3 block(kBlock);
+
+  auto with_ranks = [&](auto body) { with_rank_count(P, body); };
+  auto table = [&](auto ptag) {
     constexpr int PP = decltype(ptag)::value;
     SrcTable<float, (PP ? PP : CCN_MAX_RANKS)> tbl;
     for (int p = 0; p < (PP ? PP : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < P ? p : 0];
-    hipLaunchKernelGGL((lamb_pass1_kernel<PP>), grid, block, lds1, s, tbl, P, (const float*)w, m, v, lay, plan->partials,
-                       vec_ok, k);
+    return tbl;
   };
-  switch (P) {
-#define CCN_CASE(K) case K: pass1(std::integral_constant<int, K>{}); break;
-    CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
-#undef CCN_CASE
-    default: pass1(std::integral_constant<int, 0>{}); break;
+
+  if (plan->res_ntiles) {
+    LambLayout lay;
+    lay.tiles = plan->rtiles;
+    lay.seg_len = plan->res_uniform_seg_len;
+    lay.seg_len_f = (float)plan->res_uniform_seg_len;
+    lay.tile = (uint32_t)(plan->res_block * 4 * plan->res_sub);
+    LambResident rs;
+    rs.cnt = plan->sync;
+    rs.ndeferred = plan->sync + (size_t)plan->nseg * kResCntStride;
+    rs.ready = plan->ready;
+    rs.seg_tile_begin = plan->seg_rtile_begin;
+    rs.deferred = plan->deferred;
+    rs.ntiles = plan->res_ntiles;
+    rs.spin_limit = plan->spin_limit;
+    hipLaunchKernelGGL(lamb_reset_kernel, dim3((unsigned)((plan->nseg + kBlock - 1) / kBlock)), block, 0, s, rs.cnt, rs.ready,
+                       plan->nseg, rs.ndeferred);
+    CCN_HIP(hipGetLastError());
+    // The wait in the kernel is bounded either way, but it only pays when the whole grid is resident.
+    if (plan->occupancy[P] == 0) plan->occupancy[P] = resident_occupancy(P, plan->res_block, plan->res_sub, plan->res_lds);
+    const int occ = plan->occupancy[P];
+    if (occ < 1) return CCN_EHIP;
+    const unsigned fit = (unsigned)occ * (unsigned)di->cu_count;
+    const unsigned rgrid = plan->res_grid < fit ? plan->res_grid : fit;
+    const unsigned dgrid = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
+    with_ranks([&](auto ptag) {
+      constexpr int PP = decltype(ptag)::value;
+      const auto tbl = table(ptag);
+      with_resident_shape(plan->res_block, plan->res_sub, [&](auto bstag, auto subtag) {
+        constexpr int BS = decltype(bstag)::value;
+        constexpr int SUB = decltype(subtag)::value;
+        hipLaunchKernelGGL((lamb_resident_kernel<PP, BS, SUB>), dim3(rgrid), dim3(BS), plan->res_lds, s, tbl, P, w, m, v, lay,
+                           plan->rpartials, (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
+      });
+    });
+    CCN_HIP(hipGetLastError());
+    with_resident_shape(plan->res_block, plan->res_sub, [&](auto bstag, auto subtag) {
+      constexpr int BS = decltype(bstag)::value;
+      constexpr int SUB = decltype(subtag)::value;
+      hipLaunchKernelGGL((lamb_deferred_kernel<BS, SUB>), dim3(dgrid), dim3(BS), 0, s, w, (const float*)m, (const float*)v,
+                         lay, (const float*)plan->scale, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
+                         vec_ok, k);
+    });
+    CCN_HIP(hipGetLastError());
   }
-  CCN_HIP(hipGetLastError());
-  hipLaunchKernelGGL(lamb_finalize_kernel, dim3((unsigned)plan->nseg), block, 0, s, (const double*)plan->partials,
-                     (const uint32_t*)plan->seg_tile_begin, (const uint64_t*)plan->seg_len, plan->norms, plan->scale, mode);
-  CCN_HIP(hipGetLastError());
-  hipLaunchKernelGGL(lamb_pass2_kernel, grid, block, lds2, s, w, (const float*)m, (const float*)v, lay,
-                     (const float*)plan->scale, vec_ok, k);
-  CCN_HIP(hipGetLastError());
+
+  if (plan->ntiles) {
+    const dim3 grid((unsigned)plan->ntiles);
+    LambLayout lay;
+    lay.tiles = plan->tiles;
+    lay.seg_len = vec_ok ? plan->uniform_seg_len : 0;
+    lay.seg_len_f = (float)plan->uniform_seg_len;
+    lay.tile = kLambTile;
+    // Residency caps measured for N = 2^28, P = 8: pass 1 is fastest at 4 workgroups per CU (its float64 sums and the
+    // workgroup reduction need more wavefronts to hide than the plain Adam kernel), pass 2 uncapped.
+    const unsigned lds1 = stream_launch(1, 1, P >= 2 ? 4 : 0).lds_bytes;
+    const unsigned lds2 = 0;
+    with_ranks([&](auto ptag) {
+      constexpr int PP = decltype(ptag)::value;
+      hipLaunchKernelGGL((lamb_pass1_kernel<PP>), grid, block, lds1, s, table(ptag), P, (const float*)w, m, v, lay,
+                         plan->partials, vec_ok, k);
+    });
+    CCN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(lamb_finalize_kernel, dim3((unsigned)plan->nseg), block, 0, s, (const double*)plan->partials,
+                       (const uint32_t*)plan->seg_tile_begin, (const uint64_t*)plan->seg_len, plan->norms, plan->scale, mode);
+    CCN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(lamb_pass2_kernel, grid, block, lds2, s, w, (const float*)m, (const float*)v, lay,
+                       (const float*)plan->scale, vec_ok, k);
+    CCN_HIP(hipGetLastError());
+  }
   return CCN_OK;
 }
 

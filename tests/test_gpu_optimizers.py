@@ -345,8 +345,29 @@ def _lamb_compare(ccn, g, w0, segs, lr, b1, b2, eps, wd_, steps, mode, what, m0=
     return ulp_diff_f32(gw, w)
 
 
+# How a plan runs its segments is fixed when the plan is created, from these variables: the segment-resident kernel
+# with 256-thread or single-wavefront workgroups, the same with a spin limit of zero (every tile whose segment is
+# not ready at the first poll goes through the deferred list), or the two-pass kernels only.
+LAMB_VARIANTS = {
+    "resident": {},
+    "resident-wave": {"CCN_LAMB_RES_BLOCK": "64"},
+    "deferred": {"CCN_LAMB_SPIN": "0"},
+    "deferred-wave": {"CCN_LAMB_SPIN": "0", "CCN_LAMB_RES_BLOCK": "64"},
+    "two-pass": {"CCN_LAMB_RESIDENT": "0"},
+}
+
+
+@pytest.fixture(params=list(LAMB_VARIANTS))
+def lamb_variant(request, monkeypatch):
+    for k in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS"):
+        monkeypatch.delenv(k, raising=False)
+    for k, val in LAMB_VARIANTS[request.param].items():
+        monkeypatch.setenv(k, val)
+    return request.param
+
+
 @pytest.mark.parametrize("mode", [0, 1])
-def test_lamb_ragged_segments(ccn, mode):
+def test_lamb_ragged_segments(ccn, mode, lamb_variant):
     P = 4
     segs = [0, 5, 1029, 1030, 4096, 10000, 10000 + 8192, 10000 + 3 * 8192 + 1, 70001]
     N = segs[-1]
@@ -356,7 +377,7 @@ def test_lamb_ragged_segments(ccn, mode):
     assert ulps <= 2
 
 
-def test_lamb_config4_reduced(ccn):
+def test_lamb_config4_reduced(ccn, lamb_variant):
     # BASELINE config 4 layout at reduced size: 16 segments of 2^16, P = 8, wd = 0.01, two-pass norm + update
     P, nseg, seglen = 8, 16, 1 << 16
     N = nseg * seglen
@@ -364,6 +385,39 @@ def test_lamb_config4_reduced(ccn):
     g = grads_f32(0, P, N, 1e-3)
     w0 = weights_f32(0, N, 0.05)
     _lamb_compare(ccn, g, w0, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 3, 0, "config 4 reduced")
+
+
+def test_lamb_unaligned_buffers(ccn, lamb_variant):
+    """Buffers that start 4 bytes past a 16-byte boundary take the element-wise path of every kernel."""
+    P, segs = 3, [0, 700, 4096 + 700, 4096 + 701, 30011]
+    N = segs[-1]
+    g = grads_f32(71, P, N, 1e-3)
+    w0 = weights_f32(71, N, 0.05)
+    gd = [dev(np.concatenate([[np.float32(0)], x]))[1:] for x in g]
+    wd = dev(np.concatenate([[np.float32(0)], w0]))[1:]
+    md, vd = torch.zeros(N + 1, device=DEV)[1:], torch.zeros(N + 1, device=DEV)[1:]
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    plan = ccn.LambPlan(segs)
+    for t in (1, 2):
+        plan.step(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+        orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+    plan.close()
+    assert_f32_parity(host(md), m, "unaligned m")
+    assert_f32_parity(host(vd), v, "unaligned v")
+    assert ulp_diff_f32(host(wd), w) <= 2
+
+
+def test_lamb_mixed_resident_and_two_pass(ccn, monkeypatch):
+    """One segment too long to stay on chip (one workgroup per CU: 2 * 256 tiles of 4096 elements at most) between
+    short ones: the long one takes the two-pass kernels, the others the resident kernel, in one call."""
+    monkeypatch.setenv("CCN_LAMB_RES_WGS", "1")
+    P = 2
+    segs = [0, 3000, 3000 + 2_500_000, 3000 + 2_500_000 + 8192, 3000 + 2_500_000 + 8192 + 100_001]
+    N = segs[-1]
+    g = grads_f32(72, P, N, 1e-3)
+    w0 = weights_f32(72, N, 0.05)
+    ulps = _lamb_compare(ccn, g, w0, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 2, 0, "mixed")
+    assert ulps <= 2
 
 
 def test_lamb_reference_fixture(ccn):
