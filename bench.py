@@ -147,23 +147,23 @@ def main():
         if wl == "adam_f32":
             per_param = (P + 3) * 4 + 3 * 4
             step = lambda t: capi.adam_f32(g, w, m, v, N, 1e-3, 0.9, 0.999, 1e-6, t, stream)
-            kernel = "fused_stream_kernel<AdamMath,8,4,1>"
+            kernel = "fused_stream_kernel<AdamMath, %d, 4, 1, 64>" % (P if P <= 8 else 0)
         elif wl == "sgd_f32":
             per_param = (P + 1) * 4 + 4
             step = lambda t: capi.sgd_f32(g, w, N, 0.01, stream)
-            kernel = "fused_stream_kernel<SgdMath>"
+            kernel = "fused_stream_kernel<SgdMath, %d, 4, 1, %d>" % (P if P <= 8 else 0, 256 if P + 2 <= 3 else 64)
         elif wl == "adam_f16g":
             w16 = bufs.from_tensor(torch.empty(N, dtype=torch.float16, device="cuda"))
             flag = torch.zeros(1, dtype=torch.int32, device="cuda")
             per_param = P * 2 + 12 + 12 + 2
             step = lambda t: capi.adam_f16g(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, t, 2.0 ** -16, flag, stream)
-            kernel = "fused_stream_kernel<Adam16Math,8,4,1>"
+            kernel = "fused_stream_kernel<Adam16Math, %d, 4, 1, 64>" % (P if P <= 8 else 0)
         else:
             nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
             plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
             per_param = (P + 3) * 4 + 3 * 4
             step = lambda t: plan.step(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, capi.LAMB_TRUST_RATIO, stream)
-            kernel = "lamb_pass1_kernel<8> + lamb_finalize_kernel + lamb_pass2_kernel"
+            kernel = "lamb_reset_kernel + lamb_resident_kernel<%d, 256, 4> + lamb_deferred_kernel<256, 4>" % (P if P <= 8 else 0)
         alg_bytes = float(per_param) * N
         units = N
         config = {"workload": f"{wl} fused reduce+update, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,

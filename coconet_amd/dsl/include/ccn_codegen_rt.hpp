@@ -16,6 +16,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 #include "coconet_hip.h"
@@ -101,13 +102,15 @@ __device__ __forceinline__ double wave_sum(double x) {
   for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, kWave);
   return x;
 }
-__device__ __forceinline__ double block_sum(double x, double* lds) {
+// Sum over a workgroup of BS threads (BS = kWave: one wavefront, no LDS); valid in thread 0.
+template <int BS = kBlock> __device__ __forceinline__ double block_sum(double x, double* lds) {
   x = wave_sum(x);
+  if constexpr (BS == kWave) return x;
   if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = x;
   __syncthreads();
   double r = 0.0;
   if (threadIdx.x == 0)
-    for (int k = 0; k < kBlock / kWave; k++) r += lds[k];
+    for (int k = 0; k < BS / kWave; k++) r += lds[k];
   __syncthreads();
   return r;
 }
@@ -132,12 +135,14 @@ template <class Body> struct KernelArgs {
   typename Body::Scalars s;
 };
 
-template <class Body, int P, int VEC>
-__global__ __launch_bounds__(kBlock) void fused_pointwise_kernel(const KernelArgs<Body> a) {
+// One pack of VEC elements per thread and no loop: a workgroup issues every load of its tile at once and leaves.
+// BS = kWave (single-wavefront workgroups) for kernels that walk many arrays, kBlock for copy-like ones.
+template <class Body, int P, int VEC, int BS>
+__global__ __launch_bounds__(BS) void fused_pointwise_kernel(const KernelArgs<Body> a) {
   constexpr int NINX = Body::NIN > 0 ? Body::NIN : 1;
   constexpr int NOUTX = Body::NOUT > 0 ? Body::NOUT : 1;
   constexpr int NACCX = Body::NACC > 0 ? Body::NACC : 1;
-  constexpr int PX = P > 0 ? P : 1;
+  constexpr int PX = P > 0 ? P : kMaxRanks;
   __shared__ double lds[kBlock / kWave];
   const size_t nvec = a.n / VEC;
   double acc[NACCX];
@@ -147,33 +152,29 @@ __global__ __launch_bounds__(kBlock) void fused_pointwise_kernel(const KernelArg
 #pragma unroll
   for (int k = 0; k < Body::NNORM; k++) nrm[k] = a.norms[k];
 
-  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (size_t)gridDim.x * kBlock) {
+  const size_t i = (size_t)blockIdx.x * BS + threadIdx.x;
+  if (i < nvec) {
     const size_t e0 = i * VEC;
     Vals<VEC> rv[PX];
     Vals<VEC> iv[NINX];
-    Vals<VEC> red;
-    if constexpr (Body::HAS_RED && P > 0) {
+    if constexpr (Body::HAS_RED) {   // P = 0: the first nranks of kMaxRanks, a wave-uniform choice
 #pragma unroll
-      for (int p = 0; p < P; p++) rv[p] = load_vals<VEC>(a.red[p] + e0);
+      for (int p = 0; p < PX; p++) {
+        if (P > 0 || p < a.nranks) rv[p] = load_vals<VEC>(a.red[p] + e0);
+      }
     }
 #pragma unroll
     for (int k = 0; k < Body::NIN; k++) iv[k] = load_vals<VEC>(a.in[k] + e0);
+    Vals<VEC> red;
     if constexpr (Body::HAS_RED) {
-      if constexpr (P > 0) {
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-          float s = rv[0].d[e];
+      for (int e = 0; e < VEC; e++) {
+        float s = rv[0].d[e];
 #pragma unroll
-          for (int p = 1; p < P; p++) s = s + rv[p].d[e];
-          red.d[e] = s;
+        for (int p = 1; p < PX; p++) {
+          if (P > 0 || p < a.nranks) s = s + rv[p].d[e];
         }
-      } else {
-        red = load_vals<VEC>(a.red[0] + e0);
-        for (int p = 1; p < a.nranks; p++) {
-          const Vals<VEC> x = load_vals<VEC>(a.red[p] + e0);
-#pragma unroll
-          for (int e = 0; e < VEC; e++) red.d[e] = red.d[e] + x.d[e];
-        }
+        red.d[e] = s;
       }
     }
     Vals<VEC> ov[NOUTX];
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(kBlock) void fused_pointwise_kernel(const KernelArg
   if constexpr (Body::NACC > 0) {
 #pragma unroll
     for (int k = 0; k < Body::NACC; k++) {
-      const double s = block_sum(acc[k], lds);
+      const double s = block_sum<BS>(acc[k], lds);
       if (threadIdx.x == 0) a.partials[(size_t)blockIdx.x * Body::NACC + k] = s;
     }
   }
@@ -229,52 +230,73 @@ __global__ __launch_bounds__(kBlock) void finalize_norms_kernel(const double* pa
 // ---- host side ------------------------------------------------------------------------------------------------------
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-// Resident workgroups per CU for a kernel that walks `streams` arrays (measured on MI355X: many-stream kernels
-// reach the most HBM bandwidth with few wavefronts in flight), as unused dynamic LDS.
-inline unsigned lds_cap_bytes(int streams) {
-  const int cap = streams >= 6 ? 2 : (streams >= 4 ? 4 : 0);
-  if (cap == 0) return 0;
-  unsigned lds = (160u * 1024u / (unsigned)cap) & ~1023u;
-  return lds > 64u * 1024u ? 64u * 1024u : lds;
+// Launch shape for a kernel that walks `streams` fp32 arrays in 16-byte packs, from measurements on MI355X at 2^28
+// elements: single-wavefront workgroups, and as many of them per CU as keeps (streams x wavefronts) near 100
+// (7 for a 14-array Adam kernel, 13 for a 6-array SGD kernel), the cap expressed as unused dynamic LDS; copy-like
+// kernels want 256-thread workgroups and all the occupancy they can get.  Scalar (unaligned) launches keep 256 threads.
+struct LaunchShape {
+  int block;
+  unsigned lds;
+};
+inline LaunchShape shape_for(int streams, int vec) {
+  LaunchShape sh{kBlock, 0};
+  if (vec == 1 || streams <= 3) return sh;
+  int waves = (98 + streams / 2) / streams;
+  waves = waves < 6 ? 6 : (waves > 13 ? 13 : waves);
+  sh.block = kWave;
+  sh.lds = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
+  return sh;
 }
 
-inline unsigned grid_for(size_t n, int vec) {
-  size_t need = DIVUP(n / vec > 0 ? n / vec : 1, (size_t)kBlock);
+inline unsigned grid_for(size_t n, int vec, int block) {
+  size_t need = DIVUP(n / vec > 0 ? n / vec : 1, (size_t)block);
   return (unsigned)(need < 0x7fffffffull ? need : 0x7fffffffull);
 }
 
-template <class Body, int VEC> void launch_vec(const KernelArgs<Body>& a, hipStream_t s) {
-  const unsigned grid = grid_for(a.n, VEC);
-  const int streams = (Body::HAS_RED ? a.nranks : 0) + Body::NIN + Body::NOUT;
-  const unsigned lds = lds_cap_bytes(streams);
+template <class Body> int streams_of(const KernelArgs<Body>& a) {
+  return (Body::HAS_RED ? a.nranks : 0) + Body::NIN + Body::NOUT;
+}
+
+template <class Body, int VEC> unsigned launch_vec(const KernelArgs<Body>& a, hipStream_t s) {
+  const LaunchShape sh = shape_for(streams_of(a), VEC);
+  const unsigned grid = grid_for(a.n, VEC, sh.block);
   const int P = Body::HAS_RED ? a.nranks : 1;
+  auto go = [&](auto ptag) {
+    constexpr int PP = decltype(ptag)::value;
+    if (sh.block == kWave)
+      hipLaunchKernelGGL((fused_pointwise_kernel<Body, PP, VEC, kWave>), dim3(grid), dim3(kWave), sh.lds, s, a);
+    else
+      hipLaunchKernelGGL((fused_pointwise_kernel<Body, PP, VEC, kBlock>), dim3(grid), dim3(kBlock), sh.lds, s, a);
+  };
   switch (P) {
-#define CCN_GEN_CASE(K) \
-  case K: hipLaunchKernelGGL((fused_pointwise_kernel<Body, K, VEC>), dim3(grid), dim3(kBlock), lds, s, a); break;
+#define CCN_GEN_CASE(K) case K: go(std::integral_constant<int, K>{}); break;
     CCN_GEN_CASE(1) CCN_GEN_CASE(2) CCN_GEN_CASE(3) CCN_GEN_CASE(4) CCN_GEN_CASE(5) CCN_GEN_CASE(6) CCN_GEN_CASE(7)
     CCN_GEN_CASE(8)
 #undef CCN_GEN_CASE
-    default: hipLaunchKernelGGL((fused_pointwise_kernel<Body, 0, VEC>), dim3(grid), dim3(kBlock), lds, s, a); break;
+    default: go(std::integral_constant<int, 0>{}); break;
   }
   HIPCHECK(hipGetLastError());
+  return grid;
 }
 
-// Number of workgroups launch() will use (the size of the partials array is NACC times this).
-inline unsigned blocks_for(size_t n) { return grid_for(n, 1); }
+// An upper bound on the workgroups launch() uses for n elements, whatever the shape (the partials array holds NACC
+// values per workgroup): scalar launches have 256 threads, vector launches at least 64 threads of 4 elements.
+inline unsigned blocks_for(size_t n) { return grid_for(n, 1, kBlock); }
 
-template <class Body> void launch(const KernelArgs<Body>& a, void* stream) {
-  if (a.n == 0) return;
+// Launches the kernel and returns the number of workgroups used: that many rows of NACC partial sums are written.
+template <class Body> unsigned launch(const KernelArgs<Body>& a, void* stream) {
+  if (a.n == 0) return 0;
   bool al = true;
   if (Body::HAS_RED)
     for (int p = 0; p < a.nranks; p++) al = al && aligned16(a.red[p]);
   for (int k = 0; k < Body::NIN; k++) al = al && aligned16(a.in[k]);
   for (int k = 0; k < Body::NOUT; k++) al = al && aligned16(a.out[k]);
-  if (al) launch_vec<Body, 4>(a, (hipStream_t)stream);
-  else launch_vec<Body, 1>(a, (hipStream_t)stream);
+  if (al) return launch_vec<Body, 4>(a, (hipStream_t)stream);
+  return launch_vec<Body, 1>(a, (hipStream_t)stream);
 }
 
-inline void finalize_norms(const double* partials, size_t n, bool vec, int nacc, float* norms, void* stream) {
-  const unsigned nblocks = grid_for(n, vec ? 4 : 1);
+// norms[k] = sqrt of the sum of the nblocks partial sums of accumulator k.
+inline void finalize_norms(const double* partials, unsigned nblocks, int nacc, float* norms, void* stream) {
   hipLaunchKernelGGL(finalize_norms_kernel, dim3(1), dim3(kBlock), 0, (hipStream_t)stream, partials, nblocks, nacc, norms);
   HIPCHECK(hipGetLastError());
 }

@@ -483,13 +483,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
       o << "  {\n" << fill_args(st.body, a, st.count) << "  ccn_gen::launch(" << a << ", stream);\n  }\n";
     } else {
       const std::string a = "args" + std::to_string(argNo++), b = "args" + std::to_string(argNo++);
-      o << "  {\n" << fill_args(st.body, a, st.count) << "  ccn_gen::launch(" << a << ", stream);\n";
-      o << "  bool vec__ = true;\n";
-      o << "  if (" << a << ".nranks > 0 && " << st.body.name << "::HAS_RED) for (int p_ = 0; p_ < comm_size; p_++) vec__ = vec__ && ccn_gen::aligned16("
-        << a << ".red[p_]);\n";
-      o << "  for (int k_ = 0; k_ < " << st.body.name << "::NIN; k_++) vec__ = vec__ && ccn_gen::aligned16(" << a << ".in[k_]);\n";
-      o << "  for (int k_ = 0; k_ < " << st.body.name << "::NOUT; k_++) vec__ = vec__ && ccn_gen::aligned16(" << a << ".out[k_]);\n";
-      o << "  ccn_gen::finalize_norms(partials__, " << st.count << ", vec__, " << st.body.nacc << ", norms__, stream);\n";
+      o << "  {\n" << fill_args(st.body, a, st.count) << "  const unsigned blocks__ = ccn_gen::launch(" << a << ", stream);\n";
+      o << "  ccn_gen::finalize_norms(partials__, blocks__, " << st.body.nacc << ", norms__, stream);\n";
       o << fill_args(st.body2, b, st.count) << "  ccn_gen::launch(" << b << ", stream);\n  }\n";
     }
     o << "  CCNCHECK(ccn_event_record(stop__, stream));\n";
