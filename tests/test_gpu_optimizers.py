@@ -99,6 +99,26 @@ def test_sgd_config1_full_size(ccn):
     assert all(orc.eqFloat(a, b) for a, b in zip(w[::997], got[::997]))
 
 
+def test_sgd_more_than_2_to_32_elements(ccn):
+    """Element indices that do not fit 32 bits (17 GB per buffer): slices at the start, across 2^32 and at the ragged
+    end go through the oracle bit for bit, the whole array through a torch expression at the 1e-6 bar."""
+    P, N = 2, (1 << 32) + 4099
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(99)
+    g = [torch.empty(N, device=DEV).normal_(0.0, 1e-2, generator=gen) for _ in range(P)]
+    w = torch.empty(N, device=DEV).uniform_(-0.1, 0.1, generator=gen)
+    windows = [(0, 8192), ((1 << 32) - 4096, (1 << 32) + 4099)]
+    keep = [(host(w[a:b]).copy(), [host(x[a:b]).copy() for x in g]) for a, b in windows]
+    want_all = w - (g[0] + g[1]) * 0.01
+    ccn.sgd_f32(g, w, N, 0.01)
+    torch.cuda.synchronize()
+    assert float((w - want_all).abs().max()) <= FP32_TOL * 0.2
+    del want_all
+    for (a, b), (w0, g0) in zip(windows, keep):
+        orc.sgd_f32(g0, w0, 0.01)
+        assert_f32_parity(host(w[a:b]), w0, f"elements {a}..{b}")
+
+
 def test_reduce_in_place_and_empty(ccn):
     P, N = 4, 5000
     g = grads_f32(13, P, N, 1e-2)
