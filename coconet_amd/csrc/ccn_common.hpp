@@ -164,21 +164,17 @@ __host__ __device__ __forceinline__ bool keep_from_word(uint32_t word, float p_d
 // (a few workgroups per CU; used by the small helper kernels).
 unsigned stream_grid(size_t units, size_t tile);
 
-// Geometry of the fused reduce+update kernels.  One workgroup per tile (the kernels keep a grid-stride loop only
-// for shards beyond 2^31 tiles) and a cap on resident wavefronts per CU, enforced by requesting dynamic LDS that
-// the kernel never touches.  HBM sustains the most bandwidth when the number of address streams times the
-// wavefronts in flight stays moderate.  Measured on MI355X for the 14-stream kernel (8 gradients, w/m/v in,
-// w/m/v out; N = 2^28): full occupancy 72-75% of peak; 8 wavefronts per CU as two 256-thread workgroups 82%;
-// 7 wavefronts per CU as single-wavefront workgroups 85%; 4 wavefronts 63-70%.  A 2-stream copy wants all the
-// occupancy it can get.
+// Geometry of the fused reduce+update kernels: one workgroup per tile, no loop, and a cap on the wavefronts resident
+// per CU, enforced by requesting dynamic LDS that the kernel never touches.  HBM sustains the most bandwidth when the
+// number of address streams times the wavefronts in flight stays moderate.  Measured on MI355X for the 14-stream
+// kernel (8 gradients, w/m/v in, w/m/v out; N = 2^28): full occupancy 72-75% of peak; 8 wavefronts per CU as two
+// 256-thread workgroups 82%; 7 wavefronts per CU as single-wavefront workgroups 85%; 4 wavefronts 63-70%.  A 2-stream
+// copy wants all the occupancy it can get.
 struct StreamShape { int block; unsigned lds_bytes; };
-struct StreamLaunch { unsigned grid; unsigned lds_bytes; };
-StreamLaunch stream_launch(size_t units, size_t tile, int blocks_per_cu);
-// Shape for a kernel that reads and writes `streams` arrays with `pack_bytes` per thread and array.
-StreamShape stream_shape(int streams, int pack_bytes);
-
-// Workgroups of 256 threads per CU for the two-pass kernels that need a workgroup-wide reduction.
-inline int blocks_per_cu_for(int streams) { return streams >= 6 ? 2 : (streams >= 4 ? 4 : 0); }
+// Shape for a kernel whose threads each load `load_bytes` and store `store_bytes`, one pack per array.
+StreamShape stream_shape(int load_bytes, int store_bytes);
+// Dynamic LDS request that keeps at most `per_cu` workgroups on a CU (0 = no request).
+unsigned lds_for_residency(int per_cu);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -850,7 +850,7 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
     lay.tile = kLambTile;
     // Residency caps measured for N = 2^28, P = 8: pass 1 is fastest at 4 workgroups per CU (its float64 sums and the
     // workgroup reduction need more wavefronts to hide than the plain Adam kernel), pass 2 uncapped.
-    const unsigned lds1 = stream_launch(1, 1, P >= 2 ? 4 : 0).lds_bytes;
+    const unsigned lds1 = lds_for_residency(P >= 2 ? 4 : 0);
     const unsigned lds2 = 0;
     with_ranks([&](auto ptag) {
       constexpr int PP = decltype(ptag)::value;

@@ -56,57 +56,34 @@ unsigned stream_grid(size_t units, size_t tile) {
   const DeviceInfo* di = nullptr;
   int cus = 256;
   if (current_device_info(&di) == CCN_OK) cus = di->cu_count;
-  // Workgroups per CU for the grid-stride loop.  8 x 256 threads = one full CU of wavefronts.
-  static const int per_cu = [] {
-    const char* e = std::getenv("CCN_BLOCKS_PER_CU");
-    int v = e ? std::atoi(e) : 8;
-    return v > 0 ? v : 8;
-  }();
+  constexpr int per_cu = 8;   // 8 x 256 threads = one full CU of wavefronts
   size_t need = (units + tile - 1) / tile;
   size_t cap = (size_t)cus * (size_t)per_cu;
   if (need < 1) need = 1;
   return (unsigned)(need < cap ? need : cap);
 }
 
-StreamLaunch stream_launch(size_t units, size_t tile, int streams /* requested workgroups per CU, 0 = no cap */) {
-  // CCN_BLOCKS_PER_CU overrides the cap (0 = no cap); meant for tuning runs.
-  static const int forced = [] {
-    const char* e = std::getenv("CCN_BLOCKS_PER_CU");
-    return e ? std::atoi(e) : -1;
-  }();
-  int cap = forced;
-  if (cap < 0) cap = streams;   // the caller passes the cap it wants (see blocks_per_cu_for)
-  StreamLaunch L;
-  size_t need = (units + tile - 1) / tile;
-  if (need < 1) need = 1;
-  L.grid = (unsigned)(need < 0x7fffffffull ? need : 0x7fffffffull);
-  constexpr unsigned kLdsPerCu = 160 * 1024;
-  unsigned lds = 0;
-  if (cap >= 2 && cap <= 16) {
-    lds = (kLdsPerCu / (unsigned)cap) & ~1023u;
-    if (lds > 64 * 1024) lds = 64 * 1024;               // two per CU; larger requests need an opt-in attribute
-  }
-  L.lds_bytes = lds;
-  return L;
+unsigned lds_for_residency(int per_cu) {
+  if (per_cu < 2 || per_cu > 16) return 0;
+  const unsigned lds = (unsigned)(kLdsPerCu / (size_t)per_cu) & ~1023u;
+  return lds > 64 * 1024 ? 64 * 1024 : lds;   // two per CU; larger requests need an opt-in attribute
 }
 
-StreamShape stream_shape(int streams, int pack_bytes) {
+StreamShape stream_shape(int load_bytes, int store_bytes) {
   // CCN_BLOCK / CCN_LDS_KB override the shape; meant for tuning runs.
   static const int f_block = [] { const char* e = std::getenv("CCN_BLOCK"); return e ? std::atoi(e) : 0; }();
   static const int f_lds = [] { const char* e = std::getenv("CCN_LDS_KB"); return e ? std::atoi(e) : -1; }();
   StreamShape sh;
-  // Single-wavefront workgroups, and as many of them per CU as keeps (16-byte streams x wavefronts) near 100:
-  // measured optima on MI355X at N = 2^28 are 7 wavefronts per CU for the 14-stream fp32 Adam kernel (85% of HBM
-  // peak; 6 or 8 give 82-83%), 13 for the 6-stream SGD kernel (84%) and 12-13 for the fp16-gradient Adam kernel,
-  // whose 15 streams move 8-byte packs (80%).
-  const int eq_streams = (streams * pack_bytes + 15) / 16;
-  if (eq_streams <= 3) {
+  // Single-wavefront workgroups, and fewer of them per CU the more 16-byte loads each thread has in flight.
+  // Measured optima on MI355X at N = 2^28 (2^27 beyond 8 ranks), fp32 Adam unless said otherwise, as
+  // loads per thread -> wavefronts per CU (% of HBM peak): 4 -> 13+ (83), 5 -> 11-14 (84), 7 -> 12-13 (83; fp16-gradient
+  // Adam at 8 ranks: 81), 9 -> 8 (86; SGD at 8 ranks: 84), 11 -> 7 (85.5; 6 or 8 give 82-83), 15 -> 8 (82), 19 -> 6-10 (79).
+  const int loads = (load_bytes + 15) / 16;
+  if (loads + (store_bytes + 15) / 16 <= 3) {
     sh.block = 256;                 // copy-like kernels want all the occupancy they can get
     sh.lds_bytes = 0;
   } else {
-    int waves = (98 + eq_streams / 2) / eq_streams;
-    if (waves < 6) waves = 6;
-    if (waves > 13) waves = 13;
+    const int waves = loads <= 7 ? 13 : (loads <= 10 ? 8 : (loads <= 13 ? 7 : 8));
     sh.block = 64;
     sh.lds_bytes = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
   }

@@ -230,19 +230,18 @@ __global__ __launch_bounds__(kBlock) void finalize_norms_kernel(const double* pa
 // ---- host side ------------------------------------------------------------------------------------------------------
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-// Launch shape for a kernel that walks `streams` fp32 arrays in 16-byte packs, from measurements on MI355X at 2^28
-// elements: single-wavefront workgroups, and as many of them per CU as keeps (streams x wavefronts) near 100
-// (7 for a 14-array Adam kernel, 13 for a 6-array SGD kernel), the cap expressed as unused dynamic LDS; copy-like
-// kernels want 256-thread workgroups and all the occupancy they can get.  Scalar (unaligned) launches keep 256 threads.
+// Launch shape for a kernel whose threads load `loads` and store `stores` 16-byte packs, from measurements on MI355X
+// at 2^28 elements: single-wavefront workgroups, and fewer of them per CU the more loads a thread has in flight
+// (13 up to 7 loads, 8 up to 10, 7 up to 13, 8 beyond), the cap expressed as unused dynamic LDS; copy-like kernels
+// want 256-thread workgroups and all the occupancy they can get.  Scalar (unaligned) launches keep 256 threads.
 struct LaunchShape {
   int block;
   unsigned lds;
 };
-inline LaunchShape shape_for(int streams, int vec) {
+inline LaunchShape shape_for(int loads, int stores, int vec) {
   LaunchShape sh{kBlock, 0};
-  if (vec == 1 || streams <= 3) return sh;
-  int waves = (98 + streams / 2) / streams;
-  waves = waves < 6 ? 6 : (waves > 13 ? 13 : waves);
+  if (vec == 1 || loads + stores <= 3) return sh;
+  const int waves = loads <= 7 ? 13 : (loads <= 10 ? 8 : (loads <= 13 ? 7 : 8));
   sh.block = kWave;
   sh.lds = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
   return sh;
@@ -253,12 +252,8 @@ inline unsigned grid_for(size_t n, int vec, int block) {
   return (unsigned)(need < 0x7fffffffull ? need : 0x7fffffffull);
 }
 
-template <class Body> int streams_of(const KernelArgs<Body>& a) {
-  return (Body::HAS_RED ? a.nranks : 0) + Body::NIN + Body::NOUT;
-}
-
 template <class Body, int VEC> unsigned launch_vec(const KernelArgs<Body>& a, hipStream_t s) {
-  const LaunchShape sh = shape_for(streams_of(a), VEC);
+  const LaunchShape sh = shape_for((Body::HAS_RED ? a.nranks : 0) + Body::NIN, Body::NOUT, VEC);
   const unsigned grid = grid_for(a.n, VEC, sh.block);
   const int P = Body::HAS_RED ? a.nranks : 1;
   auto go = [&](auto ptag) {
