@@ -1,7 +1,7 @@
 // CoCoNet DSL front end, re-implemented for the MI355X target.
 //
 // Source-compatible with the user-visible API of the reference's src/dsl.hpp (namespace ACCCDSL:
-// Variable, Tensor, Stage, Update, Dropout, Sqrt, Norm, MatMul, Cast, Const, AllReduce, ReduceScatter,
+// Variable, Tensor, Stage, Update, Dropout, Sqrt, Ite, Norm, MatMul, Cast, Const, AllReduce, ReduceScatter,
 // AllGather, Scatter, Broadcast and the arithmetic operators), so that the reference's example programs
 // (examples/{sgd,adam,lamb,model-parallel}/*.cpp) compile unmodified.  Internally every expression is one
 // reference-counted Node of a small IR instead of a class hierarchy with visitors.
@@ -33,7 +33,7 @@ enum ReduceOperation { Summation, Difference, Multiplication, Division, Maximum,
 namespace ir {
 
 enum class Kind {
-  Tensor, Variable, Const, Binary, Unary, Cast, Update, Norm, Dropout, MatMul, Collective, Stage, Compare
+  Tensor, Variable, Const, Binary, Unary, Cast, Update, Norm, Dropout, MatMul, Collective, Stage, Compare, Select
 };
 enum class BinOp { Add, Sub, Mul, Div };
 enum class UnOp { Sqrt };
@@ -115,6 +115,9 @@ class Stage : public Expression {
 Expression Update(const Tensor& t, const Expression& definition);
 Expression Dropout(const Expression& x, float prob);
 Expression Sqrt(const Expression& x);
+// cond ? ifTrue : ifFalse per element (src/dsl.hpp:482-486 of the reference); cond is a comparison or any expression
+// that is non-zero where the first branch is wanted
+Expression Ite(const Expression& cond, const Expression& ifTrue, const Expression& ifFalse);
 Expression Norm(const Expression& x);
 Expression ReduceTensor(const Expression& x);
 Expression MatMul(const Expression& a, const Expression& b);

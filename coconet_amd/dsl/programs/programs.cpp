@@ -1,6 +1,6 @@
 // DSL programs for the BASELINE configurations, written against the CoCoNet API.
 //   ccn-programs <program> <schedule> [output.hip]
-// program: sgd | adam | lamb     schedule: unfused | fused
+// program: sgd | clipsgd | adam | lamb     schedule: unfused | fused
 #include <dsl.hpp>
 #include <pipeline.hpp>
 
@@ -18,6 +18,21 @@ static void sgd(bool fused, const std::string& out) {
   Stage wnew = Update(w, w - lr * gsum);
   Pipeline pl("sgd", {g, w, lr}, {wnew});
   if (fused) pl.fuse({gsum, wnew});
+  pl.codegen(out);
+}
+
+// SGD with the summed gradient clipped to [-clip, clip] element by element: exercises Ite and comparisons
+static void clipsgd(bool fused, const std::string& out) {
+  Variable N(Int32, "N");
+  Variable lr(Float32, "lr"), clip(Float32, "clip");
+  Tensor w(Float32, N, Replicated, "w");
+  Tensor g(Float32, N, Local, "g");
+  Stage gsum = AllReduce(Summation, g);
+  Stage gc = Ite(gsum > clip, clip, Ite((0 - clip) > gsum, 0 - clip, gsum));
+  Stage wnew = Update(w, w - lr * gc);
+  Pipeline pl("clipsgd", {g, w, lr, clip}, {wnew});
+  if (fused) pl.fuse({gsum, gc, wnew});
+  else pl.fuse({gc, wnew});
   pl.codegen(out);
 }
 
@@ -63,7 +78,7 @@ static void lamb(bool fused, const std::string& out) {
 
 int main(int argc, char** argv) {
   if (argc < 3) {
-    std::cout << "usage: " << argv[0] << " <sgd|adam|lamb> <unfused|fused> [output.hip]" << std::endl;
+    std::cout << "usage: " << argv[0] << " <sgd|clipsgd|adam|lamb> <unfused|fused> [output.hip]" << std::endl;
     return 1;
   }
   const std::string prog = argv[1], sched = argv[2];
@@ -71,6 +86,7 @@ int main(int argc, char** argv) {
   if (!fused && sched != "unfused") { std::cout << "Invalid schedule" << std::endl; return 1; }
   const std::string out = argc > 3 ? argv[3] : prog + "-" + sched + ".hip";
   if (prog == "sgd") sgd(fused, out);
+  else if (prog == "clipsgd") clipsgd(fused, out);
   else if (prog == "adam") adam(fused, out);
   else if (prog == "lamb") lamb(fused, out);
   else { std::cout << "Invalid program" << std::endl; return 1; }

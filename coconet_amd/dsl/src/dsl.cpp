@@ -22,6 +22,7 @@ bool is_scalar(const NodePtr& n) {
     case Kind::Unary:
     case Kind::Cast:
     case Kind::Compare:
+    case Kind::Select:
       for (auto& a : n->args) if (!is_scalar(a)) return false;
       return true;
     default: return false;
@@ -194,6 +195,16 @@ Expression Dropout(const Expression& x, float prob) {
 Expression Sqrt(const Expression& x) {
   auto n = unary_like(Kind::Unary, x);
   n->un = UnOp::Sqrt;
+  return Expression(n);
+}
+
+Expression Ite(const Expression& cond, const Expression& ifTrue, const Expression& ifFalse) {
+  // the value has the type and layout of "ifTrue op ifFalse"; the condition only has to be defined where they are
+  auto n = make(Kind::Select);
+  const NodePtr both = binary(BinOp::Add, ifTrue, ifFalse);
+  n->args = {cond.impl(), ifTrue.impl(), ifFalse.impl()};
+  n->elem = both->elem;
+  n->layout = is_scalar(both) ? cond.impl()->layout : both->layout;
   return Expression(n);
 }
 

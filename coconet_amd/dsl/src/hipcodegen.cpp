@@ -150,6 +150,13 @@ struct BodyBuilder {
         return "(" + a + " " + op[(int)n->bin] + " " + b + ")";
       }
       case Kind::Compare: return "((" + emit(n->args[0]) + " > " + emit(n->args[1]) + ") ? 1.0f : 0.0f)";
+      case Kind::Select: {   // the reference prints (cond ? a : b), src/codegen.cpp:660-666
+        const NodePtr& c = n->args[0];
+        const std::string cond = c->kind == Kind::Compare ? "(" + emit(c->args[0]) + " > " + emit(c->args[1]) + ")"
+                                                          : "(" + emit(c) + " != 0.0f)";
+        const std::string a = emit(n->args[1]), b = emit(n->args[2]);
+        return "(" + cond + " ? " + a + " : " + b + ")";
+      }
       case Kind::Unary: return "sqrtf(" + emit(n->args[0]) + ")";
       case Kind::Cast:
         if (n->elem == Float16) return "((float)(_Float16)(" + emit(n->args[0]) + "))";
@@ -519,6 +526,12 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
           return "(" + he(n->args[0]) + " " + op[(int)n->bin] + " " + he(n->args[1]) + ")";
         }
         case Kind::Compare: return "((" + he(n->args[0]) + " > " + he(n->args[1]) + ") ? 1.0f : 0.0f)";
+        case Kind::Select: {
+          const NodePtr& c = n->args[0];
+          const std::string cond = c->kind == Kind::Compare ? "(" + he(c->args[0]) + " > " + he(c->args[1]) + ")"
+                                                            : "(" + he(c) + " != 0.0f)";
+          return "(" + cond + " ? " + he(n->args[1]) + " : " + he(n->args[2]) + ")";
+        }
         case Kind::Unary: return "sqrtf(" + he(n->args[0]) + ")";
         case Kind::Cast: return n->elem == Float16 ? "((float)(_Float16)(" + he(n->args[0]) + "))" : he(n->args[0]);
         case Kind::Dropout: {

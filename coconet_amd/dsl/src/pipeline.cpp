@@ -177,6 +177,15 @@ static void print_expr(std::ostream& os, const NodePtr& n) {
       print_expr(os, n->args[1]);
       os << ")";
       break;
+    case Kind::Select:
+      os << "Ite(";
+      print_expr(os, n->args[0]);
+      os << ", ";
+      print_expr(os, n->args[1]);
+      os << ", ";
+      print_expr(os, n->args[2]);
+      os << ")";
+      break;
     case Kind::Unary: os << "Sqrt("; print_expr(os, n->args[0]); os << ")"; break;
     case Kind::Cast: os << "Cast<" << elem_c_type(n->elem) << ">("; print_expr(os, n->args[0]); os << ")"; break;
     case Kind::Update:

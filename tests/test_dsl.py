@@ -108,6 +108,18 @@ def test_emitted_expressions_keep_the_users_grouping(dsl_build, tmp_path):
     assert re.search(r'printf\("\{SZ: %ld, Epochs: %d, AllReduce: %f, kernel0: %f, Total: %f\}', t2)   # reference line format
 
 
+def test_ite_lowers_to_a_conditional_in_kernel_and_checker(dsl_build, tmp_path):
+    """Ite(cond, a, b) prints (cond ? a : b) as the reference's generator does (src/codegen.cpp:660-666), nested
+    selects included, in the device body and in the emitted CPU re-execution alike."""
+    exe = os.path.join(dsl_build, "ccn-programs")
+    out = tmp_path / "clipsgd.hip"
+    assert run(exe, "clipsgd", "fused", str(out)).returncode == 0
+    text = out.read_text()
+    assert "((v_S0 > s.clip) ? s.clip : (((0 - s.clip) > v_S0) ? (0 - s.clip) : v_S0))" in text
+    assert "((h.S0[i0] > clip) ? clip : (((0 - clip) > h.S0[i0]) ? (0 - clip) : h.S0[i0]))" in text
+    assert "HAS_RED = true" in text
+
+
 def test_two_pass_lowering_of_norms(dsl_build, tmp_path):
     exe = os.path.join(dsl_build, "ccn-programs")
     out = tmp_path / "lamb.hip"
