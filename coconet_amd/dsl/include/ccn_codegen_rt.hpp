@@ -216,6 +216,21 @@ __global__ __launch_bounds__(BS) void fused_pointwise_kernel(const KernelArgs<Bo
   }
 }
 
+// First level of the norm reduction for large launches: workgroup b adds rows [b*rows, (b+1)*rows) of the partial
+// sums, thread t taking rows t, t+256, ... in ascending order, into row b of `out`.  Fixed order: deterministic.
+__global__ __launch_bounds__(kBlock) void fold_partials_kernel(const double* partials, unsigned nblocks, unsigned rows, int nacc,
+                                                               double* out) {
+  __shared__ double lds[kBlock / kWave];
+  const size_t lo = (size_t)blockIdx.x * rows;
+  const size_t hi = lo + rows < nblocks ? lo + rows : nblocks;
+  for (int k = 0; k < nacc; k++) {
+    double s = 0.0;
+    for (size_t b = lo + threadIdx.x; b < hi; b += kBlock) s += partials[b * nacc + k];
+    const double t = block_sum(s, lds);
+    if (threadIdx.x == 0) out[(size_t)blockIdx.x * nacc + k] = t;
+  }
+}
+
 // norms[k] = sqrt(sum over workgroups of partials[b*nacc + k]); one workgroup, fixed order: deterministic.
 __global__ __launch_bounds__(kBlock) void finalize_norms_kernel(const double* partials, unsigned nblocks, int nacc, float* norms) {
   __shared__ double lds[kBlock / kWave];
@@ -232,8 +247,10 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // Launch shape for a kernel whose threads load `loads` and store `stores` 16-byte packs, from measurements on MI355X
 // at 2^28 elements: single-wavefront workgroups, and fewer of them per CU the more loads a thread has in flight
-// (13 up to 7 loads, 8 up to 10, 7 up to 13, 8 beyond), the cap expressed as unused dynamic LDS; copy-like kernels
-// want 256-thread workgroups and all the occupancy they can get.  Scalar (unaligned) launches keep 256 threads.
+// (13 up to 7 loads, 7 up to 10, 6 up to 13, 8 beyond: one fewer than the library's kernels of the same shape, whose
+// double-precision bias correction keeps a wavefront busy for longer), the cap expressed as unused dynamic LDS;
+// copy-like kernels want 256-thread workgroups and all the occupancy they can get.  Scalar (unaligned) launches keep
+// 256 threads.
 struct LaunchShape {
   int block;
   unsigned lds;
@@ -241,7 +258,7 @@ struct LaunchShape {
 inline LaunchShape shape_for(int loads, int stores, int vec) {
   LaunchShape sh{kBlock, 0};
   if (vec == 1 || loads + stores <= 3) return sh;
-  const int waves = loads <= 7 ? 13 : (loads <= 10 ? 8 : (loads <= 13 ? 7 : 8));
+  const int waves = loads <= 7 ? 13 : (loads <= 10 ? 7 : (loads <= 13 ? 6 : 8));
   sh.block = kWave;
   sh.lds = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
   return sh;
@@ -290,8 +307,25 @@ template <class Body> unsigned launch(const KernelArgs<Body>& a, void* stream) {
   return launch_vec<Body, 1>(a, (hipStream_t)stream);
 }
 
-// norms[k] = sqrt of the sum of the nblocks partial sums of accumulator k.
-inline void finalize_norms(const double* partials, unsigned nblocks, int nacc, float* norms, void* stream) {
+// Rows of the scratch area behind the partial sums that finalize_norms folds large launches into.
+constexpr unsigned kFoldRows = 8192;
+// Doubles to allocate for the partial sums of launches over up to n elements (8 accumulators at most).
+inline size_t partials_doubles(size_t n) { return ((size_t)blocks_for(n) + kFoldRows) * 8; }
+
+// norms[k] = sqrt of the sum of the nblocks partial sums of accumulator k.  A single workgroup would take 2 ms to read
+// the 2^20 rows of a 2^28-element launch, so beyond 4096 rows a first level folds them, 4096 or more rows per
+// workgroup, into the scratch rows at partials + blocks_for(n) * 8.
+inline void finalize_norms(const double* partials, double* scratch, unsigned nblocks, int nacc, float* norms, void* stream) {
+  if (nblocks > 4096) {
+    unsigned rows = (nblocks + kFoldRows - 1) / kFoldRows;
+    if (rows < 4096) rows = 4096;
+    const unsigned folded = (nblocks + rows - 1) / rows;
+    hipLaunchKernelGGL(fold_partials_kernel, dim3(folded), dim3(kBlock), 0, (hipStream_t)stream, partials, nblocks, rows, nacc,
+                       scratch);
+    HIPCHECK(hipGetLastError());
+    partials = scratch;
+    nblocks = folded;
+  }
   hipLaunchKernelGGL(finalize_norms_kernel, dim3(1), dim3(kBlock), 0, (hipStream_t)stream, partials, nblocks, nacc, norms);
   HIPCHECK(hipGetLastError());
 }

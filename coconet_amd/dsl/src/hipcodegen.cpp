@@ -425,7 +425,7 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   o << "// Generated by the coconet_amd HIP target from pipeline \"" << p.name() << "\".  Do not edit.\n";
   o << "// Build: hipcc --offload-arch=gfx950 -O3 -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops \\\n"
        "//        -I <repo>/include -I <repo>/coconet_amd/dsl/include <this file> -L <repo>/coconet_amd/lib -lcoconet_hip\n";
-  o << "// Run:   ./a.out <epochs> [ranks=4] [min_log2_size=10] [max_log2_size=29] [check=1]\n";
+  o << "// Run:   ./a.out <epochs> [ranks=4] [min_log2_size=10] [max_log2_size=29] [check=1] [untimed_warmup_epochs=0]\n";
   o << "#include \"ccn_codegen_rt.hpp\"\n\n";
   for (auto& st : steps) {
     if (st.type == Step::Kernel) o << body_text(st.body, prog.scalarVars);
@@ -491,7 +491,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
     } else {
       const std::string a = "args" + std::to_string(argNo++), b = "args" + std::to_string(argNo++);
       o << "  {\n" << fill_args(st.body, a, st.count) << "  const unsigned blocks__ = ccn_gen::launch(" << a << ", stream);\n";
-      o << "  ccn_gen::finalize_norms(partials__, blocks__, " << st.body.nacc << ", norms__, stream);\n";
+      o << "  ccn_gen::finalize_norms(partials__, partials__ + (size_t)ccn_gen::blocks_for(" << st.count << ") * 8, blocks__, "
+        << st.body.nacc << ", norms__, stream);\n";
       o << fill_args(st.body2, b, st.count) << "  ccn_gen::launch(" << b << ", stream);\n  }\n";
     }
     o << "  CCNCHECK(ccn_event_record(stop__, stream));\n";
@@ -587,6 +588,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   o << "  const int comm_size = argc > 2 ? atoi(argv[2]) : 4;\n";
   o << "  const int lo__ = argc > 3 ? atoi(argv[3]) : 10, hi__ = argc > 4 ? atoi(argv[4]) : 29;\n";
   o << "  const bool check__ = argc > 5 ? atoi(argv[5]) != 0 : true;\n";
+  // The reference times every epoch, the first (cold) one included; warm-up epochs are an addition, off by default.
+  o << "  const int warmup__ = argc > 6 && atoi(argv[6]) > 0 ? atoi(argv[6]) : 0;\n";
   o << "  if (comm_size < 1 || comm_size > ccn_gen::kMaxRanks) { printf(\"ranks must be 1..%d\\n\", ccn_gen::kMaxRanks); return 1; }\n";
   o << "  CCNCHECK(ccn_init(0));\n  void* stream;\n  CCNCHECK(ccn_stream_create(&stream));\n  const uint64_t seed__ = 1234;\n  bool allOk__ = true;\n\n";
   // size loop: explicit bounds when given, otherwise powers of two for every dimension variable
@@ -639,7 +642,7 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   for (size_t k = 0; k < p.stages().size(); k++) allStages__.push_back((int)k);
   const std::string anyCount = count_expr(p.stages()[first_tensor_stage(p, allStages__)]);
   o << ind << "double* partials__;\n" << ind << "float* norms__;\n";
-  o << ind << "CCNCHECK(ccn_malloc((void**)&partials__, (size_t)ccn_gen::blocks_for(" << anyCount << ") * 8 * sizeof(double)));\n";
+  o << ind << "CCNCHECK(ccn_malloc((void**)&partials__, ccn_gen::partials_doubles(" << anyCount << ") * sizeof(double)));\n";
   o << ind << "CCNCHECK(ccn_malloc((void**)&norms__, 8 * sizeof(float)));\n";
   o << ind << "// Outputs\n";
   for (auto& st : steps) o << ind << "float elapsedTime" << st.label << " = 0;\n";
@@ -647,7 +650,10 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   o << ind << "if (check__) {\n";
   for (auto& t : prog.tensors) o << ind << "  h." << t->name << " = h_" << t->name << ";\n";
   o << ind << "}\n";
-  o << ind << "for (int iter = 0; iter < epochs; iter++) {\n";
+  o << ind << "for (int iter = -warmup__; iter < epochs; iter++) {\n";
+  o << ind << "  if (iter == 0) {";
+  for (auto& st : steps) o << " elapsedTime" << st.label << " = 0;";
+  o << " }\n";
   o << ind << "  " << fn << "(";
   {
     // call with the same argument order as the signature
@@ -667,7 +673,7 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
     o << q.str();
   }
   o << ");\n";
-  o << ind << "  if (check__ && iter == 0) {\n";
+  o << ind << "  if (check__ && iter == -warmup__) {\n";
   o << ind << "    CCNCHECK(ccn_stream_sync(stream));\n";
   o << ind << "    " << fn << "_cpu(h";
   for (auto& d : prog.dimVars) o << ", " << d->name;

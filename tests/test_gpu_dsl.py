@@ -76,8 +76,15 @@ def test_model_parallel_program():
 
 
 def test_fusion_pays_off_at_config2_size():
-    """The point of CoCoNet's fusion, measured: at N = 2^28, P = 8 the fused schedule must beat
-    all-reduce-then-update by a clear margin (one pass over the gradients instead of two)."""
-    fused = run_program("adam-fused", 5, 8, 28, 28, 0)[0][2]["Total"]
-    unfused = run_program("adam-unfused", 5, 8, 28, 28, 0)[0][2]["Total"]
-    assert fused < 0.85 * unfused, (fused, unfused)
+    """The point of CoCoNet's fusion on one GPU, measured: at N = 2^28, P = 8 the fused schedule streams 56 bytes per
+    element, all-reduce-then-update 64 (the summed gradient is written and read again), so once the first, cold epoch
+    is left out (sixth argument: untimed warm-up epochs) the fused program must be faster by a clear margin."""
+    fused = run_program("adam-fused", 5, 8, 28, 28, 0, 1)[0][2]["Total"]
+    unfused = run_program("adam-unfused", 5, 8, 28, 28, 0, 1)[0][2]["Total"]
+    assert fused < 0.95 * unfused, (fused, unfused)
+
+
+def test_warmup_epochs_are_not_timed():
+    cold = run_program("sgd-fused", 2, 4, 24, 24, 1)[0]
+    warm = run_program("sgd-fused", 2, 4, 24, 24, 1, 2)[0]
+    assert cold[1] == warm[1] == 2 and warm[2]["Total"] <= cold[2]["Total"]
