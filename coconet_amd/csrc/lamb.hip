@@ -249,6 +249,27 @@ __global__ __launch_bounds__(kBlock) void lamb_finalize_kernel(const double* __r
   lamb_finalize_segment<kBlock, false>(partials, lo, hi, seg_len[b], b, norms, scale, mode, lds);
 }
 
+// First level for long segments: workgroup q adds the tile pairs [group_begin[q], group_begin[q+1]), all of one
+// segment, in the same fixed order as above, into pair q of `folded`; the finalize kernel then runs over those.
+constexpr uint32_t kLambFold = 4096;   // tiles per group
+__global__ __launch_bounds__(kBlock) void lamb_fold_kernel(const double* __restrict__ partials,
+                                                           const uint32_t* __restrict__ group_begin,
+                                                           double* __restrict__ folded) {
+  __shared__ double lds[2 * kBlock / kWave];
+  const uint32_t lo = group_begin[blockIdx.x], hi = group_begin[blockIdx.x + 1];
+  double aW = 0.0, aR = 0.0;
+  for (uint32_t t = lo + threadIdx.x; t < hi; t += kBlock) {
+    aW += partials[2 * (size_t)t];
+    aR += partials[2 * (size_t)t + 1];
+  }
+  const double sW = block_sum(aW, lds);
+  const double sR = block_sum(aR, lds + kBlock / kWave);
+  if (threadIdx.x == 0) {
+    folded[2 * (size_t)blockIdx.x] = sW;
+    folded[2 * (size_t)blockIdx.x + 1] = sR;
+  }
+}
+
 template <int VEC>
 __device__ __forceinline__ void lamb_pass2_pack(float* w, const float* m, const float* v, size_t e0, float step_scale,
                                                 const LambPrm& k) {
@@ -548,6 +569,10 @@ struct ccn_lamb_plan {
   LambTile* tiles = nullptr;
   uint32_t* seg_tile_begin = nullptr;
   double* partials = nullptr;
+  uint32_t ngroups = 0;                 // non-zero: some segment has more than kLambFold tiles, sums go through groups
+  uint32_t* group_begin = nullptr;      // [ngroups+1] tile index where each group starts
+  uint32_t* seg_group_begin = nullptr;  // [nseg+1]
+  double* folded = nullptr;             // [2*ngroups]
   // resident part: tiles of res_block * 4 * res_sub elements of the other segments
   int res_block = 0;              // 64 or kBlock
   unsigned res_grid = 0, res_lds = 0;
@@ -637,7 +662,8 @@ int ccn_lamb_plan_destroy(ccn_lamb_plan* plan) {
   if (!plan) return CCN_OK;
   int rc = CCN_OK;
   void* bufs[] = {plan->tiles,  plan->seg_tile_begin,  plan->seg_len,   plan->partials, plan->norms,   plan->scale,
-                  plan->rtiles, plan->seg_rtile_begin, plan->rpartials, plan->sync,     plan->deferred, plan->ready};
+                  plan->rtiles, plan->seg_rtile_begin, plan->rpartials, plan->sync,     plan->deferred, plan->ready,
+                  plan->group_begin, plan->seg_group_begin, plan->folded};
   for (void* b : bufs) {
     if (b && hipFree(b) != hipSuccess) rc = CCN_EHIP;
   }
@@ -716,6 +742,19 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   uint64_t uniform = len[0];
   for (int b = 1; b < nseg; b++) if (len[b] != uniform) uniform = 0;
 
+  // groups of at most kLambFold tiles for the two-pass segments, if any of them is longer than that
+  std::vector<uint32_t> group_begin, seg_group_begin;
+  bool need_groups = false;
+  for (int b = 0; b < nseg; b++) need_groups = need_groups || begin[b + 1] - begin[b] > kLambFold;
+  if (need_groups) {
+    for (int b = 0; b < nseg; b++) {
+      seg_group_begin.push_back((uint32_t)group_begin.size());
+      for (uint32_t t = begin[b]; t < begin[b + 1]; t += kLambFold) group_begin.push_back(t);
+    }
+    seg_group_begin.push_back((uint32_t)group_begin.size());
+    group_begin.push_back(begin[nseg]);
+  }
+
   ccn_lamb_plan* p = new (std::nothrow) ccn_lamb_plan();
   if (!p) return CCN_ENOMEM;
   p->device = di->device;
@@ -750,6 +789,14 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   upload(p->tiles, tiles.data(), tiles.size() * sizeof(LambTile));
   upload(p->seg_tile_begin, begin.data(), begin.size() * sizeof(uint32_t));
   upload(p->seg_len, len.data(), len.size() * sizeof(uint64_t));
+  if (need_groups) {
+    p->ngroups = (uint32_t)group_begin.size() - 1;
+    alloc((void**)&p->group_begin, group_begin.size() * sizeof(uint32_t));
+    alloc((void**)&p->seg_group_begin, seg_group_begin.size() * sizeof(uint32_t));
+    alloc((void**)&p->folded, 2 * (size_t)p->ngroups * sizeof(double));
+    upload(p->group_begin, group_begin.data(), group_begin.size() * sizeof(uint32_t));
+    upload(p->seg_group_begin, seg_group_begin.data(), seg_group_begin.size() * sizeof(uint32_t));
+  }
   upload(p->rtiles, rtiles.data(), rtiles.size() * sizeof(LambTile));
   upload(p->seg_rtile_begin, rbegin.data(), rbegin.size() * sizeof(uint32_t));
   if (e != hipSuccess) {
@@ -858,8 +905,17 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
                          plan->partials, vec_ok, k);
     });
     CCN_HIP(hipGetLastError());
-    hipLaunchKernelGGL(lamb_finalize_kernel, dim3((unsigned)plan->nseg), block, 0, s, (const double*)plan->partials,
-                       (const uint32_t*)plan->seg_tile_begin, (const uint64_t*)plan->seg_len, plan->norms, plan->scale, mode);
+    const double* sums = plan->partials;
+    const uint32_t* seg_begin = plan->seg_tile_begin;
+    if (plan->ngroups) {
+      hipLaunchKernelGGL(lamb_fold_kernel, dim3(plan->ngroups), block, 0, s, (const double*)plan->partials,
+                         (const uint32_t*)plan->group_begin, plan->folded);
+      CCN_HIP(hipGetLastError());
+      sums = plan->folded;
+      seg_begin = plan->seg_group_begin;
+    }
+    hipLaunchKernelGGL(lamb_finalize_kernel, dim3((unsigned)plan->nseg), block, 0, s, sums, seg_begin,
+                       (const uint64_t*)plan->seg_len, plan->norms, plan->scale, mode);
     CCN_HIP(hipGetLastError());
     hipLaunchKernelGGL(lamb_pass2_kernel, grid, block, lds2, s, w, (const float*)m, (const float*)v, lay,
                        (const float*)plan->scale, vec_ok, k);

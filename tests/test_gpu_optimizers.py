@@ -440,6 +440,18 @@ def test_lamb_mixed_resident_and_two_pass(ccn, monkeypatch):
     assert ulps <= 2
 
 
+def test_lamb_long_segment_two_level_sums(ccn):
+    """A segment of more than 4096 two-pass tiles (5 M elements: too long to stay on chip) has its tile sums folded in
+    groups before the finalize step; short segments on either side take the resident kernel in the same call."""
+    P = 2
+    segs = [0, 4097, 4097 + 5_000_001, 4097 + 5_000_001 + 70_000]
+    N = segs[-1]
+    g = grads_f32(73, P, N, 1e-3)
+    w0 = weights_f32(73, N, 0.05)
+    ulps = _lamb_compare(ccn, g, w0, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 2, 1, "long segment")
+    assert ulps <= 2
+
+
 def test_lamb_reference_fixture(ccn):
     """Reference harness for LAMB (multi-process-adam-scattered.cpp:464-698): integer pattern, beta = .5,
     alpha = 1, weight decay 1.0, reference scale; head and tail of its buffer-size list scaled to fit a test."""
