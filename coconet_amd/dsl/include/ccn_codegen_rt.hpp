@@ -231,14 +231,16 @@ __global__ __launch_bounds__(kBlock) void fold_partials_kernel(const double* par
   }
 }
 
-// norms[k] = sqrt(sum over workgroups of partials[b*nacc + k]); one workgroup, fixed order: deterministic.
-__global__ __launch_bounds__(kBlock) void finalize_norms_kernel(const double* partials, unsigned nblocks, int nacc, float* norms) {
+// norms[k] = the sum over workgroups of partials[b*nacc + k], or its square root where bit k of sqrt_mask is set;
+// one workgroup, fixed order: deterministic.
+__global__ __launch_bounds__(kBlock) void finalize_norms_kernel(const double* partials, unsigned nblocks, int nacc,
+                                                                unsigned sqrt_mask, float* norms) {
   __shared__ double lds[kBlock / kWave];
   for (int k = 0; k < nacc; k++) {
     double s = 0.0;
     for (unsigned b = threadIdx.x; b < nblocks; b += kBlock) s += partials[(size_t)b * nacc + k];
     const double t = block_sum(s, lds);
-    if (threadIdx.x == 0) norms[k] = (float)sqrt(t);
+    if (threadIdx.x == 0) norms[k] = (float)(((sqrt_mask >> k) & 1u) ? sqrt(t) : t);
   }
 }
 
@@ -312,10 +314,11 @@ constexpr unsigned kFoldRows = 8192;
 // Doubles to allocate for the partial sums of launches over up to n elements (8 accumulators at most).
 inline size_t partials_doubles(size_t n) { return ((size_t)blocks_for(n) + kFoldRows) * 8; }
 
-// norms[k] = sqrt of the sum of the nblocks partial sums of accumulator k.  A single workgroup would take 2 ms to read
+// norms[k] = the sum of the nblocks partial sums of accumulator k, or its square root.  A single workgroup would take 2 ms to read
 // the 2^20 rows of a 2^28-element launch, so beyond 4096 rows a first level folds them, 4096 or more rows per
 // workgroup, into the scratch rows at partials + blocks_for(n) * 8.
-inline void finalize_norms(const double* partials, double* scratch, unsigned nblocks, int nacc, float* norms, void* stream) {
+inline void finalize_norms(const double* partials, double* scratch, unsigned nblocks, int nacc, unsigned sqrt_mask,
+                           float* norms, void* stream) {
   if (nblocks > 4096) {
     unsigned rows = (nblocks + kFoldRows - 1) / kFoldRows;
     if (rows < 4096) rows = 4096;
@@ -326,7 +329,8 @@ inline void finalize_norms(const double* partials, double* scratch, unsigned nbl
     partials = scratch;
     nblocks = folded;
   }
-  hipLaunchKernelGGL(finalize_norms_kernel, dim3(1), dim3(kBlock), 0, (hipStream_t)stream, partials, nblocks, nacc, norms);
+  hipLaunchKernelGGL(finalize_norms_kernel, dim3(1), dim3(kBlock), 0, (hipStream_t)stream, partials, nblocks, nacc, sqrt_mask,
+                     norms);
   HIPCHECK(hipGetLastError());
 }
 

@@ -1,7 +1,7 @@
 // CoCoNet DSL front end, re-implemented for the MI355X target.
 //
 // Source-compatible with the user-visible API of the reference's src/dsl.hpp (namespace ACCCDSL:
-// Variable, Tensor, Stage, Update, Dropout, Sqrt, Ite, Norm, MatMul, Cast, Const, AllReduce, ReduceScatter,
+// Variable, Tensor, Stage, Update, Dropout, Sqrt, Ite, Norm, ReduceStage, MatMul, Cast, Const, AllReduce, ReduceScatter,
 // AllGather, Scatter, Broadcast and the arithmetic operators), so that the reference's example programs
 // (examples/{sgd,adam,lamb,model-parallel}/*.cpp) compile unmodified.  Internally every expression is one
 // reference-counted Node of a small IR instead of a class hierarchy with visitors.
@@ -57,6 +57,7 @@ struct Node {
   double cval = 0.0;               // Const
   bool cval_is_int = false;
   float prob = 0.f;                // Dropout
+  bool plain_sum = false;          // Norm nodes: the sum of the elements (ReduceStage) instead of the L2 norm
 };
 
 NodePtr make(Kind k);
@@ -119,7 +120,9 @@ Expression Sqrt(const Expression& x);
 // that is non-zero where the first branch is wanted
 Expression Ite(const Expression& cond, const Expression& ifTrue, const Expression& ifFalse);
 Expression Norm(const Expression& x);
-Expression ReduceTensor(const Expression& x);
+// Sum over all elements of a stage or tensor, a single replicated value (class ReduceStage of the reference,
+// src/dsl.hpp:269-275; its generated form is the S2 loop of examples/test-reduction.cu:17-19).  Summation only.
+Expression ReduceStage(const Expression& definition, ReduceOperation op);
 Expression MatMul(const Expression& a, const Expression& b);
 Expression Cast(TensorElemType t, const Expression& x);
 

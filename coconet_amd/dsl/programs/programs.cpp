@@ -1,6 +1,6 @@
 // DSL programs for the BASELINE configurations, written against the CoCoNet API.
 //   ccn-programs <program> <schedule> [output.hip]
-// program: sgd | clipsgd | adam | lamb     schedule: unfused | fused
+// program: sgd | clipsgd | reduction | adam | lamb     schedule: unfused | fused
 #include <dsl.hpp>
 #include <pipeline.hpp>
 
@@ -33,6 +33,23 @@ static void clipsgd(bool fused, const std::string& out) {
   Pipeline pl("clipsgd", {g, w, lr, clip}, {wnew});
   if (fused) pl.fuse({gsum, gc, wnew});
   else pl.fuse({gc, wnew});
+  pl.codegen(out);
+}
+
+// The pipeline behind the reference's examples/test-reduction.cu: a whole-tensor sum feeds the update.
+//   S0 = AllReduce(g); S1 = w + S0; S2 = sum(S1); w <- w - S2 * S0     (S2 scaled by `damp` to keep w finite over epochs)
+static void reduction(bool fused, const std::string& out) {
+  Variable N(Int32, "N");
+  Variable damp(Float32, "damp");
+  Tensor w(Float32, N, Replicated, "w");
+  Tensor g(Float32, N, Local, "g");
+  Stage s0 = AllReduce(Summation, g);
+  Stage s1 = w + s0;
+  Stage s2 = ReduceStage(s1, Summation);
+  Stage s3 = Update(w, w - (damp * s2) * s0);
+  Pipeline pl("reduction", {g, w, damp}, {s3});
+  if (fused) pl.fuse({s0, s1, s2, s3});
+  else pl.fuse({s1, s2, s3});
   pl.codegen(out);
 }
 
@@ -78,7 +95,7 @@ static void lamb(bool fused, const std::string& out) {
 
 int main(int argc, char** argv) {
   if (argc < 3) {
-    std::cout << "usage: " << argv[0] << " <sgd|clipsgd|adam|lamb> <unfused|fused> [output.hip]" << std::endl;
+    std::cout << "usage: " << argv[0] << " <sgd|clipsgd|reduction|adam|lamb> <unfused|fused> [output.hip]" << std::endl;
     return 1;
   }
   const std::string prog = argv[1], sched = argv[2];
@@ -87,6 +104,7 @@ int main(int argc, char** argv) {
   const std::string out = argc > 3 ? argv[3] : prog + "-" + sched + ".hip";
   if (prog == "sgd") sgd(fused, out);
   else if (prog == "clipsgd") clipsgd(fused, out);
+  else if (prog == "reduction") reduction(fused, out);
   else if (prog == "adam") adam(fused, out);
   else if (prog == "lamb") lamb(fused, out);
   else { std::cout << "Invalid program" << std::endl; return 1; }

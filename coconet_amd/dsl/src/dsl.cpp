@@ -214,7 +214,14 @@ Expression Norm(const Expression& x) {
   n->layout = Replicated;
   return Expression(n);
 }
-Expression ReduceTensor(const Expression& x) { return Norm(x); }
+Expression ReduceStage(const Expression& definition, ReduceOperation op) {
+  ASSERT(op == Summation, "ReduceStage: only Summation is lowered");
+  auto n = unary_like(Kind::Norm, definition);
+  n->layout = Replicated;
+  n->red = op;
+  n->plain_sum = true;
+  return Expression(n);
+}
 
 Expression MatMul(const Expression& a, const Expression& b) {
   auto n = make(Kind::MatMul);

@@ -107,6 +107,7 @@ struct Body {
   std::vector<std::string> outArrays;
   std::vector<std::string> code;         // statements
   int nacc = 0, nnorm = 0;
+  unsigned sqrtMask = 0;                 // accumulator k finishes as sqrt(sum) (a norm) rather than as the sum
   std::set<std::string> scalars;         // variable names used
   bool usesSeed = false;
 };
@@ -220,7 +221,12 @@ struct BodyBuilder {
       ASSERT(!phase2, "internal: norm accumulated in the second pass");
       const std::string x = emit(def->args[0]);
       const int slot = normIndex.count(k) ? normIndex[k] : (normIndex[k] = body.nacc++);
-      body.code.push_back("{ const float x_ = " + x + "; acc[" + std::to_string(slot) + "] += (double)(x_ * x_); }");
+      if (def->plain_sum) {
+        body.code.push_back("acc[" + std::to_string(slot) + "] += (double)(" + x + ");");
+      } else {
+        body.sqrtMask |= 1u << slot;
+        body.code.push_back("{ const float x_ = " + x + "; acc[" + std::to_string(slot) + "] += (double)(x_ * x_); }");
+      }
       return;
     }
     if (def->kind == Kind::Update) {
@@ -492,7 +498,7 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
       const std::string a = "args" + std::to_string(argNo++), b = "args" + std::to_string(argNo++);
       o << "  {\n" << fill_args(st.body, a, st.count) << "  const unsigned blocks__ = ccn_gen::launch(" << a << ", stream);\n";
       o << "  ccn_gen::finalize_norms(partials__, partials__ + (size_t)ccn_gen::blocks_for(" << st.count << ") * 8, blocks__, "
-        << st.body.nacc << ", norms__, stream);\n";
+        << st.body.nacc << ", " << st.body.sqrtMask << "u, norms__, stream);\n";
       o << fill_args(st.body2, b, st.count) << "  ccn_gen::launch(" << b << ", stream);\n  }\n";
     }
     o << "  CCNCHECK(ccn_event_record(stop__, stream));\n";
@@ -563,8 +569,13 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
         const NodePtr& x = def->args[0];
         ASSERT(x->kind == Kind::Stage || x->kind == Kind::Tensor, "Norm takes a stage or a tensor");
         o << "  { double a_ = 0.0; const size_t n_ = " << count_expr(x) << ";\n";
-        o << "    for (size_t i0 = 0; i0 < n_; i0++) { const float x_ = " << he(x) << "; a_ += (double)(x_ * x_); }\n";
-        o << "    h." << st->name << ".assign(1, (float)sqrt(a_)); }\n";
+        if (def->plain_sum) {
+          o << "    for (size_t i0 = 0; i0 < n_; i0++) a_ += (double)(" << he(x) << ");\n";
+          o << "    h." << st->name << ".assign(1, (float)a_); }\n";
+        } else {
+          o << "    for (size_t i0 = 0; i0 < n_; i0++) { const float x_ = " << he(x) << "; a_ += (double)(x_ * x_); }\n";
+          o << "    h." << st->name << ".assign(1, (float)sqrt(a_)); }\n";
+        }
         continue;
       }
       const std::string cnt = count_expr(st);

@@ -193,7 +193,7 @@ static void print_expr(std::ostream& os, const NodePtr& n) {
       print_expr(os, n->args[1]);
       os << ")";
       break;
-    case Kind::Norm: os << "Norm("; print_expr(os, n->args[0]); os << ")"; break;
+    case Kind::Norm: os << (n->plain_sum ? "ReduceStage(" : "Norm("); print_expr(os, n->args[0]); os << ")"; break;
     case Kind::Dropout: os << "Dropout("; print_expr(os, n->args[0]); os << ", " << n->prob << ")"; break;
     case Kind::MatMul:
       os << "MatMul(";

@@ -120,6 +120,21 @@ def test_ite_lowers_to_a_conditional_in_kernel_and_checker(dsl_build, tmp_path):
     assert "HAS_RED = true" in text
 
 
+def test_reduce_stage_is_a_plain_sum(dsl_build, tmp_path):
+    """ReduceStage(stage, Summation) (the S2 loop of the reference's examples/test-reduction.cu:17-19) accumulates the
+    values, not their squares, and finishes without a square root; it shares the two-pass lowering with Norm."""
+    exe = os.path.join(dsl_build, "ccn-programs")
+    out = tmp_path / "reduction.hip"
+    assert run(exe, "reduction", "fused", str(out)).returncode == 0
+    text = out.read_text()
+    assert "acc[0] += (double)(v_S1);" in text and "x_ * x_" not in text
+    assert re.search(r"finalize_norms\(partials__, [^;]*, 1, 0u, norms__, stream\)", text)       # one accumulator, no sqrt
+    assert "a_ += (double)(h.S1[i0])" in text.replace("(h.S1[i0])", "(h.S1[i0])") and "(float)a_" in text
+    lamb = tmp_path / "lamb.hip"
+    assert run(exe, "lamb", "fused", str(lamb)).returncode == 0
+    assert re.search(r"finalize_norms\(partials__, [^;]*, 2, 3u, norms__, stream\)", lamb.read_text())    # two norms, both sqrt
+
+
 def test_two_pass_lowering_of_norms(dsl_build, tmp_path):
     exe = os.path.join(dsl_build, "ccn-programs")
     out = tmp_path / "lamb.hip"
