@@ -36,6 +36,9 @@ def parse():
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph-steps", type=int, default=0,
+                    help="record this many steps once (ccn_graph_*) and time replays of the recording: for launch-bound "
+                         "sizes such as config 1; a recorded step keeps its step number")
     ap.add_argument("--allocator", default="ccn", choices=["ccn", "torch"],
                     help="ccn: buffers from ccn_malloc (channel-staggered); torch: plain torch allocations")
     return ap.parse_args()
@@ -139,7 +142,8 @@ def main():
     info = capi.device_info()
     K, W = a.steps, a.warmup
     wl = a.workload
-    stream = torch.cuda.current_stream().cuda_stream
+    own_stream = capi.Stream() if a.graph_steps > 0 else None      # the null stream cannot be recorded
+    stream = own_stream.h if own_stream else torch.cuda.current_stream().cuda_stream
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
 
@@ -212,6 +216,17 @@ def main():
         kernel = "torch copy"
         config = {"workload": f"device copy of 2^{int(np.log2(N))} fp32"}
 
+    if a.graph_steps > 0:
+        if wl in ("copy",):
+            sys.exit("--graph-steps records library calls only")
+        step(1)                                  # first call outside the recording (LAMB plans query occupancy once)
+        torch.cuda.synchronize()
+        with capi.Graph(own_stream) as graph:
+            for t in range(a.graph_steps):
+                step(2 + t)
+        eager_step, K = step, max(1, K // a.graph_steps)
+        step = lambda t: graph.launch()
+        config["graph_steps"] = a.graph_steps
     for t in range(1, W + 1):
         step(t)
     torch.cuda.synchronize()
@@ -223,6 +238,8 @@ def main():
     e1.record(stream)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    if a.graph_steps > 0:
+        K *= a.graph_steps                       # steps actually run
     wall_ms = (t1 - t0) * 1e3 / K
     ev_ms = e0.elapsed_ms(e1) / K
 

@@ -31,7 +31,7 @@ SYMBOLS = [
     "ccn_strerror", "ccn_reduce_f32", "ccn_sgd_f32", "ccn_sgd_axpby_f32", "ccn_pseudo_adam_f32", "ccn_adam_f32",
     "ccn_adam_f16g", "ccn_overflow_check_f16", "ccn_fused_adam_ref_f16g", "ccn_lamb_plan_create",
     "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
-    "ccn_bias_dropout_residual",
+    "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
 ]
 
 
@@ -98,6 +98,10 @@ def _declare(L):
     sig("ccn_lamb_plan_norms", [_vp, _vp, _vp])
     sig("ccn_mlp_outproj_bf16", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _vp])
     sig("ccn_bias_dropout_residual", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _vp])
+    sig("ccn_graph_begin", [_vp])
+    sig("ccn_graph_end", [_vp, _pp])
+    sig("ccn_graph_launch", [_vp, _vp])
+    sig("ccn_graph_destroy", [_vp])
 
 
 def strerror(code):
@@ -194,6 +198,50 @@ class Event:
                 load().ccn_event_destroy(self.h)
         except Exception:
             pass
+
+
+class Stream:
+    """A stream of the library's own (ccn_stream_create); pass `.h` wherever a stream is taken."""
+
+    def __init__(self):
+        h = C.c_void_p()
+        _check(load().ccn_stream_create(C.byref(h)), "ccn_stream_create")
+        self.h = h
+
+    def sync(self):
+        _check(load().ccn_stream_sync(self.h), "ccn_stream_sync")
+
+    def close(self):
+        if self.h:
+            _check(load().ccn_stream_destroy(self.h), "ccn_stream_destroy")
+            self.h = None
+
+
+class Graph:
+    """Records the update calls made on `stream` inside the with-block; launch() replays them."""
+
+    def __init__(self, stream):
+        self.stream, self.h = stream, None
+
+    def __enter__(self):
+        _check(load().ccn_graph_begin(self.stream.h), "ccn_graph_begin")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        h = C.c_void_p()
+        rc = load().ccn_graph_end(self.stream.h, C.byref(h))
+        if exc_type is None:
+            _check(rc, "ccn_graph_end")
+            self.h = h
+        return False
+
+    def launch(self, stream=None):
+        _check(load().ccn_graph_launch(self.h, (stream or self.stream).h), "ccn_graph_launch")
+
+    def close(self):
+        if self.h:
+            _check(load().ccn_graph_destroy(self.h), "ccn_graph_destroy")
+            self.h = None
 
 
 # ---- hot path --------------------------------------------------------------------------------------------------------

@@ -1,6 +1,8 @@
 // Runtime glue of libcoconet_hip: device set-up, memory, streams, events, error strings.
 #include "ccn_common.hpp"
 
+#include <new>
+
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -236,6 +238,56 @@ int ccn_event_elapsed_ms(void* start, void* stop, float* ms) {
   CCN_HIP(hipEventSynchronize((hipEvent_t)stop));
   CCN_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
   return CCN_OK;
+}
+
+struct ccn_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
+int ccn_graph_begin(void* stream) {
+  if (!stream) return CCN_EINVAL;   // the null stream cannot be captured
+  CCN_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+  return CCN_OK;
+}
+
+int ccn_graph_end(void* stream, ccn_graph** graph) {
+  if (!stream || !graph) return CCN_EINVAL;
+  *graph = nullptr;
+  hipGraph_t g = nullptr;
+  CCN_HIP(hipStreamEndCapture(as_stream(stream), &g));
+  if (!g) return CCN_EHIP;
+  hipGraphExec_t exec = nullptr;
+  const hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    return hip_fail(e);
+  }
+  ccn_graph* out = new (std::nothrow) ccn_graph();
+  if (!out) {
+    (void)hipGraphExecDestroy(exec);
+    (void)hipGraphDestroy(g);
+    return CCN_ENOMEM;
+  }
+  out->graph = g;
+  out->exec = exec;
+  *graph = out;
+  return CCN_OK;
+}
+
+int ccn_graph_launch(ccn_graph* graph, void* stream) {
+  if (!graph || !graph->exec) return CCN_EINVAL;
+  CCN_HIP(hipGraphLaunch(graph->exec, as_stream(stream)));
+  return CCN_OK;
+}
+
+int ccn_graph_destroy(ccn_graph* graph) {
+  if (!graph) return CCN_OK;
+  int rc = CCN_OK;
+  if (graph->exec && hipGraphExecDestroy(graph->exec) != hipSuccess) rc = CCN_EHIP;
+  if (graph->graph && hipGraphDestroy(graph->graph) != hipSuccess) rc = CCN_EHIP;
+  delete graph;
+  return rc;
 }
 
 int ccn_last_hip_error(void) { return g_last_hip_error; }

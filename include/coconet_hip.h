@@ -65,6 +65,20 @@ int  ccn_event_elapsed_ms(void* start, void* stop, float* ms);        /* synchro
 int  ccn_last_hip_error(void);
 const char* ccn_strerror(int code);
 
+/* ---- replaying a recorded sequence of calls.  The generated main() launches every epoch's kernels from the host
+ *      (epoch loop, src/codegen.cpp:4690-4720); at small sizes (config 1: a 3 us kernel) the launches, not the kernels,
+ *      set the pace.  Between ccn_graph_begin and ccn_graph_end the update entry points called on `stream` (a stream from
+ *      ccn_stream_create, not the null stream) are recorded instead of run; ccn_graph_launch replays the recording.
+ *      Recorded calls keep the arguments they were made with (pointers, sizes, and `step`, which is evaluated on the
+ *      host: a recording of Adam or LAMB steps replays the same bias corrections).  Not recordable: ccn_malloc/free,
+ *      the memcpy and sync calls, ccn_lamb_plan_create/norms, and the first ccn_lamb_f32 call of a plan for a given
+ *      rank count (it queries occupancy; make one call before recording). ---- */
+typedef struct ccn_graph ccn_graph;
+int  ccn_graph_begin(void* stream);
+int  ccn_graph_end(void* stream, ccn_graph** graph);
+int  ccn_graph_launch(ccn_graph* graph, void* stream);
+int  ccn_graph_destroy(ccn_graph* graph);
+
 /* ---- plain P-way reduce: out[i] = sum_p g[p][i].
  *      Replaces the stock ncclAllReduce of the unfused schedules (src/codegen.cpp:4146-4189;
  *      device loop nccl/src/collectives/device/common_kernel.h:1310-1427 ReduceOrCopyMulti).

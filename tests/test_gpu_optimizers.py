@@ -529,3 +529,45 @@ def test_lamb_nccl_global_variant(ccn):
     assert rel_err(plan.norms(), norms) < 1e-6
     assert np.max(np.abs(host(wd).astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
     plan.close()
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+def test_recorded_steps_replay_like_eager_calls(ccn):
+    """ccn_graph_*: eight SGD steps and a mixed-precision Adam step recorded on a stream, replayed three times with
+    eager work and synchronisations of the program's own in between; every replay is checked against the oracle."""
+    P, N = 4, (1 << 20) + 3
+    g = grads_f32(81, P, N, 1e-2)
+    w0 = weights_f32(81, N, 0.1)
+    g16 = [orc.f32_to_f16(x * np.float32(64.0)) for x in grads_f32(82, P, N, 1e-2)]
+    g16[1][12345] = np.uint16(0x7c00)                       # one overflowing element
+    gd, wd = [dev(x) for x in g], dev(w0)
+    g16d = [dev_u16(x) for x in g16]
+    w2d, m2d, v2d = dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w16d = torch.zeros(N, dtype=torch.int16, device=DEV)
+    flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+    torch.cuda.synchronize()
+    stream = ccn.Stream()
+    with ccn.Graph(stream) as graph:
+        for _ in range(8):
+            ccn.sgd_f32(gd, wd, N, 0.01, stream.h)
+        ccn.adam_f16g(g16d, w2d, m2d, v2d, w16d, N, 1e-3, 0.9, 0.999, 1e-6, 1, 1.0 / 64.0, flag, stream.h)
+    assert np.array_equal(host(wd), w0)                     # recording runs nothing
+    w = w0.copy()
+    w2, m2, v2, w16 = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros(N, np.uint16)
+    scratch = torch.zeros(1 << 22, device=DEV)
+    for replay in range(3):
+        graph.launch()
+        stream.sync()
+        for _ in range(8):
+            orc.sgd_f32(g, w, 0.01)
+        want_flag = orc.adam_f16g(g16, w2, m2, v2, w16, 1e-3, 0.9, 0.999, 1e-6, 1, 1.0 / 64.0)
+        assert_f32_parity(host(wd), w, f"replay {replay}: sgd w")
+        assert_f32_parity(host(w2d), w2, f"replay {replay}: adam w")
+        assert_f32_parity(host(v2d), v2, f"replay {replay}: adam v")
+        assert np.array_equal(host_u16(w16d), w16) and int(flag.item()) == want_flag == 1
+        flag.zero_()                                        # the recorded call clears and sets it again
+        scratch.add_(1.0)                                   # eager work between replays
+        ccn.sgd_f32(gd, scratch[:N], N, 0.0)
+        torch.cuda.synchronize()
+    graph.close()
+    stream.close()
