@@ -571,3 +571,32 @@ def test_recorded_steps_replay_like_eager_calls(ccn):
         torch.cuda.synchronize()
     graph.close()
     stream.close()
+
+
+def test_recorded_lamb_step_replays(ccn):
+    """A LAMB step through the segment-resident kernel, recorded after one eager call and replayed twice."""
+    P, segs = 3, [0, 5000, 5000 + 40960, 5000 + 40960 + 12289]
+    N = segs[-1]
+    g = grads_f32(83, P, N, 1e-3)
+    w0 = weights_f32(83, N, 0.05)
+    gd, wd = [dev(x) for x in g], dev(w0)
+    md, vd = torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    plan = ccn.LambPlan(segs)
+    stream = ccn.Stream()
+    plan.step(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, 0, stream.h)
+    stream.sync()
+    orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, 0)
+    with ccn.Graph(stream) as graph:
+        plan.step(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, 0.01, 2, 0, stream.h)
+    for replay in range(2):
+        graph.launch()
+        stream.sync()
+        orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 2, 0)
+        assert_f32_parity(host(md), m, f"replay {replay}: m")
+        assert_f32_parity(host(vd), v, f"replay {replay}: v")
+        assert ulp_diff_f32(host(wd), w) <= 2
+        torch.cuda.synchronize()
+    graph.close()
+    plan.close()
+    stream.close()
