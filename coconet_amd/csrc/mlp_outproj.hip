@@ -66,6 +66,46 @@ __device__ __forceinline__ void epilogue_quad(f32x4 acc, const SrcTable<float, 8
   *reinterpret_cast<u32x2*>(out + idx) = o;
 }
 
+// The same epilogue in two steps, so that the loads of one quad can be in flight while the previous one is finished.
+template <int NP> struct EpiIn {
+  f32x4 pv[NP > 0 ? NP : 1];
+  u32x2 rv;
+};
+template <int NP>
+__device__ __forceinline__ void epilogue_load(EpiIn<NP>& in, const SrcTable<float, 8>& parts,
+                                              const uint16_t* __restrict__ resid, size_t idx) {
+#pragma unroll
+  for (int q = 0; q < NP; q++) in.pv[q] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts.p[q] + idx));
+  in.rv = u32x2{0u, 0u};
+  if (resid) in.rv = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(resid + idx));
+}
+template <int NP>
+__device__ __forceinline__ void epilogue_finish(f32x4 acc, const EpiIn<NP>& in, const float* __restrict__ bias,
+                                                uint16_t* __restrict__ out, size_t idx, size_t n, const EpiPrm& k) {
+  const f32x4 bv = *reinterpret_cast<const f32x4*>(bias + n);
+  f32x4 s = acc;
+#pragma unroll
+  for (int q = 0; q < NP; q++) s = s + in.pv[q];
+  const f32x4 t = s + bv;
+  f32x4 d = t;
+  if (k.apply_dropout) {
+    const uint64_t blk = (uint64_t)idx >> 2;
+    const Philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u, k.seed_lo, k.seed_hi);
+    d[0] = keep_from_word(r.x, k.p_drop) ? t[0] * k.keep_scale : 0.0f;
+    d[1] = keep_from_word(r.y, k.p_drop) ? t[1] * k.keep_scale : 0.0f;
+    d[2] = keep_from_word(r.z, k.p_drop) ? t[2] * k.keep_scale : 0.0f;
+    d[3] = keep_from_word(r.w, k.p_drop) ? t[3] * k.keep_scale : 0.0f;
+  }
+  const float y0 = d[0] + bf16_bits_to_f32((uint16_t)(in.rv[0] & 0xffffu));
+  const float y1 = d[1] + bf16_bits_to_f32((uint16_t)(in.rv[0] >> 16));
+  const float y2 = d[2] + bf16_bits_to_f32((uint16_t)(in.rv[1] & 0xffffu));
+  const float y3 = d[3] + bf16_bits_to_f32((uint16_t)(in.rv[1] >> 16));
+  u32x2 o;
+  o[0] = (uint32_t)f32_to_bf16_bits(y0) | ((uint32_t)f32_to_bf16_bits(y1) << 16);
+  o[1] = (uint32_t)f32_to_bf16_bits(y2) | ((uint32_t)f32_to_bf16_bits(y3) << 16);
+  __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(out + idx));
+}
+
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 7); }
 
 template <int NP>
@@ -195,12 +235,33 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
       }
     }
     __syncthreads();
+    constexpr int kIters = (BM / 2) * (BN / 4) / kBlock;
+    if constexpr (NP > 0) {
+      // the loads of quad it+1 are issued before quad it is finished
+      auto index_of = [&](int it) {
+        const int q = it * kBlock + t;
+        return (m0 + half * 64 + q / (BN / 4)) * (size_t)N + n0 + (q % (BN / 4)) * 4;
+      };
+      EpiIn<NP> cur;
+      epilogue_load<NP>(cur, parts, resid, index_of(0));
 #pragma unroll
-    for (int it = 0; it < (BM / 2) * (BN / 4) / kBlock; it++) {
-      const int q = it * kBlock + t;
-      const int row = q / (BN / 4), colq = q % (BN / 4);
-      const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
-      epilogue_quad<NP>(a, parts, nPartials, bias, resid, out, m0 + half * 64 + row, n0 + colq * 4, (size_t)N, ep);
+      for (int it = 0; it < kIters; it++) {
+        EpiIn<NP> nxt;
+        if (it + 1 < kIters) epilogue_load<NP>(nxt, parts, resid, index_of(it + 1));
+        const int q = it * kBlock + t;
+        const int row = q / (BN / 4), colq = q % (BN / 4);
+        const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
+        epilogue_finish<NP>(a, cur, bias, out, index_of(it), n0 + colq * 4, ep);
+        if (it + 1 < kIters) cur = nxt;
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < kIters; it++) {
+        const int q = it * kBlock + t;
+        const int row = q / (BN / 4), colq = q % (BN / 4);
+        const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
+        epilogue_quad<NP>(a, parts, nPartials, bias, resid, out, m0 + half * 64 + row, n0 + colq * 4, (size_t)N, ep);
+      }
     }
   }
 }
