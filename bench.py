@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload adam_f32]
 
 A "step" is one launch of the hot path over the whole shard with inputs resident in HBM.  The default
-workload is BASELINE config 2: fused reduce + bias-corrected Adam, fp32, N = 2^28 parameters, P = 8
+workload is benchmark configuration 2: fused reduce + bias-corrected Adam, fp32, N = 2^28 parameters, P = 8
 rank-gradient buffers.  One JSON line is printed: whole-job algorithmic GB/s (56 B/param for Adam), the
 roofline of the dominant kernel from HIP events recorded on the launch stream, and the CPU restatement of the
 reference checker loop timed on a bounded sample on this box's host cores.
@@ -158,7 +158,7 @@ def main():
             if gbytes == 2:
                 t = (torch.randn(N, device="cuda", generator=gen) * (1e-3 * 65536.0)).to(torch.float16)
                 if p == 0:
-                    t[::1 << 20] = float("inf")        # BASELINE config 3: one entry in 2^20 overflows
+                    t[::1 << 20] = float("inf")        # benchmark configuration 3: one entry in 2^20 overflows
             else:
                 t = torch.empty(N, device="cuda").normal_(0.0, 1e-3 if wl != "sgd_f32" else 1e-2, generator=gen)
             g.append(bufs.from_tensor(t))

@@ -1,4 +1,4 @@
-// DSL programs for the BASELINE configurations, written against the CoCoNet API.
+// DSL programs for the benchmark configurations, written against the CoCoNet API.
 //   ccn-programs <program> <schedule> [output.hip]
 // program: sgd | clipsgd | reduction | adam | lamb     schedule: unfused | fused
 #include <dsl.hpp>
@@ -8,7 +8,7 @@
 
 using namespace ACCCDSL;
 
-// w <- w - lr * sum_p g_p   (BASELINE config 1)
+// w <- w - lr * sum_p g_p   (benchmark configuration 1)
 static void sgd(bool fused, const std::string& out) {
   Variable N(Int32, "N");
   Variable lr(Float32, "lr");
@@ -53,7 +53,7 @@ static void reduction(bool fused, const std::string& out) {
   pl.codegen(out);
 }
 
-// bias-corrected Adam (BASELINE config 2).  The DSL has no pow(), so the caller passes the two bias
+// bias-corrected Adam (benchmark configuration 2).  The DSL has no pow(), so the caller passes the two bias
 // corrections 1-beta^t as scalars; eps as well.
 static void adam(bool fused, const std::string& out) {
   Variable N(Int32, "N");

@@ -170,7 +170,7 @@ void orc_fused_adam_a3(const uint16_t* const* g, int P, float* w, float* m, floa
  *   v_ = v/(1 - pow(beta2, epoch+1))
  *   x  = stepsize * m_ / (sqrt(v_) + epsilon)            -- (stepsize*m_) / (sqrtf(v_)+eps), fp32
  *   w  = w + x
- * The reference passes stepsize = +alpha; BASELINE's "w -= lr*..." is stepsize = -lr, which is the
+ * The reference passes stepsize = +alpha; the benchmark's "w -= lr*..." is stepsize = -lr, which is the
  * same fp32 result as subtracting (negation is exact).
  * sqrt: the unqualified call resolves to the float overload when the C++ <math.h> wrapper is in
  * scope (it is pulled in by the CUDA runtime header); the device functor computes

@@ -111,7 +111,7 @@ def test_standalone_epilogue_bit_exact(ccn, M, N, nP, p):
 
 
 def test_outproj_config5_full_size(ccn):
-    """BASELINE config 5 at full size (8192 x 1024 x 8192, 7 partials, p = 0.1, seed 0).  Checked by:
+    """benchmark configuration 5 at full size (8192 x 1024 x 8192, 7 partials, p = 0.1, seed 0).  Checked by:
     the exact dropout mask over all 2^26 outputs (torch recomputes nothing: dropped outputs equal the
     residual, kept ones almost never do), and the oracle on sampled rows."""
     M = N = 8192

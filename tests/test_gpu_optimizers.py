@@ -1,6 +1,6 @@
 """GPU parity tests: the HIP kernels behind the C ABI against the CPU oracle on identical seeded inputs.
 
-Bars (BASELINE north star): fp32 state within 1e-6 relative, fp16 weight copies within 1e-3, overflow
+Bars (north star of the benchmark): fp32 state within 1e-6 relative, fp16 weight copies within 1e-3, overflow
 flags exact.  The kernels are written to round where the oracle rounds, so the tests first ask for
 bit-identical results and report the largest ulp distance if that ever fails.
 """
@@ -85,7 +85,7 @@ def test_sgd_sizes_and_tails(ccn, N):
 
 
 def test_sgd_config1_full_size(ccn):
-    # BASELINE config 1: N = 2^20, P = 4, g ~ N(0, 1e-2), w ~ U(-0.1, 0.1), lr = 0.01
+    # benchmark configuration 1: N = 2^20, P = 4, g ~ N(0, 1e-2), w ~ U(-0.1, 0.1), lr = 0.01
     P, N = 4, 1 << 20
     g = grads_f32(0, P, N, 1e-2)
     w0 = weights_f32(0, N, 0.1)
@@ -172,7 +172,7 @@ def test_pseudo_adam_known_answer_and_parity(ccn):
 
 @pytest.mark.parametrize("P,N", [(8, 1 << 20), (8, 4099), (1, 1000), (5, 12345), (12, 7777)])
 def test_adam_config2_ten_steps(ccn, P, N):
-    # BASELINE config 2 at reduced N: fresh gradients every step, bias correction at t = 1..10
+    # benchmark configuration 2 at reduced N: fresh gradients every step, bias correction at t = 1..10
     w0 = weights_f32(0, N, 0.05)
     wd, md, vd = dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
     w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
@@ -203,7 +203,7 @@ def test_adam_reference_fixture(ccn):
 
 
 def test_adam_full_size_sampled(ccn):
-    """BASELINE config 2 at its full size (N = 2^28, P = 8).  Adam is elementwise, so the oracle is run on
+    """benchmark configuration 2 at its full size (N = 2^28, P = 8).  Adam is elementwise, so the oracle is run on
     the elements gathered at sampled indices (first/last elements, block edges and random positions)."""
     P, N = 8, 1 << 28
     gen = torch.Generator(device=DEV)
@@ -273,7 +273,7 @@ def test_mixed_precision_adam(ccn, P, N, plant):
 
 
 def test_mixed_precision_full_size_flag_and_skips(ccn):
-    """BASELINE config 3 at full size: one in 2^20 entries forced to inf.  Checked through properties:
+    """benchmark configuration 3 at full size: one in 2^20 entries forced to inf.  Checked through properties:
     flag == 1, exactly the planted elements keep their state, fp16 copy == fp16(w) everywhere."""
     P, N = 8, 1 << 28
     gen = torch.Generator(device=DEV)
@@ -398,7 +398,7 @@ def test_lamb_ragged_segments(ccn, mode, lamb_variant):
 
 
 def test_lamb_config4_reduced(ccn, lamb_variant):
-    # BASELINE config 4 layout at reduced size: 16 segments of 2^16, P = 8, wd = 0.01, two-pass norm + update
+    # benchmark configuration 4 layout at reduced size: 16 segments of 2^16, P = 8, wd = 0.01, two-pass norm + update
     P, nseg, seglen = 8, 16, 1 << 16
     N = nseg * seglen
     segs = [i * seglen for i in range(nseg + 1)]
@@ -475,7 +475,7 @@ def test_lamb_reference_fixture(ccn):
 
 
 def test_lamb_full_size_segments(ccn):
-    """BASELINE config 4 at full size (N = 2^28 as 256 segments of 2^20, P = 8): the oracle is run on four
+    """benchmark configuration 4 at full size (N = 2^28 as 256 segments of 2^20, P = 8): the oracle is run on four
     whole segments (first, two inner, last); segments are independent, so this is exact for them."""
     P, nseg, seglen = 8, 256, 1 << 20
     N = nseg * seglen

@@ -171,7 +171,7 @@ def test_adam_step1_closed_form():
 
 
 def test_adam_against_torch_optim():
-    # textbook Adam from a library (torch.optim.Adam on the CPU), 10 steps of BASELINE config 2 at small N
+    # textbook Adam from a library (torch.optim.Adam on the CPU), 10 steps of benchmark configuration 2 at small N
     P, N = 8, 1 << 14
     w0 = weights_f32(6, N, 0.05)
     w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)

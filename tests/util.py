@@ -1,4 +1,4 @@
-"""Seeded input generators for the BASELINE configurations and small helpers shared by the tests."""
+"""Seeded input generators for the benchmark configurations and small helpers shared by the tests."""
 import numpy as np
 
 
