@@ -420,28 +420,29 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
           slot[(u * 2 + 1) * BS + threadIdx.x] = w4;
           if (u + 1 < SUB) cur = nxt;
         }
-      } else
+      } else {
 #pragma unroll
-      for (int u = 0; u < SUB; u++) {
-        const uint32_t j0 = (u * BS + threadIdx.x) * 4;
-        Pack<float, 4> r4 = {}, w4 = {};
-        if (j0 < t.count) {
-          if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-            lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
-          } else {
+        for (int u = 0; u < SUB; u++) {
+          const uint32_t j0 = (u * BS + threadIdx.x) * 4;
+          Pack<float, 4> r4 = {}, w4 = {};
+          if (j0 < t.count) {
+            if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+              lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-              if (j0 + e < t.count) {
-                Pack<float, 1> r1, w1;
-                lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
-                r4.d[e] = r1.d[0];
-                w4.d[e] = w1.d[0];
+              for (int e = 0; e < 4; e++) {
+                if (j0 + e < t.count) {
+                  Pack<float, 1> r1, w1;
+                  lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
+                  r4.d[e] = r1.d[0];
+                  w4.d[e] = w1.d[0];
+                }
               }
             }
           }
+          slot[(u * 2) * BS + threadIdx.x] = r4;
+          slot[(u * 2 + 1) * BS + threadIdx.x] = w4;
         }
-        slot[(u * 2) * BS + threadIdx.x] = r4;
-        slot[(u * 2 + 1) * BS + threadIdx.x] = w4;
       }
       if (it + 1 < rounds && tile + G < rs.ntiles) {
         next = lamb_tile_of(lay, tile + G);
