@@ -103,7 +103,7 @@ def cpu_baseline_adam(P, budget_s=8.0):
             step_fn(reps + 2)
             reps += 1
             el = time.perf_counter() - t0
-            if el > budget_s or reps >= 50:
+            if el > budget_s or reps >= 400:
                 return el / (reps * n), reps
 
     one, reps1 = timed(lambda t: orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t))
