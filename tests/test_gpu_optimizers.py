@@ -600,3 +600,37 @@ def test_recorded_lamb_step_replays(ccn):
     graph.close()
     plan.close()
     stream.close()
+
+
+def test_lamb_resident_kernel_shares_the_gpu(ccn):
+    """The resident kernel assumes its whole grid is on the chip at once.  With another stream keeping the GPU busy that
+    need not hold: waits may run out and tiles go through the deferred list.  Whatever happens, the result is the same."""
+    P, nseg, seglen = 4, 16, 1 << 20
+    N = nseg * seglen
+    segs = [i * seglen for i in range(nseg + 1)]
+    g = grads_f32(91, P, N, 1e-3)
+    w0 = weights_f32(91, N, 0.05)
+    gd, wd = [dev(x) for x in g], dev(w0)
+    md, vd = torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    # the competing work: Adam steps over other buffers on a second stream
+    M = 1 << 26
+    og = [torch.zeros(M, device=DEV) for _ in range(8)]
+    ow, om, ov = (torch.zeros(M, device=DEV) for _ in range(3))
+    plan = ccn.LambPlan(segs)
+    a, b = ccn.Stream(), ccn.Stream()
+    torch.cuda.synchronize()
+    for t in (1, 2, 3):
+        for _ in range(6):
+            ccn.adam_f32(og, ow, om, ov, M, 1e-3, 0.9, 0.999, 1e-6, 1, b.h)
+        plan.step(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0, a.h)
+    a.sync()
+    b.sync()
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    for t in (1, 2, 3):
+        orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+    assert_f32_parity(host(md), m, "shared GPU: m")
+    assert_f32_parity(host(vd), v, "shared GPU: v")
+    assert ulp_diff_f32(host(wd), w) <= 2
+    plan.close()
+    a.close()
+    b.close()
