@@ -68,8 +68,12 @@ def test_unaligned_size_takes_scalar_tail():
     assert [r[0] for r in rows] == [1 << k for k in range(1, 10)]
 
 
-def test_model_parallel_program():
-    rows = run_program("ref-model-parallel-mm-ar-c", 2, 8, 1)
+@pytest.mark.parametrize("name", ["ref-model-parallel-mm-ar-c", "ref-model-parallel-mm-rs-c-ag",
+                                  "ref-model-parallel-ol-mm-fuse-rs-c-ag"])
+def test_model_parallel_programs(name):
+    """Every schedule of the reference's examples/model-parallel/model-parallel.cpp (the last one has no bias and no
+    dropout in its expression): each emitted program checks its GEMM + epilogue against its own CPU re-execution."""
+    rows = run_program(name, 2, 8, 1)
     # B in {8, 16}, S = 1024, H = 3072: M = B*S rows, N = 3072
     assert [r[0] for r in rows] == [8 * 1024 * 3072, 16 * 1024 * 3072]
     assert all("MatMulFused" in r[2] for r in rows)
