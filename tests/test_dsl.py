@@ -167,7 +167,7 @@ def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path)
     unf = (tmp_path / "adam-rs-c-ag.hip").read_text()
     assert "ccn_reduce_f32" in unf and "ccn_memcpy_d2d(w, S5" in unf         # ReduceScatter, kernel, AllGather
     mlp = (tmp_path / "model-parallel-mm-ar-c.hip").read_text()
-    assert "ccn_mlp_outproj_bf16" in mlp and "p_drop = 0.5f" in mlp
+    assert "ccn_mlp_outproj_bf16" in mlp and "p_drop = (float)0.5;" in mlp
 
 
 @pytest.mark.skipif(not os.path.exists(os.path.join(ROOT, "oracle", "_ref", "ref-adam")), reason="oracle/_ref not built")
