@@ -61,6 +61,27 @@ template <int VEC> __device__ __forceinline__ Vals<VEC> load_vals(const float* p
   }
   return r;
 }
+// fp16 gradients (stored as raw 16-bit patterns): widened to fp32 on load, four at a time from one 8-byte access.
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+__host__ __device__ inline float f16_bits_to_f32(uint16_t h) {
+  _Float16 x;
+  memcpy(&x, &h, 2);
+  return (float)x;
+}
+template <int VEC> __device__ __forceinline__ Vals<VEC> load_vals(const uint16_t* p) {
+  Vals<VEC> r;
+  if constexpr (VEC == 1) {
+    r.d[0] = f16_bits_to_f32(__builtin_nontemporal_load(p));
+  } else {
+    const u32x2 x = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+    r.d[0] = f16_bits_to_f32((uint16_t)(x[0] & 0xffffu)); r.d[1] = f16_bits_to_f32((uint16_t)(x[0] >> 16));
+    r.d[2] = f16_bits_to_f32((uint16_t)(x[1] & 0xffffu)); r.d[3] = f16_bits_to_f32((uint16_t)(x[1] >> 16));
+  }
+  return r;
+}
+__device__ __forceinline__ float load_one(const float* p) { return *p; }
+__device__ __forceinline__ float load_one(const uint16_t* p) { return f16_bits_to_f32(*p); }
+
 template <int VEC> __device__ __forceinline__ void store_vals(float* p, const Vals<VEC>& v) {
   if constexpr (VEC == 1) {
     __builtin_nontemporal_store(v.d[0], p);
@@ -120,12 +141,13 @@ template <int BS = kBlock> __device__ __forceinline__ double block_sum(double x,
 //   NIN        plain fp32 input arrays, read at the element index
 //   NOUT       fp32 output arrays (an in-place update lists the array under both)
 //   HAS_RED    the body's first operand is the sum over rank buffers (the lowered AllReduce / ReduceScatter)
+//   RedT       element type of those buffers: float, or uint16_t holding fp16 bits (widened, then summed in fp32)
 //   NACC       sums of squares the body accumulates (inputs of Norm stages), float64
 //   NNORM      finished norms the body reads
 //   struct Scalars
 //   static void apply(float red, const float* in, float* out, const Scalars&, double* acc, const float* norms, uint64_t idx)
 template <class Body> struct KernelArgs {
-  const float* red[kMaxRanks];
+  const typename Body::RedT* red[kMaxRanks];
   int nranks;
   const float* in[Body::NIN > 0 ? Body::NIN : 1];
   float* out[Body::NOUT > 0 ? Body::NOUT : 1];
@@ -197,8 +219,8 @@ __global__ __launch_bounds__(BS) void fused_pointwise_kernel(const KernelArgs<Bo
       const size_t i = nvec * VEC + threadIdx.x;
       float red = 0.0f;
       if constexpr (Body::HAS_RED) {
-        red = a.red[0][i];
-        for (int p = 1; p < a.nranks; p++) red = red + a.red[p][i];
+        red = load_one(a.red[0] + i);
+        for (int p = 1; p < a.nranks; p++) red = red + load_one(a.red[p] + i);
       }
       float in1[NINX], out1[NOUTX];
       for (int k = 0; k < Body::NIN; k++) in1[k] = a.in[k][i];
@@ -272,7 +294,9 @@ inline unsigned grid_for(size_t n, int vec, int block) {
 }
 
 template <class Body, int VEC> unsigned launch_vec(const KernelArgs<Body>& a, hipStream_t s) {
-  const LaunchShape sh = shape_for((Body::HAS_RED ? a.nranks : 0) + Body::NIN, Body::NOUT, VEC);
+  // 16-byte loads per thread: an fp16 gradient pack is half of one
+  const int red_loads = Body::HAS_RED ? (a.nranks * (int)sizeof(typename Body::RedT) + 3) / 4 : 0;
+  const LaunchShape sh = shape_for(red_loads + Body::NIN, Body::NOUT, VEC);
   const unsigned grid = grid_for(a.n, VEC, sh.block);
   const int P = Body::HAS_RED ? a.nranks : 1;
   auto go = [&](auto ptag) {
@@ -301,8 +325,8 @@ inline unsigned blocks_for(size_t n) { return grid_for(n, 1, kBlock); }
 template <class Body> unsigned launch(const KernelArgs<Body>& a, void* stream) {
   if (a.n == 0) return 0;
   bool al = true;
-  if (Body::HAS_RED)
-    for (int p = 0; p < a.nranks; p++) al = al && aligned16(a.red[p]);
+  if (Body::HAS_RED)   // a pack of four is 16 bytes of fp32 or 8 bytes of fp16
+    for (int p = 0; p < a.nranks; p++) al = al && ((uintptr_t)a.red[p] & (4 * sizeof(typename Body::RedT) - 1)) == 0;
   for (int k = 0; k < Body::NIN; k++) al = al && aligned16(a.in[k]);
   for (int k = 0; k < Body::NOUT; k++) al = al && aligned16(a.out[k]);
   if (al) return launch_vec<Body, 4>(a, (hipStream_t)stream);
@@ -351,6 +375,21 @@ inline void fill_uniform(float* dev, size_t n, uint64_t seed, std::vector<float>
   CCNCHECK(ccn_memcpy_h2d(dev, h.data(), n * sizeof(float), nullptr));
   CCNCHECK(ccn_stream_sync(nullptr));
   if (keep) keep->swap(h);
+}
+
+// fp16 inputs: the same uniform stream rounded to fp16 (round to nearest even); `keep` receives the rounded values
+// widened back to fp32, which is what the kernels see.
+inline void fill_uniform_f16(uint16_t* dev, size_t n, uint64_t seed, std::vector<float>* keep = nullptr) {
+  std::vector<uint16_t> h(n);
+  std::vector<float> wide(keep ? n : 0);
+  for (size_t i = 0; i < n; i++) {
+    const _Float16 x = (_Float16)uniform01(seed, i);
+    memcpy(&h[i], &x, 2);
+    if (keep) wide[i] = (float)x;
+  }
+  CCNCHECK(ccn_memcpy_h2d(dev, h.data(), n * sizeof(uint16_t), nullptr));
+  CCNCHECK(ccn_stream_sync(nullptr));
+  if (keep) keep->swap(wide);
 }
 
 // relative comparison in the spirit of the reference's eqFloat (examples/header.h:55-62), with a tighter bound:

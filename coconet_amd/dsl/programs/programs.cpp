@@ -1,6 +1,6 @@
 // DSL programs for the benchmark configurations, written against the CoCoNet API.
 //   ccn-programs <program> <schedule> [output.hip]
-// program: sgd | clipsgd | reduction | adam | lamb     schedule: unfused | fused
+// program: sgd | clipsgd | reduction | adam | adamf16 | lamb     schedule: unfused | fused (adamf16: fused only)
 #include <dsl.hpp>
 #include <pipeline.hpp>
 
@@ -73,6 +73,25 @@ static void adam(bool fused, const std::string& out) {
   pl.codegen(out);
 }
 
+// The pipeline behind the reference's examples/test-adamf16.cu: fp16 gradients, fp32 state, the DSL example's
+// "Adam" (divide by beta, no square root), all in one kernel.  A Float16 tensor can only be reduced inside a fused kernel.
+static void adamf16(bool fused, const std::string& out) {
+  ASSERT(fused, "adamf16 has a fused schedule only");
+  Variable N(Int32, "N");
+  Variable lr(Float32, "lr"), b1(Float32, "beta1"), b2(Float32, "beta2");
+  Tensor g(Float16, N, Local, "g");
+  Tensor w(Float32, N, Replicated, "w"), m(Float32, N, Replicated, "m"), v(Float32, N, Replicated, "v");
+  Stage gs = AllReduce(Summation, g);
+  Stage vn = Update(v, b2 * v + (1 - b2) * (gs * gs));
+  Stage vh = vn / b2;
+  Stage mn = Update(m, b1 * m + (1 - b1) * gs);
+  Stage mh = mn / b1;
+  Stage wn = Update(w, w - (lr * mh) / vh);
+  Pipeline pl("adamf16", {g, w, m, v, lr, b1, b2}, {mn, vn, wn});
+  pl.fuse({gs, vn, vh, mn, mh, wn});
+  pl.codegen(out);
+}
+
 // LAMB with one global trust ratio (the DSL's Norm is over the whole tensor)
 static void lamb(bool fused, const std::string& out) {
   Variable N(Int32, "N");
@@ -95,7 +114,7 @@ static void lamb(bool fused, const std::string& out) {
 
 int main(int argc, char** argv) {
   if (argc < 3) {
-    std::cout << "usage: " << argv[0] << " <sgd|clipsgd|reduction|adam|lamb> <unfused|fused> [output.hip]" << std::endl;
+    std::cout << "usage: " << argv[0] << " <sgd|clipsgd|reduction|adam|adamf16|lamb> <unfused|fused> [output.hip]" << std::endl;
     return 1;
   }
   const std::string prog = argv[1], sched = argv[2];
@@ -106,6 +125,7 @@ int main(int argc, char** argv) {
   else if (prog == "clipsgd") clipsgd(fused, out);
   else if (prog == "reduction") reduction(fused, out);
   else if (prog == "adam") adam(fused, out);
+  else if (prog == "adamf16") adamf16(fused, out);
   else if (prog == "lamb") lamb(fused, out);
   else { std::cout << "Invalid program" << std::endl; return 1; }
   return 0;

@@ -101,6 +101,7 @@ const Node* strip(const Node* n) {
 struct Body {
   std::string name;
   bool hasRed = false;
+  bool redHalf = false;                  // the folded tensor holds fp16 elements
   std::string redTensor;                 // name of the Local tensor folded over ranks
   std::vector<std::string> inArrays;     // C expressions of device pointers, order = in[k]
   std::vector<std::string> inNames;      // local value names
@@ -175,6 +176,7 @@ struct BodyBuilder {
           ASSERT(n->args[0]->kind == Kind::Tensor, "fused reduce must read a Local tensor directly");
           ASSERT(!body.hasRed || body.redTensor == n->args[0]->name, "one reduced tensor per fused kernel");
           body.hasRed = true;
+          body.redHalf = n->args[0]->elem == Float16;
           body.redTensor = n->args[0]->name;
           return "red";
         }
@@ -251,6 +253,7 @@ std::string body_text(const Body& b, const std::vector<NodePtr>& scalarVars) {
   o << "  static constexpr int NIN = " << b.inArrays.size() << ", NOUT = " << b.outArrays.size() << ", NACC = " << b.nacc
     << ", NNORM = " << b.nnorm << ";\n";
   o << "  static constexpr bool HAS_RED = " << (b.hasRed ? "true" : "false") << ";\n";
+  o << "  using RedT = " << (b.redHalf ? "uint16_t" : "float") << ";\n";
   o << "  struct Scalars {";
   for (auto& v : scalarVars) o << " " << elem_c_type(v->elem) << " " << v->name << ";";
   o << " uint64_t seed__; };\n";
@@ -303,8 +306,10 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
              "variable '" << v->name << "' is used but is not a pipeline argument");
     find_reduced(st->args[0], prog.reducedTensors);
   }
+  // fp32 everywhere, except that a gradient tensor folded over the ranks may hold fp16 (widened on load, summed in fp32)
   for (auto& t : prog.tensors)
-    ASSERT(t->elem == Float32, "HIP target: tensor '" << t->name << "' must be Float32 in pointwise pipelines");
+    ASSERT(t->elem == Float32 || (t->elem == Float16 && prog.reducedTensors.count(t.get())),
+           "HIP target: tensor '" << t->name << "' must be Float32 (Float16 only for a tensor read through AllReduce/ReduceScatter)");
 
   const auto groups = p.groupsInOrder();
   const std::string fn = [&] { std::string s = p.name(); for (auto& c : s) if (!isalnum((unsigned char)c)) c = '_'; return s; }();
@@ -337,6 +342,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
     if (g.stages.size() == 1 && core->kind == Kind::Collective && core->args[0]->kind == Kind::Tensor &&
         prog.reducedTensors.count(core->args[0].get())) {
       // a collective on its own: the stock all-reduce, here the library's P-way reduce into rank 0's buffer
+      ASSERT(core->args[0]->elem == Float32, "HIP target: a Float16 tensor can only be reduced inside a fused kernel; fuse '"
+                                                 << p.stages()[g.stages[0]]->name << "' with its consumers");
       step.type = Step::Reduce;
       step.label = core->coll == CollOp::AllReduce ? "AllReduce" : "ReduceScatter";
       step.src = core->args[0]->name;
@@ -449,7 +456,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
     };
     for (auto& d : prog.dimVars) add("size_t", d->name);
     for (auto& v : prog.scalarVars) add(elem_c_type(v->elem), v->name);
-    for (auto& t : prog.tensors) add(prog.reducedTensors.count(t.get()) ? "float* const*" : "float*", t->name);
+    for (auto& t : prog.tensors)
+      add(prog.reducedTensors.count(t.get()) ? (t->elem == Float16 ? "uint16_t* const*" : "float* const*") : "float*", t->name);
     for (int k : prog.ownBuffers) add("float*", p.stages()[k]->name);
     add("double*", "partials__");
     add("float*", "norms__");
@@ -628,11 +636,12 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   for (auto& t : prog.tensors) {
     const std::string cnt = count_expr(t);
     if (prog.reducedTensors.count(t.get())) {
-      o << ind << "std::vector<float*> " << t->name << "(comm_size);\n";
+      const bool half = t->elem == Float16;
+      o << ind << "std::vector<" << (half ? "uint16_t" : "float") << "*> " << t->name << "(comm_size);\n";
       o << ind << "std::vector<std::vector<float>> h_" << t->name << "(comm_size);\n";
       o << ind << "for (int p_ = 0; p_ < comm_size; p_++) {\n";
-      o << ind << "  CCNCHECK(ccn_malloc((void**)&" << t->name << "[p_], (" << cnt << ") * sizeof(float)));\n";
-      o << ind << "  ccn_gen::fill_uniform(" << t->name << "[p_], " << cnt << ", seed__ + " << (seedNo + 100) << " + p_, check__ ? &h_"
+      o << ind << "  CCNCHECK(ccn_malloc((void**)&" << t->name << "[p_], (" << cnt << ") * sizeof(" << (half ? "uint16_t" : "float") << ")));\n";
+      o << ind << "  ccn_gen::fill_uniform" << (half ? "_f16" : "") << "(" << t->name << "[p_], " << cnt << ", seed__ + " << (seedNo + 100) << " + p_, check__ ? &h_"
         << t->name << "[p_] : nullptr);\n" << ind << "}\n";
       seedNo += 100;
     } else {

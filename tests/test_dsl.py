@@ -120,6 +120,19 @@ def test_ite_lowers_to_a_conditional_in_kernel_and_checker(dsl_build, tmp_path):
     assert "HAS_RED = true" in text
 
 
+def test_fp16_gradients_are_widened_inside_the_fused_kernel(dsl_build, tmp_path):
+    """A Float16 Local tensor (the reference's examples/test-adamf16.cu pipeline) is read as 16-bit patterns by the fused
+    kernel and summed in fp32; reducing it outside a fused kernel is refused with a message."""
+    exe = os.path.join(dsl_build, "ccn-programs")
+    out = tmp_path / "adamf16.hip"
+    assert run(exe, "adamf16", "fused", str(out)).returncode == 0
+    text = out.read_text()
+    assert "using RedT = uint16_t;" in text and "uint16_t* const* g" in text and "fill_uniform_f16(g[p_]" in text
+    assert "sizeof(uint16_t)" in text
+    r = run(exe, "adamf16", "unfused", str(tmp_path / "x.hip"))
+    assert r.returncode != 0 and "fused schedule only" in r.stderr
+
+
 def test_reduce_stage_is_a_plain_sum(dsl_build, tmp_path):
     """ReduceStage(stage, Summation) (the S2 loop of the reference's examples/test-reduction.cu:17-19) accumulates the
     values, not their squares, and finishes without a square root; it shares the two-pass lowering with Norm."""

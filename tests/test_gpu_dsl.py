@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GEN = os.path.join(ROOT, "coconet_amd", "dsl", "build", "gen")
 LINE = re.compile(r"^\{SZ: (\d+), Epochs: (\d+)((?:, \w+: [0-9.eE+-]+)+)\}$")
 
-OWN = ["sgd-fused", "sgd-unfused", "clipsgd-fused", "clipsgd-unfused", "reduction-fused", "reduction-unfused", "adam-fused", "adam-unfused", "lamb-fused", "lamb-unfused"]
+OWN = ["sgd-fused", "sgd-unfused", "clipsgd-fused", "clipsgd-unfused", "reduction-fused", "reduction-unfused", "adam-fused", "adam-unfused", "adamf16-fused", "lamb-fused", "lamb-unfused"]
 REF = ["ref-sgd-ar-c", "ref-sgd-rs-c-ag", "ref-sgd-fuse-rs-c-ag", "ref-adam-ar-c", "ref-adam-rs-c-ag",
        "ref-adam-fuse-rs-c-ag", "ref-lamb-ar-c", "ref-lamb-rs-c-ag", "ref-lamb-fuse-rs-c-ag"]
 
