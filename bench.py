@@ -32,7 +32,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adam_f32",
-                    choices=["adam_f32", "sgd_f32", "adam_f16g", "lamb_f32", "mlp_outproj", "copy"])
+                    choices=["adam_f32", "adam_f32_scattered", "sgd_f32", "adam_f16g", "lamb_f32", "mlp_outproj", "copy"])
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -148,7 +148,27 @@ def main():
     gen.manual_seed(0)
 
     flops = None
-    if wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g"):
+    if wl == "adam_f32_scattered":
+        # the same step with gradients and weights in 256 separate buffers (one per "parameter tensor")
+        P = a.ranks or 8
+        N = 1 << (a.log2n or 28)
+        nbuff = 256
+        per = N // nbuff
+        bufs = Buffers(capi, torch, a.allocator == "torch")
+        mk = lambda scale: bufs.from_tensor(torch.empty(per, device="cuda").normal_(0.0, scale, generator=gen))
+        g = [[mk(1e-3) for _ in range(nbuff)] for _ in range(P)]
+        w = [mk(0.05) for _ in range(nbuff)]
+        m = bufs.from_tensor(torch.zeros(N, device="cuda"))
+        v = bufs.from_tensor(torch.zeros(N, device="cuda"))
+        plan = capi.ScatterPlan([per] * nbuff)
+        per_param = (P + 3) * 4 + 3 * 4
+        step = lambda t: plan.adam(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t, stream)
+        kernel = "scattered_stream_kernel<AdamMath, %d>" % (P if P <= 8 else 0)
+        alg_bytes = float(per_param) * N
+        units = N
+        config = {"workload": f"adam_f32 over {nbuff} scattered buffers, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,
+                  "algorithmic_bytes_per_param": per_param, "allocator": a.allocator}
+    elif wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g"):
         P = a.ranks or (4 if wl == "sgd_f32" else 8)
         N = 1 << (a.log2n or (20 if wl == "sgd_f32" else 28))
         gbytes = 2 if wl == "adam_f16g" else 4

@@ -32,6 +32,7 @@ SYMBOLS = [
     "ccn_adam_f16g", "ccn_overflow_check_f16", "ccn_fused_adam_ref_f16g", "ccn_lamb_plan_create",
     "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
     "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
+    "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
 ]
 
 
@@ -98,6 +99,10 @@ def _declare(L):
     sig("ccn_lamb_plan_norms", [_vp, _vp, _vp])
     sig("ccn_mlp_outproj_bf16", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _vp])
     sig("ccn_bias_dropout_residual", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _vp])
+    sig("ccn_scatter_plan_create", [C.POINTER(_sz), _i, _pp])
+    sig("ccn_scatter_plan_destroy", [_vp])
+    sig("ccn_sgd_f32_scattered", [_vp, _pp, _i, _pp, _f, _vp])
+    sig("ccn_adam_f32_scattered", [_vp, _pp, _i, _pp, _vp, _vp, _f, _f, _f, _f, _i, _vp])
     sig("ccn_graph_begin", [_vp])
     sig("ccn_graph_end", [_vp, _pp])
     sig("ccn_graph_launch", [_vp, _vp])
@@ -198,6 +203,39 @@ class Event:
                 load().ccn_event_destroy(self.h)
         except Exception:
             pass
+
+
+class ScatterPlan:
+    """Tile table for nbuff separate gradient / weight buffers of the given element counts (ccn_scatter_plan)."""
+
+    def __init__(self, counts):
+        self.counts = [int(c) for c in counts]
+        arr = (_sz * len(self.counts))(*self.counts)
+        h = C.c_void_p()
+        _check(load().ccn_scatter_plan_create(arr, len(self.counts), C.byref(h)), "ccn_scatter_plan_create")
+        self.h = h
+
+    def _tables(self, g, w):
+        """g: P lists of nbuff buffers; w: nbuff buffers."""
+        nb = len(self.counts)
+        assert len(w) == nb and all(len(gp) == nb for gp in g)
+        gt = (C.c_void_p * (len(g) * nb))(*[addr(x) for gp in g for x in gp])
+        wt = (C.c_void_p * nb)(*[addr(x) for x in w])
+        return gt, wt
+
+    def sgd(self, g, w, lr, stream=None):
+        gt, wt = self._tables(g, w)
+        _check(load().ccn_sgd_f32_scattered(self.h, gt, len(g), wt, lr, stream), "ccn_sgd_f32_scattered")
+
+    def adam(self, g, w, m, v, lr, beta1, beta2, eps, step, stream=None):
+        gt, wt = self._tables(g, w)
+        _check(load().ccn_adam_f32_scattered(self.h, gt, len(g), wt, addr(m), addr(v), lr, beta1, beta2, eps, step, stream),
+               "ccn_adam_f32_scattered")
+
+    def close(self):
+        if self.h:
+            _check(load().ccn_scatter_plan_destroy(self.h), "ccn_scatter_plan_destroy")
+            self.h = None
 
 
 class Stream:

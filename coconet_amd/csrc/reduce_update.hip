@@ -10,6 +10,9 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <cstring>
+#include <new>
+#include <vector>
 
 namespace ccn {
 
@@ -275,6 +278,90 @@ __global__ __launch_bounds__(kBlock) void fill_f32_kernel(float* __restrict__ ds
 }
 
 // ------------------------------------------------------------------------------------------------------------------
+// Scattered layout: gradients and weights live in nbuff separate buffers (one per parameter tensor), the moments in
+// single arrays that follow the buffers' concatenation, as ncclAllReduceScatteredAdam takes them
+// (nccl-overlap/src/nccl.h.in:216-218).  A plan cuts every buffer into tiles of kScatTile elements; one
+// single-wavefront workgroup per tile reads the tile record, then the buffer's pointers from a device table
+// (rank-major gradient pointers, then the weight pointers), then streams exactly like fused_stream_kernel.
+// State array 0 of the policy (w) is scattered, the others (m, v) are contiguous.
+// ------------------------------------------------------------------------------------------------------------------
+constexpr int kScatTile = kWave * 4;   // 256 elements: one 4-element pack per lane
+
+struct ScatTile {
+  uint64_t off;    // first element inside the buffer
+  uint64_t goff;   // first element in the concatenation (index into the moment arrays)
+  uint32_t buf;
+  uint32_t count;  // elements in the tile (<= kScatTile)
+};
+
+template <class M, int P>
+__global__ __launch_bounds__(kWave) void scattered_stream_kernel(const ScatTile* __restrict__ tiles,
+                                                                 const float* const* __restrict__ gtab,
+                                                                 float* const* __restrict__ wtab, const int nP,
+                                                                 const uint32_t nbuff, const StateTable<M::NS> moments,
+                                                                 const typename M::Prm prm) {
+  static_assert(M::NS >= 1 && !M::OUT16 && !M::OUTF && !M::FLAG, "fp32 policies with w as state 0");
+  constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
+  const ScatTile t = tiles[(size_t)blockIdx.x + (size_t)blockIdx.y * gridDim.x];
+  const float* gp[PX];
+  uintptr_t bits = 0;
+#pragma unroll
+  for (int p = 0; p < PX; p++) {
+    if (P > 0 || p < nP) {
+      gp[p] = gtab[(size_t)p * nbuff + t.buf] + t.off;
+      bits |= reinterpret_cast<uintptr_t>(gp[p]);
+    }
+  }
+  float* sp[M::NS];
+  sp[0] = wtab[t.buf] + t.off;
+#pragma unroll
+  for (int k = 1; k < M::NS; k++) sp[k] = moments.p[k] + t.goff;
+#pragma unroll
+  for (int k = 0; k < M::NS; k++) bits |= reinterpret_cast<uintptr_t>(sp[k]);
+  const uint32_t j0 = threadIdx.x * 4;
+  if (j0 >= t.count) return;
+  if ((bits & 15u) == 0 && j0 + 4 <= t.count) {
+    Pack<float, 4> gv[PX], sv[M::NS];
+#pragma unroll
+    for (int p = 0; p < PX; p++)
+      if (P > 0 || p < nP) gv[p] = load_stream<float, 4>(gp[p] + j0);
+#pragma unroll
+    for (int k = 0; k < M::NS; k++) sv[k] = load_stream<float, 4>(sp[k] + j0);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      typename M::Acc a = M::first(gv[0].d[e], prm);
+#pragma unroll
+      for (int p = 1; p < PX; p++)
+        if (P > 0 || p < nP) M::next(a, gv[p].d[e], prm);
+      float s[M::NS];
+#pragma unroll
+      for (int k = 0; k < M::NS; k++) s[k] = sv[k].d[e];
+      uint16_t o16 = 0;
+      float of = 0.f;
+      (void)M::apply(a, s, o16, of, prm);
+#pragma unroll
+      for (int k = 0; k < M::NS; k++) sv[k].d[e] = s[k];
+    }
+#pragma unroll
+    for (int k = 0; k < M::NS; k++) store_stream<float, 4>(sp[k] + j0, sv[k]);
+  } else {
+    const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
+    for (uint32_t j = j0; j < j1; j++) {
+      typename M::Acc a = M::first(gp[0][j], prm);
+      for (int p = 1; p < (P ? P : nP); p++) M::next(a, gp[p][j], prm);
+      float s[M::NS];
+#pragma unroll
+      for (int k = 0; k < M::NS; k++) s[k] = sp[k][j];
+      uint16_t o16 = 0;
+      float of = 0.f;
+      (void)M::apply(a, s, o16, of, prm);
+#pragma unroll
+      for (int k = 0; k < M::NS; k++) sp[k][j] = s[k];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
 // Host side: validation, alignment-based choice of the access width, dispatch on P.
 // ------------------------------------------------------------------------------------------------------------------
 template <class M, int P, int VEC, int UNROLL>
@@ -363,6 +450,86 @@ static AdamPrm make_adam_prm(float lr, float beta1, float beta2, float eps, int 
 
 using namespace ccn;
 
+struct ccn_scatter_plan {
+  int device = -1;
+  uint32_t nbuff = 0;
+  size_t total = 0;
+  size_t ntiles = 0;
+  ScatTile* tiles = nullptr;
+  const void** table_dev = nullptr;    // [CCN_MAX_RANKS * nbuff] gradient pointers, rank-major, then [nbuff] weight pointers
+  const void** table_pinned = nullptr; // staging copy in pinned host memory
+  std::vector<const void*> shadow;     // what the device table holds
+  int shadow_ranks = 0;
+};
+
+namespace {
+
+// Brings the device pointer table in line with the caller's pointers; copies (and waits for the copy, so that the
+// staging buffer can be reused) only when they have changed since the last call.
+int sync_pointer_table(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, hipStream_t s) {
+  const size_t nb = plan->nbuff, words = (size_t)(CCN_MAX_RANKS + 1) * nb;
+  bool same = plan->shadow_ranks == P && plan->shadow.size() == words;
+  for (int p = 0; same && p < P; p++)
+    for (size_t b = 0; b < nb; b++) same = same && plan->shadow[(size_t)p * nb + b] == g[(size_t)p * nb + b];
+  for (size_t b = 0; same && b < nb; b++) same = same && plan->shadow[(size_t)CCN_MAX_RANKS * nb + b] == w[b];
+  if (same) return CCN_OK;
+  plan->shadow.assign(words, nullptr);
+  for (int p = 0; p < P; p++)
+    for (size_t b = 0; b < nb; b++) plan->shadow[(size_t)p * nb + b] = g[(size_t)p * nb + b];
+  for (size_t b = 0; b < nb; b++) plan->shadow[(size_t)CCN_MAX_RANKS * nb + b] = w[b];
+  plan->shadow_ranks = P;
+  std::memcpy(plan->table_pinned, plan->shadow.data(), words * sizeof(void*));
+  CCN_HIP(hipMemcpyAsync(plan->table_dev, plan->table_pinned, words * sizeof(void*), hipMemcpyHostToDevice, s));
+  CCN_HIP(hipStreamSynchronize(s));
+  return CCN_OK;
+}
+
+template <class M>
+int launch_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, float* const* moments,
+                     const typename M::Prm& prm, void* stream) {
+  if (!plan || !g || !w || P < 1 || P > CCN_MAX_RANKS) return CCN_EINVAL;
+  for (size_t i = 0; i < (size_t)P * plan->nbuff; i++) if (!g[i]) return CCN_EINVAL;
+  for (size_t b = 0; b < plan->nbuff; b++) if (!w[b]) return CCN_EINVAL;
+  StateTable<M::NS> st;
+  st.p[0] = nullptr;
+  for (int k = 1; k < M::NS; k++) {
+    if (!moments || !moments[k - 1]) return CCN_EINVAL;
+    st.p[k] = moments[k - 1];
+  }
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  if (di->device != plan->device) return CCN_EINVAL;
+  hipStream_t s = as_stream(stream);
+  rc = sync_pointer_table(plan, g, P, w, s);
+  if (rc != CCN_OK) return rc;
+  const float* const* gtab = reinterpret_cast<const float* const*>(plan->table_dev);
+  float* const* wtab = reinterpret_cast<float* const*>(const_cast<void**>(plan->table_dev) + (size_t)CCN_MAX_RANKS * plan->nbuff);
+  // A wavefront here reads its tile record, then the buffer's pointers, and only then its data: two more round trips
+  // than the flat kernels, so more wavefronts per CU are needed to keep loads in flight (measured at P = 8: 10-16 per
+  // CU give 76 % of HBM peak, the flat kernels' 7 give 73 %).  The tuning override of stream_shape still applies.
+  const StreamShape sh = stream_shape((P + M::NS) * 16, M::NS * 16);
+  unsigned lds = lds_for_residency(10);
+  if (sh.lds_bytes != 0 && sh.lds_bytes < lds) lds = sh.lds_bytes;
+  const size_t gx = plan->ntiles < 0x40000000ull ? plan->ntiles : 0x40000000ull;
+  const dim3 grid((unsigned)gx, (unsigned)((plan->ntiles + gx - 1) / gx));
+  if (grid.x * (size_t)grid.y != plan->ntiles) return CCN_ERANGE;   // the kernel has no bounds check on the tile index
+  switch (P) {
+#define CCN_CASE(K) \
+  case K: hipLaunchKernelGGL((scattered_stream_kernel<M, K>), grid, dim3(kWave), lds, s, (const ScatTile*)plan->tiles, gtab, \
+                             wtab, P, plan->nbuff, st, prm); break;
+    CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
+#undef CCN_CASE
+    default:
+      hipLaunchKernelGGL((scattered_stream_kernel<M, 0>), grid, dim3(kWave), lds, s, (const ScatTile*)plan->tiles, gtab, wtab, P,
+                         plan->nbuff, st, prm);
+  }
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int ccn_fill_f32(float* dst, float value, size_t n, void* stream) {
@@ -419,6 +586,67 @@ int ccn_fused_adam_ref_f16g(const uint16_t* const* g, int P, float* w, uint16_t*
   float* st[3] = {w, m, v};
   FusedAdamRefMath::Prm k{lr, beta1, beta2, 1 - beta2};
   return launch<FusedAdamRefMath>(g, P, st, halfw, nullptr, nullptr, N, k, stream);
+}
+
+int ccn_scatter_plan_destroy(ccn_scatter_plan* plan) {
+  if (!plan) return CCN_OK;
+  int rc = CCN_OK;
+  if (plan->tiles && hipFree(plan->tiles) != hipSuccess) rc = CCN_EHIP;
+  if (plan->table_dev && hipFree(plan->table_dev) != hipSuccess) rc = CCN_EHIP;
+  if (plan->table_pinned && hipHostFree(plan->table_pinned) != hipSuccess) rc = CCN_EHIP;
+  delete plan;
+  return rc;
+}
+
+int ccn_scatter_plan_create(const size_t* counts, int nbuff, ccn_scatter_plan** out) {
+  if (!out) return CCN_EINVAL;
+  *out = nullptr;
+  if (!counts || nbuff < 1) return CCN_EINVAL;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  std::vector<ScatTile> tiles;
+  size_t total = 0;
+  for (int b = 0; b < nbuff; b++) {
+    if (counts[b] == 0) return CCN_EINVAL;
+    for (size_t off = 0; off < counts[b]; off += kScatTile) {
+      ScatTile t;
+      t.off = off;
+      t.goff = total + off;
+      t.buf = (uint32_t)b;
+      t.count = (uint32_t)(counts[b] - off < (size_t)kScatTile ? counts[b] - off : (size_t)kScatTile);
+      tiles.push_back(t);
+    }
+    total += counts[b];
+  }
+  ccn_scatter_plan* p = new (std::nothrow) ccn_scatter_plan();
+  if (!p) return CCN_ENOMEM;
+  p->device = di->device;
+  p->nbuff = (uint32_t)nbuff;
+  p->total = total;
+  p->ntiles = tiles.size();
+  const size_t words = (size_t)(CCN_MAX_RANKS + 1) * (size_t)nbuff;
+  hipError_t e = hipMalloc((void**)&p->tiles, tiles.size() * sizeof(ScatTile));
+  if (e == hipSuccess) e = hipMalloc((void**)&p->table_dev, words * sizeof(void*));
+  if (e == hipSuccess) e = hipHostMalloc((void**)&p->table_pinned, words * sizeof(void*), hipHostMallocDefault);
+  if (e == hipSuccess) e = hipMemcpy(p->tiles, tiles.data(), tiles.size() * sizeof(ScatTile), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    ccn_scatter_plan_destroy(p);
+    return hip_fail(e);
+  }
+  *out = p;
+  return CCN_OK;
+}
+
+int ccn_sgd_f32_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, float lr, void* stream) {
+  return launch_scattered<SgdMath>(plan, g, P, w, nullptr, SgdMath::Prm{lr}, stream);
+}
+
+int ccn_adam_f32_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v,
+                           float lr, float beta1, float beta2, float eps, int step, void* stream) {
+  if (step < 1) return CCN_EINVAL;
+  float* mom[2] = {m, v};
+  return launch_scattered<AdamMath>(plan, g, P, w, mom, make_adam_prm(lr, beta1, beta2, eps, step, 1.0f), stream);
 }
 
 }  // extern "C"

@@ -112,6 +112,20 @@ int  ccn_pseudo_adam_f32(const float* const* g, int P, float* w, float* m, float
 int  ccn_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
                   float lr, float beta1, float beta2, float eps, int step, void* stream);
 
+/* ---- the same SGD and Adam steps over scattered buffers: gradients and weights stay in nbuff separate buffers (one
+ *      per parameter tensor, counts[b] elements each), the moments in single arrays of sum(counts) elements that
+ *      follow the buffers' concatenation.  This is the layout ncclAllReduceScatteredAdam takes
+ *      (nccl-overlap/src/nccl.h.in:216-218; caller nccl-overlap/samples/multi-process-adam-scattered.cpp:334-337).
+ *      g is a host array of P*nbuff device pointers, rank-major (g[p*nbuff + b]); w a host array of nbuff device
+ *      pointers.  The plan keeps a device copy of the pointers and refreshes it, with one stream synchronisation,
+ *      only when they change; calls on one plan must be ordered (same stream). ---- */
+typedef struct ccn_scatter_plan ccn_scatter_plan;
+int  ccn_scatter_plan_create(const size_t* counts, int nbuff, ccn_scatter_plan** plan);
+int  ccn_scatter_plan_destroy(ccn_scatter_plan* plan);
+int  ccn_sgd_f32_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, float lr, void* stream);
+int  ccn_adam_f32_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v,
+                            float lr, float beta1, float beta2, float eps, int step, void* stream);
+
 /* ---- mixed-precision Adam: fp16 gradients carrying a loss scale, fp32 master state, fp16 weight copy.
  *      gs = sum_p float(g[p][i])*inv_scale.  overflow_flag (device, one uint32) is SET by the call:
  *      1 if any g[p][i] is inf/nan, else 0.  Elements whose gradients overflow keep w, m, v unchanged;

@@ -634,3 +634,47 @@ def test_lamb_resident_kernel_shares_the_gpu(ccn):
     plan.close()
     a.close()
     b.close()
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("P", [1, 3, 8, 11])
+def test_scattered_adam_and_sgd(ccn, P):
+    """Gradients and weights in separate buffers of ragged sizes (two of them misaligned by 4 bytes), moments in single
+    arrays over the concatenation: the same results, bit for bit, as the oracle on the concatenated arrays."""
+    counts = [1, 255, 256, 257, 1000, 4096, 70001, 3]
+    offs = np.concatenate([[0], np.cumsum(counts)])
+    N = int(offs[-1])
+    g = grads_f32(95 + P, P, N, 1e-3)
+    w0 = weights_f32(95, N, 0.05)
+
+    def pieces(flat, shift_some):
+        out = []
+        for b, n in enumerate(counts):
+            lo = int(offs[b])
+            if shift_some and b in (3, 5):      # a buffer that starts 4 bytes past a 16-byte boundary
+                out.append(dev(np.concatenate([[np.float32(0)], flat[lo:lo + n]]))[1:])
+            else:
+                out.append(dev(flat[lo:lo + n]))
+        return out
+
+    gd = [pieces(x, True) for x in g]
+    wd = pieces(w0, True)
+    md, vd = torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    plan = ccn.ScatterPlan(counts)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    for t in (1, 2, 3):
+        plan.adam(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, t)
+        orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t)
+    plan.sgd(gd, wd, 0.01)
+    orc.sgd_f32(g, w, 0.01)
+    got_w = np.concatenate([host(x) for x in wd])
+    assert_f32_parity(got_w, w, "scattered w")
+    assert_f32_parity(host(md), m, "scattered m")
+    assert_f32_parity(host(vd), v, "scattered v")
+    # new weight buffers: the pointer table follows
+    wd2 = pieces(w0, False)
+    plan.sgd(gd, wd2, 0.5)
+    w2 = w0.copy()
+    orc.sgd_f32(g, w2, 0.5)
+    assert_f32_parity(np.concatenate([host(x) for x in wd2]), w2, "scattered w after a pointer change")
+    plan.close()
