@@ -16,6 +16,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <cstring>
 #include <new>
 #include <type_traits>
 #include <vector>
@@ -39,7 +40,35 @@ struct LambLayout {
   uint64_t seg_len;         // common segment length, or 0 for a ragged layout
   float seg_len_f;
   uint32_t tile;            // elements per full tile
+  // Scattered buffers (one gradient / weight buffer per segment, moments still in single arrays): device tables of the
+  // segments' pointers, each already moved back by the segment's first element index, so that "pointer + global element
+  // index" addresses the segment's elements exactly as it does for flat arrays.  Null for flat arrays.
+  const float* const* gtab;   // [P][nseg], rank-major
+  float* const* wtab;         // [nseg]
+  uint32_t nseg;
 };
+
+// Gradient table and weight pointer to use for the elements of segment `seg`.
+// SCAT is a compile-time choice so that the flat kernels carry none of this.
+template <int P, bool SCAT>
+__device__ __forceinline__ void lamb_buffers_of(const LambLayout& L, const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g_flat,
+                                                float* w_flat, int nP, uint32_t seg,
+                                                SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, float*& w) {
+  if constexpr (!SCAT) {
+    g = g_flat;
+    w = w_flat;
+    return;
+  }
+  constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
+#pragma unroll
+  for (int p = 0; p < PX; p++) g.p[p] = (P > 0 || p < nP) ? L.gtab[(size_t)p * L.nseg + seg] : nullptr;
+  w = L.wtab[seg];
+}
+template <bool SCAT>
+__device__ __forceinline__ float* lamb_weights_of(const LambLayout& L, float* w_flat, uint32_t seg) {
+  if constexpr (SCAT) return L.wtab[seg];
+  return w_flat;
+}
 
 __device__ __forceinline__ LambTile lamb_tile_of(const LambLayout& L, unsigned b) {
   if (L.seg_len != 0) {
@@ -132,23 +161,26 @@ __device__ __forceinline__ void lamb_pass1_pack(const SrcTable<float, (P ? P : C
   lamb_pass1_math<P, VEC>(in, nP, m, v, e0, nf, k, accW, accR, r_out, w_out);
 }
 
-template <int P>
+template <int P, bool SCAT>
 __global__ __launch_bounds__(kBlock) void lamb_pass1_kernel(const SrcTable<float, (P ? P : CCN_MAX_RANKS)> g, const int nP,
                                                             const float* w, float* m, float* v, const LambLayout lay,
                                                             double* __restrict__ partials, const int vec_ok,
                                                             const LambPrm k) {
   __shared__ double lds[2 * kBlock / kWave];
   const LambTile t = lamb_tile_of(lay, blockIdx.x);
+  SrcTable<float, (P ? P : CCN_MAX_RANKS)> gt;
+  float* wt;
+  lamb_buffers_of<P, SCAT>(lay, g, const_cast<float*>(w), nP, t.seg, gt, wt);
   double accW = 0.0, accR = 0.0;
   const uint32_t j0 = threadIdx.x * 4;          // this thread's elements of the tile: [j0, j0+4) clipped to count
   if (j0 < t.count) {
     if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
       Pack<float, 4> r4, w4;
-      lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
+      lamb_pass1_pack<P, 4>(gt, nP, wt, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
     } else {
       const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
       Pack<float, 1> r1, w1;
-      for (uint32_t j = j0; j < j1; j++) lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j, t.nf, k, accW, accR, r1, w1);
+      for (uint32_t j = j0; j < j1; j++) lamb_pass1_pack<P, 1>(gt, nP, wt, m, v, t.start + j, t.nf, k, accW, accR, r1, w1);
     }
   }
   const double sW = block_sum(accW, lds);
@@ -286,18 +318,20 @@ __device__ __forceinline__ void lamb_pass2_pack(float* w, const float* m, const 
   store_stream<float, VEC>(w + e0, wv);
 }
 
+template <bool SCAT>
 __global__ __launch_bounds__(kBlock) void lamb_pass2_kernel(float* w, const float* m, const float* v, const LambLayout lay,
                                                             const float* __restrict__ scale, const int vec_ok,
                                                             const LambPrm k) {
   const LambTile t = lamb_tile_of(lay, blockIdx.x);
+  float* const wt = lamb_weights_of<SCAT>(lay, w, t.seg);
   const float step_scale = k.lr * scale[t.seg];   // stepsize * scale, then times r
   const uint32_t j0 = threadIdx.x * 4;
   if (j0 >= t.count) return;
   if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-    lamb_pass2_pack<4>(w, m, v, t.start + j0, step_scale, k);
+    lamb_pass2_pack<4>(wt, m, v, t.start + j0, step_scale, k);
   } else {
     const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
-    for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(w, m, v, t.start + j, step_scale, k);
+    for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(wt, m, v, t.start + j, step_scale, k);
   }
 }
 
@@ -365,7 +399,7 @@ __device__ __forceinline__ void lamb_retire_tile(float* w, const LambTile& t, co
 }
 
 // BS threads per workgroup, SUB packs per thread per tile: a tile is BS * 4 * SUB elements.
-template <int P, int BS, int SUB>
+template <int P, int BS, int SUB, bool SCAT>
 __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float, (P ? P : CCN_MAX_RANKS)> g, const int nP,
                                                            float* w, float* m, float* v, const LambLayout lay,
                                                            double* partials, const uint64_t* __restrict__ seg_len,
@@ -390,9 +424,12 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
   };
   LambTile next{};
   LambIn<P, 4> pre;
+  SrcTable<float, (P ? P : CCN_MAX_RANKS)> gt = g;   // buffers of the tile in `next`
+  float* wt = w;
   if (blockIdx.x < rs.ntiles) {
     next = lamb_tile_of(lay, blockIdx.x);
-    if (is_fast(next)) lamb_pass1_load<P, 4>(pre, g, nP, w, m, v, next.start + threadIdx.x * 4);
+    lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.seg, gt, wt);
+    if (is_fast(next)) lamb_pass1_load<P, 4>(pre, gt, nP, wt, m, v, next.start + threadIdx.x * 4);
   }
   for (unsigned it = 0; it < rounds + (kResDepth - 1); it++) {
     const unsigned tile = blockIdx.x + it * G;
@@ -405,6 +442,8 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
     uint32_t arrived = 0, fan_target = 0, seg_tiles = 0;
     if (have_tile) {
       t = next;
+      const SrcTable<float, (P ? P : CCN_MAX_RANKS)> gc = gt;   // this tile's buffers
+      float* const wc = wt;
       Pack<float, 4>* slot = park + (size_t)(it % kResDepth) * kSlotPacks;
       double accW = 0.0, accR = 0.0;
       if (is_fast(t)) {
@@ -413,7 +452,7 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
         for (int u = 0; u < SUB; u++) {
           const size_t e0 = t.start + (size_t)(u * BS + threadIdx.x) * 4;
           LambIn<P, 4> nxt;
-          if (u + 1 < SUB) lamb_pass1_load<P, 4>(nxt, g, nP, w, m, v, e0 + BS * 4);
+          if (u + 1 < SUB) lamb_pass1_load<P, 4>(nxt, gc, nP, wc, m, v, e0 + BS * 4);
           Pack<float, 4> r4, w4;
           lamb_pass1_math<P, 4>(cur, nP, m, v, e0, t.nf, k, accW, accR, r4, w4);
           slot[(u * 2) * BS + threadIdx.x] = r4;
@@ -427,13 +466,13 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
           Pack<float, 4> r4 = {}, w4 = {};
           if (j0 < t.count) {
             if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-              lamb_pass1_pack<P, 4>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
+              lamb_pass1_pack<P, 4>(gc, nP, wc, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
             } else {
 #pragma unroll
               for (int e = 0; e < 4; e++) {
                 if (j0 + e < t.count) {
                   Pack<float, 1> r1, w1;
-                  lamb_pass1_pack<P, 1>(g, nP, w, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
+                  lamb_pass1_pack<P, 1>(gc, nP, wc, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
                   r4.d[e] = r1.d[0];
                   w4.d[e] = w1.d[0];
                 }
@@ -446,7 +485,8 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       }
       if (it + 1 < rounds && tile + G < rs.ntiles) {
         next = lamb_tile_of(lay, tile + G);
-        if (is_fast(next)) lamb_pass1_load<P, 4>(pre, g, nP, w, m, v, next.start + threadIdx.x * 4);
+        lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.seg, gt, wt);
+        if (is_fast(next)) lamb_pass1_load<P, 4>(pre, gt, nP, wt, m, v, next.start + threadIdx.x * 4);
       }
       const double sW = group_sum<BS>(accW, red);
       const double sR = group_sum<BS>(accR, red + kBlock / kWave);
@@ -473,8 +513,8 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       }
       __syncthreads();
       if (bc[1]) {
-        lamb_retire_tile<BS, SUB>(w, prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks, k.lr * __uint_as_float(bc[2]),
-                                  vec_ok);
+        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.seg), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
+                                  k.lr * __uint_as_float(bc[2]), vec_ok);
         retired = true;
       }
     }
@@ -519,8 +559,8 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       }
       __syncthreads();
       if (bc[1])
-        lamb_retire_tile<BS, SUB>(w, prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks, k.lr * __uint_as_float(bc[2]),
-                                  vec_ok);
+        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.seg), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
+                                  k.lr * __uint_as_float(bc[2]), vec_ok);
     }
     __syncthreads();   // bc and the retired slot are reused by the next round
     prev = t;
@@ -529,7 +569,7 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
 }
 
 // Finishes the deferred tiles: pass 2 from the stored m and v, as the two-pass path does.
-template <int BS, int SUB>
+template <int BS, int SUB, bool SCAT>
 __global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, const float* m, const float* v, const LambLayout lay,
                                                            const float* __restrict__ scale,
                                                            const uint32_t* __restrict__ deferred,
@@ -538,15 +578,16 @@ __global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, const float
   const uint32_t n = *ndeferred;
   for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
     const LambTile t = lamb_tile_of(lay, deferred[i]);
+    float* const wt = lamb_weights_of<SCAT>(lay, w, t.seg);
     const float step_scale = k.lr * scale[t.seg];
     for (int u = 0; u < SUB; u++) {
       const uint32_t j0 = (u * BS + threadIdx.x) * 4;
       if (j0 >= t.count) continue;
       if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-        lamb_pass2_pack<4>(w, m, v, t.start + j0, step_scale, k);
+        lamb_pass2_pack<4>(wt, m, v, t.start + j0, step_scale, k);
       } else {
         const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
-        for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(w, m, v, t.start + j, step_scale, k);
+        for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(wt, m, v, t.start + j, step_scale, k);
       }
     }
   }
@@ -588,6 +629,12 @@ struct ccn_lamb_plan {
   unsigned long long* ready = nullptr;
   uint32_t* deferred = nullptr;
   int occupancy[CCN_MAX_RANKS + 1] = {0};   // resident workgroups per CU by rank count, 0 = not asked yet
+  // scattered buffers: the segments' gradient and weight pointers, moved back by the segment's first element index
+  std::vector<uint64_t> seg_start;
+  const void** ptr_dev = nullptr;       // [CCN_MAX_RANKS * nseg] gradients, rank-major, then [nseg] weights; made on first use
+  const void** ptr_pinned = nullptr;
+  std::vector<const void*> ptr_shadow;  // what the device table holds
+  int ptr_ranks = 0;
 };
 
 namespace {
@@ -627,7 +674,7 @@ int resident_occupancy(int P, int block, int sub, unsigned lds) {
   int occ = 0;
   with_rank_count(P, [&](auto ptag) {
     with_resident_shape(block, sub, [&](auto bstag, auto subtag) {
-      auto* fn = lamb_resident_kernel<decltype(ptag)::value, decltype(bstag)::value, decltype(subtag)::value>;
+      auto* fn = lamb_resident_kernel<decltype(ptag)::value, decltype(bstag)::value, decltype(subtag)::value, false>;
       if (lds > 64 * 1024 &&
           hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
         (void)hipGetLastError();
@@ -664,10 +711,11 @@ int ccn_lamb_plan_destroy(ccn_lamb_plan* plan) {
   int rc = CCN_OK;
   void* bufs[] = {plan->tiles,  plan->seg_tile_begin,  plan->seg_len,   plan->partials, plan->norms,   plan->scale,
                   plan->rtiles, plan->seg_rtile_begin, plan->rpartials, plan->sync,     plan->deferred, plan->ready,
-                  plan->group_begin, plan->seg_group_begin, plan->folded};
+                  plan->group_begin, plan->seg_group_begin, plan->folded, (void*)plan->ptr_dev};
   for (void* b : bufs) {
     if (b && hipFree(b) != hipSuccess) rc = CCN_EHIP;
   }
+  if (plan->ptr_pinned && hipHostFree(plan->ptr_pinned) != hipSuccess) rc = CCN_EHIP;
   delete plan;
   return rc;
 }
@@ -761,6 +809,7 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   p->device = di->device;
   p->nseg = nseg;
   p->N = seg_offsets[nseg];
+  p->seg_start.assign(seg_offsets, seg_offsets + nseg);
   p->ntiles = tiles.size();
   p->uniform_seg_len = (all_two_pass && uniform % kLambTile == 0) ? uniform : 0;
   p->res_block = res_block;
@@ -808,15 +857,55 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   return CCN_OK;
 }
 
-int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, float* m, float* v, float lr, float beta1,
-                 float beta2, float eps, float wd, int step, int mode, void* stream) {
-  if (!plan || !g || !w || !m || !v || P < 1 || P > CCN_MAX_RANKS || step < 1) return CCN_EINVAL;
+}  // extern "C"
+
+namespace {
+
+// Brings the plan's device table of per-segment pointers in line with the caller's; copies (and waits for the copy, so
+// that the staging buffer can be reused) only when they have changed since the last call.  Returns whether every
+// pointer, moved back by its segment's first element index, is 16-byte aligned.
+int sync_segment_pointers(ccn_lamb_plan* plan, const float* const* g, int P, float* const* w, hipStream_t s, bool* aligned) {
+  const size_t ns = (size_t)plan->nseg, words = (size_t)(CCN_MAX_RANKS + 1) * ns;
+  if (!plan->ptr_dev) {
+    CCN_HIP(hipMalloc((void**)&plan->ptr_dev, words * sizeof(void*)));
+    CCN_HIP(hipHostMalloc((void**)&plan->ptr_pinned, words * sizeof(void*), hipHostMallocDefault));
+  }
+  std::vector<const void*> want(words, nullptr);
+  bool al = true;
+  auto moved = [&](const float* base, size_t seg) {
+    const float* q = base - plan->seg_start[seg];
+    al = al && aligned16(q);
+    return (const void*)q;
+  };
+  for (int p = 0; p < P; p++)
+    for (size_t b = 0; b < ns; b++) want[(size_t)p * ns + b] = moved(g[(size_t)p * ns + b], b);
+  for (size_t b = 0; b < ns; b++) want[(size_t)CCN_MAX_RANKS * ns + b] = moved(w[b], b);
+  *aligned = al;
+  if (plan->ptr_ranks == P && plan->ptr_shadow == want) return CCN_OK;
+  plan->ptr_shadow.swap(want);
+  plan->ptr_ranks = P;
+  std::memcpy(plan->ptr_pinned, plan->ptr_shadow.data(), words * sizeof(void*));
+  CCN_HIP(hipMemcpyAsync(plan->ptr_dev, plan->ptr_pinned, words * sizeof(void*), hipMemcpyHostToDevice, s));
+  CCN_HIP(hipStreamSynchronize(s));
+  return CCN_OK;
+}
+
+// One step.  Flat arrays: g holds P pointers, w_flat the weights, w_seg is null.  Scattered buffers: g holds P * nseg
+// pointers (rank-major), w_seg nseg pointers, w_flat is null.
+int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, float* const* w_seg, float* m, float* v, float lr,
+              float beta1, float beta2, float eps, float wd, int step, int mode, void* stream) {
+  const bool scattered = w_seg != nullptr;
+  if (!plan || !g || (!w_flat && !w_seg) || !m || !v || P < 1 || P > CCN_MAX_RANKS || step < 1) return CCN_EINVAL;
   if (mode != CCN_LAMB_TRUST_RATIO && mode != CCN_LAMB_REFERENCE && mode != CCN_LAMB_NCCL_GLOBAL) return CCN_EINVAL;
-  for (int p = 0; p < P; p++) if (!g[p]) return CCN_EINVAL;
+  const size_t ng = scattered ? (size_t)P * (size_t)plan->nseg : (size_t)P;
+  for (size_t i = 0; i < ng; i++) if (!g[i]) return CCN_EINVAL;
+  if (scattered)
+    for (int b = 0; b < plan->nseg; b++) if (!w_seg[b]) return CCN_EINVAL;
   const DeviceInfo* di = nullptr;
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
   if (di->device != plan->device) return CCN_EINVAL;
+  float* const w = w_flat;   // null for scattered buffers: the kernels then take every weight pointer from the table
 
   LambPrm k;
   k.b1 = beta1;
@@ -830,17 +919,28 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
   k.bc1 = 1 - std::pow((double)beta1, (double)step);
   k.bc2 = 1 - std::pow((double)beta2, (double)step);
 
-  bool al = aligned16(w) && aligned16(m) && aligned16(v);
-  for (int p = 0; p < P; p++) al = al && aligned16(g[p]);
-  const int vec_ok = al ? 1 : 0;
   hipStream_t s = as_stream(stream);
+  bool al = aligned16(m) && aligned16(v);
+  if (scattered) {
+    bool tal = true;
+    rc = sync_segment_pointers(plan, g, P, w_seg, s, &tal);
+    if (rc != CCN_OK) return rc;
+    al = al && tal;
+  } else {
+    al = al && aligned16(w);
+    for (int p = 0; p < P; p++) al = al && aligned16(g[p]);
+  }
+  const int vec_ok = al ? 1 : 0;
   const dim3 block(kBlock);
+  const float* const* gtab = scattered ? reinterpret_cast<const float* const*>(plan->ptr_dev) : nullptr;
+  float* const* wtab =
+      scattered ? reinterpret_cast<float* const*>(const_cast<void**>(plan->ptr_dev) + (size_t)CCN_MAX_RANKS * plan->nseg) : nullptr;
 
   auto with_ranks = [&](auto body) { with_rank_count(P, body); };
-  auto table = [&](auto ptag) {
+  auto table = [&](auto ptag) {   // the flat arrays' gradient pointers; unused (null) for scattered buffers
     constexpr int PP = decltype(ptag)::value;
     SrcTable<float, (PP ? PP : CCN_MAX_RANKS)> tbl;
-    for (int p = 0; p < (PP ? PP : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < P ? p : 0];
+    for (int p = 0; p < (PP ? PP : CCN_MAX_RANKS); p++) tbl.p[p] = scattered ? nullptr : g[p < P ? p : 0];
     return tbl;
   };
 
@@ -850,6 +950,9 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
     lay.seg_len = plan->res_uniform_seg_len;
     lay.seg_len_f = (float)plan->res_uniform_seg_len;
     lay.tile = (uint32_t)(plan->res_block * 4 * plan->res_sub);
+    lay.gtab = gtab;
+    lay.wtab = wtab;
+    lay.nseg = (uint32_t)plan->nseg;
     LambResident rs;
     rs.cnt = plan->sync;
     rs.ndeferred = plan->sync + (size_t)plan->nseg * kResCntStride;
@@ -874,7 +977,12 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
       with_resident_shape(plan->res_block, plan->res_sub, [&](auto bstag, auto subtag) {
         constexpr int BS = decltype(bstag)::value;
         constexpr int SUB = decltype(subtag)::value;
-        hipLaunchKernelGGL((lamb_resident_kernel<PP, BS, SUB>), dim3(rgrid), dim3(BS), plan->res_lds, s, tbl, P, w, m, v, lay,
+        auto* flat = lamb_resident_kernel<PP, BS, SUB, false>;
+        auto* scat = lamb_resident_kernel<PP, BS, SUB, true>;
+        if (scattered && plan->res_lds > 64 * 1024 &&
+            hipFuncSetAttribute((const void*)scat, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan->res_lds) != hipSuccess)
+          return;   // the launch below then fails and reports
+        hipLaunchKernelGGL(scattered ? scat : flat, dim3(rgrid), dim3(BS), plan->res_lds, s, tbl, P, w, m, v, lay,
                            plan->rpartials, (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
       });
     });
@@ -882,7 +990,8 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
     with_resident_shape(plan->res_block, plan->res_sub, [&](auto bstag, auto subtag) {
       constexpr int BS = decltype(bstag)::value;
       constexpr int SUB = decltype(subtag)::value;
-      hipLaunchKernelGGL((lamb_deferred_kernel<BS, SUB>), dim3(dgrid), dim3(BS), 0, s, w, (const float*)m, (const float*)v,
+      hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<BS, SUB, true> : lamb_deferred_kernel<BS, SUB, false>), dim3(dgrid),
+                         dim3(BS), 0, s, w, (const float*)m, (const float*)v,
                          lay, (const float*)plan->scale, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
                          vec_ok, k);
     });
@@ -896,13 +1005,17 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
     lay.seg_len = vec_ok ? plan->uniform_seg_len : 0;
     lay.seg_len_f = (float)plan->uniform_seg_len;
     lay.tile = kLambTile;
+    lay.gtab = gtab;
+    lay.wtab = wtab;
+    lay.nseg = (uint32_t)plan->nseg;
     // Residency caps measured for N = 2^28, P = 8: pass 1 is fastest at 4 workgroups per CU (its float64 sums and the
     // workgroup reduction need more wavefronts to hide than the plain Adam kernel), pass 2 uncapped.
     const unsigned lds1 = lds_for_residency(P >= 2 ? 4 : 0);
     const unsigned lds2 = 0;
     with_ranks([&](auto ptag) {
       constexpr int PP = decltype(ptag)::value;
-      hipLaunchKernelGGL((lamb_pass1_kernel<PP>), grid, block, lds1, s, table(ptag), P, (const float*)w, m, v, lay,
+      hipLaunchKernelGGL((scattered ? lamb_pass1_kernel<PP, true> : lamb_pass1_kernel<PP, false>), grid, block, lds1, s,
+                         table(ptag), P, (const float*)w, m, v, lay,
                          plan->partials, vec_ok, k);
     });
     CCN_HIP(hipGetLastError());
@@ -918,11 +1031,28 @@ int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, fl
     hipLaunchKernelGGL(lamb_finalize_kernel, dim3((unsigned)plan->nseg), block, 0, s, sums, seg_begin,
                        (const uint64_t*)plan->seg_len, plan->norms, plan->scale, mode);
     CCN_HIP(hipGetLastError());
-    hipLaunchKernelGGL(lamb_pass2_kernel, grid, block, lds2, s, w, (const float*)m, (const float*)v, lay,
+    hipLaunchKernelGGL((scattered ? lamb_pass2_kernel<true> : lamb_pass2_kernel<false>), grid, block, lds2, s, w,
+                       (const float*)m, (const float*)v, lay,
                        (const float*)plan->scale, vec_ok, k);
     CCN_HIP(hipGetLastError());
   }
   return CCN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, float* m, float* v, float lr, float beta1,
+                 float beta2, float eps, float wd, int step, int mode, void* stream) {
+  if (!w) return CCN_EINVAL;
+  return lamb_step(plan, g, P, w, nullptr, m, v, lr, beta1, beta2, eps, wd, step, mode, stream);
+}
+
+int ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v, float lr,
+                           float beta1, float beta2, float eps, float wd, int step, int mode, void* stream) {
+  if (!w) return CCN_EINVAL;
+  return lamb_step(plan, g, P, nullptr, w, m, v, lr, beta1, beta2, eps, wd, step, mode, stream);
 }
 
 int ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream) {

@@ -161,6 +161,12 @@ int  ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** p
 int  ccn_lamb_plan_destroy(ccn_lamb_plan* plan);
 int  ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, float* m, float* v,
                   float lr, float beta1, float beta2, float eps, float wd, int step, int mode, void* stream);
+/* The same step with every segment's gradients and weights in a buffer of their own (the segments of the plan are the
+ * buffers; moments stay in single arrays over the concatenation), as ncclAllReduceScatteredLAMB takes them
+ * (nccl-overlap/src/nccl.h.in:219-221).  g: host array of P*nseg device pointers, rank-major; w: host array of nseg
+ * device pointers.  The plan keeps a device copy of the pointers, refreshed (one stream synchronisation) when they change. */
+int  ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v,
+                            float lr, float beta1, float beta2, float eps, float wd, int step, int mode, void* stream);
 /* copies W_b, R_b of the last ccn_lamb_f32 on this plan to a HOST array of 2*nseg doubles (synchronises) */
 int  ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream);
 

@@ -678,3 +678,40 @@ def test_scattered_adam_and_sgd(ccn, P):
     orc.sgd_f32(g, w2, 0.5)
     assert_f32_parity(np.concatenate([host(x) for x in wd2]), w2, "scattered w after a pointer change")
     plan.close()
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+def test_scattered_lamb(ccn, mode, lamb_variant):
+    """LAMB with every segment's gradients and weights in a buffer of its own (one of them misaligned by 4 bytes in a
+    second run), moments over the concatenation: same results as the oracle on the concatenated arrays."""
+    P = 3
+    counts = [700, 4096 + 5, 1, 30000, 8192]
+    segs = np.concatenate([[0], np.cumsum(counts)]).tolist()
+    N = segs[-1]
+    g = grads_f32(97, P, N, 1e-3)
+    w0 = weights_f32(97, N, 0.05)
+    eps, wd_ = (1e-6, 0.01) if mode == 0 else (0.0, 1.0)
+    for shift in (False, True):
+        def pieces(flat):
+            out = []
+            for b, n in enumerate(counts):
+                lo = segs[b]
+                if shift and b == 3:
+                    out.append(dev(np.concatenate([[np.float32(0)], flat[lo:lo + n]]))[1:])
+                else:
+                    out.append(dev(flat[lo:lo + n]))
+            return out
+        gd, wd = [pieces(x) for x in g], pieces(w0)
+        m0 = weights_f32(98, N, 0.01)
+        v0 = np.abs(weights_f32(99, N, 1e-3)) + np.float32(1e-5)
+        md, vd = dev(m0), dev(v0)
+        w, m, v = w0.copy(), m0.copy(), v0.copy()
+        plan = ccn.LambPlan(segs)
+        for t in (1, 2):
+            plan.step_scattered(gd, wd, md, vd, 1e-3, 0.9, 0.999, eps, wd_, t, mode)
+            orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, eps, wd_, t, mode)
+        plan.close()
+        assert_f32_parity(host(md), m, "scattered lamb m")
+        assert_f32_parity(host(vd), v, "scattered lamb v")
+        got = np.concatenate([host(x) for x in wd])
+        assert np.max(np.abs(got.astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
