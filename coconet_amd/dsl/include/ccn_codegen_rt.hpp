@@ -82,6 +82,22 @@ template <int VEC> __device__ __forceinline__ Vals<VEC> load_vals(const uint16_t
 __device__ __forceinline__ float load_one(const float* p) { return *p; }
 __device__ __forceinline__ float load_one(const uint16_t* p) { return f16_bits_to_f32(*p); }
 
+__host__ __device__ inline uint16_t f32_to_f16_bits(float f) {
+  const _Float16 x = (_Float16)f;
+  uint16_t h;
+  memcpy(&h, &x, 2);
+  return h;
+}
+template <int VEC> __device__ __forceinline__ void store_vals(uint16_t* p, const Vals<VEC>& v) {
+  if constexpr (VEC == 1) {
+    __builtin_nontemporal_store(f32_to_f16_bits(v.d[0]), p);
+  } else {
+    u32x2 x;
+    x[0] = (unsigned)f32_to_f16_bits(v.d[0]) | ((unsigned)f32_to_f16_bits(v.d[1]) << 16);
+    x[1] = (unsigned)f32_to_f16_bits(v.d[2]) | ((unsigned)f32_to_f16_bits(v.d[3]) << 16);
+    __builtin_nontemporal_store(x, reinterpret_cast<u32x2*>(p));
+  }
+}
 template <int VEC> __device__ __forceinline__ void store_vals(float* p, const Vals<VEC>& v) {
   if constexpr (VEC == 1) {
     __builtin_nontemporal_store(v.d[0], p);
@@ -139,7 +155,8 @@ template <int BS = kBlock> __device__ __forceinline__ double block_sum(double x,
 // ---- kernel arguments ---------------------------------------------------------------------------------------------
 // A generated Body declares:
 //   NIN        plain fp32 input arrays, read at the element index
-//   NOUT       fp32 output arrays (an in-place update lists the array under both)
+//   NOUT       output arrays (an in-place update lists the array under both); fp32, except those whose bit is set
+//   OUT_F16    in this mask: they hold fp16 (the body has already rounded the value to fp16, the store narrows it)
 //   HAS_RED    the body's first operand is the sum over rank buffers (the lowered AllReduce / ReduceScatter)
 //   RedT       element type of those buffers: float, or uint16_t holding fp16 bits (widened, then summed in fp32)
 //   NACC       sums of squares the body accumulates (inputs of Norm stages), float64
@@ -150,7 +167,7 @@ template <class Body> struct KernelArgs {
   const typename Body::RedT* red[kMaxRanks];
   int nranks;
   const float* in[Body::NIN > 0 ? Body::NIN : 1];
-  float* out[Body::NOUT > 0 ? Body::NOUT : 1];
+  void* out[Body::NOUT > 0 ? Body::NOUT : 1];
   double* partials;      // NACC values per workgroup
   const float* norms;    // NNORM values
   size_t n;
@@ -210,7 +227,10 @@ __global__ __launch_bounds__(BS) void fused_pointwise_kernel(const KernelArgs<Bo
       for (int k = 0; k < Body::NOUT; k++) ov[k].d[e] = out1[k];
     }
 #pragma unroll
-    for (int k = 0; k < Body::NOUT; k++) store_vals<VEC>(a.out[k] + e0, ov[k]);
+    for (int k = 0; k < Body::NOUT; k++) {
+      if ((Body::OUT_F16 >> k) & 1u) store_vals<VEC>(static_cast<uint16_t*>(a.out[k]) + e0, ov[k]);
+      else store_vals<VEC>(static_cast<float*>(a.out[k]) + e0, ov[k]);
+    }
   }
 
   if constexpr (VEC > 1) {   // the last n % VEC elements, scalar, by the first lanes of workgroup 0
@@ -225,7 +245,10 @@ __global__ __launch_bounds__(BS) void fused_pointwise_kernel(const KernelArgs<Bo
       float in1[NINX], out1[NOUTX];
       for (int k = 0; k < Body::NIN; k++) in1[k] = a.in[k][i];
       Body::apply(red, in1, out1, a.s, acc, nrm, (uint64_t)i);
-      for (int k = 0; k < Body::NOUT; k++) a.out[k][i] = out1[k];
+      for (int k = 0; k < Body::NOUT; k++) {
+        if ((Body::OUT_F16 >> k) & 1u) static_cast<uint16_t*>(a.out[k])[i] = f32_to_f16_bits(out1[k]);
+        else static_cast<float*>(a.out[k])[i] = out1[k];
+      }
     }
   }
 
@@ -328,7 +351,8 @@ template <class Body> unsigned launch(const KernelArgs<Body>& a, void* stream) {
   if (Body::HAS_RED)   // a pack of four is 16 bytes of fp32 or 8 bytes of fp16
     for (int p = 0; p < a.nranks; p++) al = al && ((uintptr_t)a.red[p] & (4 * sizeof(typename Body::RedT) - 1)) == 0;
   for (int k = 0; k < Body::NIN; k++) al = al && aligned16(a.in[k]);
-  for (int k = 0; k < Body::NOUT; k++) al = al && aligned16(a.out[k]);
+  for (int k = 0; k < Body::NOUT; k++)   // a pack of four is 16 bytes of fp32 or 8 bytes of fp16
+    al = al && ((uintptr_t)a.out[k] & (((Body::OUT_F16 >> k) & 1u) ? 7u : 15u)) == 0;
   if (al) return launch_vec<Body, 4>(a, (hipStream_t)stream);
   return launch_vec<Body, 1>(a, (hipStream_t)stream);
 }
@@ -407,6 +431,20 @@ inline bool compare(const char* what, const std::vector<float>& ref, const float
   for (size_t i = 0; i < n; i++) {
     if (!eqFloat(ref[i], got[i], tol)) {
       printf("Mismatch in %s at %zu : ref '%.9g', computed '%.9g'\n", what, i, ref[i], got[i]);
+      return false;
+    }
+  }
+  return true;
+}
+
+// fp16 outputs: widened and compared like fp32 ones
+inline bool compare(const char* what, const std::vector<float>& ref, const uint16_t* dev, size_t n, float tol = 1e-5f) {
+  std::vector<uint16_t> got(n);
+  CCNCHECK(ccn_memcpy_d2h(got.data(), dev, n * sizeof(uint16_t), nullptr));
+  for (size_t i = 0; i < n; i++) {
+    const float x = f16_bits_to_f32(got[i]);
+    if (!eqFloat(ref[i], x, tol)) {
+      printf("Mismatch in %s at %zu : ref '%.9g', computed '%.9g'\n", what, i, ref[i], x);
       return false;
     }
   }

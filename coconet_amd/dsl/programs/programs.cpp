@@ -74,7 +74,8 @@ static void adam(bool fused, const std::string& out) {
 }
 
 // The pipeline behind the reference's examples/test-adamf16.cu: fp16 gradients, fp32 state, the DSL example's
-// "Adam" (divide by beta, no square root), all in one kernel.  A Float16 tensor can only be reduced inside a fused kernel.
+// "Adam" (divide by beta, no square root) and an fp16 copy of the new weights, all in one kernel.  A Float16 tensor can
+// only be reduced inside a fused kernel.
 static void adamf16(bool fused, const std::string& out) {
   ASSERT(fused, "adamf16 has a fused schedule only");
   Variable N(Int32, "N");
@@ -87,8 +88,10 @@ static void adamf16(bool fused, const std::string& out) {
   Stage mn = Update(m, b1 * m + (1 - b1) * gs);
   Stage mh = mn / b1;
   Stage wn = Update(w, w - (lr * mh) / vh);
-  Pipeline pl("adamf16", {g, w, m, v, lr, b1, b2}, {mn, vn, wn});
-  pl.fuse({gs, vn, vh, mn, mh, wn});
+  Tensor hw(Float16, N, Replicated, "halfw");            // the fp16 copy of the weights the reference's kernel also writes
+  Stage hwn = Update(hw, Cast(Float16, wn));
+  Pipeline pl("adamf16", {g, w, hw, m, v, lr, b1, b2}, {mn, vn, wn, hwn});
+  pl.fuse({gs, vn, vh, mn, mh, wn, hwn});
   pl.codegen(out);
 }
 

@@ -109,6 +109,7 @@ struct Body {
   std::vector<std::string> code;         // statements
   int nacc = 0, nnorm = 0;
   unsigned sqrtMask = 0;                 // accumulator k finishes as sqrt(sum) (a norm) rather than as the sum
+  unsigned outHalfMask = 0;              // output array k holds fp16
   std::set<std::string> scalars;         // variable names used
   bool usesSeed = false;
 };
@@ -203,13 +204,14 @@ struct BodyBuilder {
     return "";
   }
 
-  void store(const std::string& array, const std::string& value) {
+  void store(const std::string& array, const std::string& value, bool half = false) {
     for (size_t k = 0; k < body.outArrays.size(); k++) {
       if (body.outArrays[k] == array) {
         body.code.push_back("out[" + std::to_string(k) + "] = " + value + ";");
         return;
       }
     }
+    if (half) body.outHalfMask |= 1u << body.outArrays.size();
     body.outArrays.push_back(array);
     body.code.push_back("out[" + std::to_string(body.outArrays.size() - 1) + "] = " + value + ";");
   }
@@ -233,11 +235,12 @@ struct BodyBuilder {
     }
     if (def->kind == Kind::Update) {
       const NodePtr& t = def->args[0];
-      const std::string x = emit(def->args[1]);
+      std::string x = emit(def->args[1]);
+      if (t->elem == Float16) x = "((float)(_Float16)(" + x + "))";   // the value the fp16 array will hold
       body.code.push_back("const float " + v + " = " + x + ";");
       tensorValue[t.get()] = v;
       stageValue[k] = v;
-      if (withStores) store(t->name, v);
+      if (withStores) store(t->name, v, t->elem == Float16);
       return;
     }
     const std::string x = emit(def);
@@ -254,6 +257,7 @@ std::string body_text(const Body& b, const std::vector<NodePtr>& scalarVars) {
     << ", NNORM = " << b.nnorm << ";\n";
   o << "  static constexpr bool HAS_RED = " << (b.hasRed ? "true" : "false") << ";\n";
   o << "  using RedT = " << (b.redHalf ? "uint16_t" : "float") << ";\n";
+  o << "  static constexpr unsigned OUT_F16 = " << b.outHalfMask << "u;\n";
   o << "  struct Scalars {";
   for (auto& v : scalarVars) o << " " << elem_c_type(v->elem) << " " << v->name << ";";
   o << " uint64_t seed__; };\n";
@@ -306,10 +310,16 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
              "variable '" << v->name << "' is used but is not a pipeline argument");
     find_reduced(st->args[0], prog.reducedTensors);
   }
-  // fp32 everywhere, except that a gradient tensor folded over the ranks may hold fp16 (widened on load, summed in fp32)
+  // fp32 everywhere, with two exceptions: a gradient tensor folded over the ranks may hold fp16 (widened on load, summed
+  // in fp32), and so may a tensor that stages only write (Update targets such as an fp16 copy of the weights; reading
+  // one is refused where the read would be emitted)
+  std::set<const Node*> updateTargets;
+  for (auto& st : p.stages())
+    if (st->args[0]->kind == Kind::Update) updateTargets.insert(st->args[0]->args[0].get());
   for (auto& t : prog.tensors)
-    ASSERT(t->elem == Float32 || (t->elem == Float16 && prog.reducedTensors.count(t.get())),
-           "HIP target: tensor '" << t->name << "' must be Float32 (Float16 only for a tensor read through AllReduce/ReduceScatter)");
+    ASSERT(t->elem == Float32 || (t->elem == Float16 && (prog.reducedTensors.count(t.get()) || updateTargets.count(t.get()))),
+           "HIP target: tensor '" << t->name << "' must be Float32 (Float16 only for a tensor read through AllReduce/"
+           "ReduceScatter or written by Update)");
 
   const auto groups = p.groupsInOrder();
   const std::string fn = [&] { std::string s = p.name(); for (auto& c : s) if (!isalnum((unsigned char)c)) c = '_'; return s; }();
@@ -457,7 +467,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
     for (auto& d : prog.dimVars) add("size_t", d->name);
     for (auto& v : prog.scalarVars) add(elem_c_type(v->elem), v->name);
     for (auto& t : prog.tensors)
-      add(prog.reducedTensors.count(t.get()) ? (t->elem == Float16 ? "uint16_t* const*" : "float* const*") : "float*", t->name);
+      add(prog.reducedTensors.count(t.get()) ? (t->elem == Float16 ? "uint16_t* const*" : "float* const*")
+                                             : (t->elem == Float16 ? "uint16_t*" : "float*"), t->name);
     for (int k : prog.ownBuffers) add("float*", p.stages()[k]->name);
     add("double*", "partials__");
     add("float*", "norms__");
@@ -590,7 +601,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
       o << "  h." << st->name << ".resize(" << cnt << ");\n";
       o << "  for (size_t i0 = 0; i0 < " << cnt << "; i0++) {\n";
       if (def->kind == Kind::Update) {
-        o << "    h." << st->name << "[i0] = " << he(def->args[1]) << ";\n";
+        if (def->args[0]->elem == Float16) o << "    h." << st->name << "[i0] = (float)(_Float16)(" << he(def->args[1]) << ");\n";
+        else o << "    h." << st->name << "[i0] = " << he(def->args[1]) << ";\n";
         o << "    h." << def->args[0]->name << "[i0] = h." << st->name << "[i0];\n";
       } else {
         o << "    h." << st->name << "[i0] = " << he(def) << ";\n";
@@ -645,10 +657,11 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
         << t->name << "[p_] : nullptr);\n" << ind << "}\n";
       seedNo += 100;
     } else {
-      o << ind << "float* " << t->name << ";\n";
+      const bool half = t->elem == Float16;
+      o << ind << (half ? "uint16_t* " : "float* ") << t->name << ";\n";
       o << ind << "std::vector<float> h_" << t->name << ";\n";
-      o << ind << "CCNCHECK(ccn_malloc((void**)&" << t->name << ", (" << cnt << ") * sizeof(float)));\n";
-      o << ind << "ccn_gen::fill_uniform(" << t->name << ", " << cnt << ", seed__ + " << (++seedNo) << ", check__ ? &h_" << t->name
+      o << ind << "CCNCHECK(ccn_malloc((void**)&" << t->name << ", (" << cnt << ") * sizeof(" << (half ? "uint16_t" : "float") << ")));\n";
+      o << ind << "ccn_gen::fill_uniform" << (half ? "_f16" : "") << "(" << t->name << ", " << cnt << ", seed__ + " << (++seedNo) << ", check__ ? &h_" << t->name
         << " : nullptr);\n";
     }
   }

@@ -129,6 +129,9 @@ def test_fp16_gradients_are_widened_inside_the_fused_kernel(dsl_build, tmp_path)
     text = out.read_text()
     assert "using RedT = uint16_t;" in text and "uint16_t* const* g" in text and "fill_uniform_f16(g[p_]" in text
     assert "sizeof(uint16_t)" in text
+    # the fp16 copy of the weights: an Update target of type Float16 is stored as halves, output slot 3 of the body
+    assert "static constexpr unsigned OUT_F16 = 8u;" in text and "uint16_t* halfw" in text
+    assert 'compare("halfw", h.halfw, halfw' in text
     r = run(exe, "adamf16", "unfused", str(tmp_path / "x.hip"))
     assert r.returncode != 0 and "fused schedule only" in r.stderr
 
