@@ -71,8 +71,9 @@ const char* ccn_strerror(int code);
  *      ccn_stream_create, not the null stream) are recorded instead of run; ccn_graph_launch replays the recording.
  *      Recorded calls keep the arguments they were made with (pointers, sizes, and `step`, which is evaluated on the
  *      host: a recording of Adam or LAMB steps replays the same bias corrections).  Not recordable: ccn_malloc/free,
- *      the memcpy and sync calls, ccn_lamb_plan_create/norms, and the first ccn_lamb_f32 call of a plan for a given
- *      rank count (it queries occupancy; make one call before recording). ---- */
+ *      the memcpy and sync calls, ccn_lamb_plan_create/norms, the first ccn_lamb_f32 call of a plan for a given
+ *      rank count (it queries occupancy; make one call before recording), and a *_scattered call whose buffer
+ *      pointers differ from the previous call's (it refreshes the plan's device table and waits for the copy). ---- */
 typedef struct ccn_graph ccn_graph;
 int  ccn_graph_begin(void* stream);
 int  ccn_graph_end(void* stream, ccn_graph** graph);
