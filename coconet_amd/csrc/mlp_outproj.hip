@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
                                                              const SrcTable<float, 8> parts,
                                                              const float* __restrict__ bias,
                                                              const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
-                                                             const int M, const int N, const int K, const EpiPrm ep) {
+                                                             const int N, const int K, const EpiPrm ep) {
   // main loop: X tile [m][k] and transposed W tile [n][k], 16 KiB each, chunk-swizzled.
   // epilogue: half of the fp32 C tile, 64 rows x (128 + 4 pad) floats, to turn the MFMA register layout
   // into whole 512-byte row segments per wavefront.
@@ -274,7 +274,7 @@ int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* cons
   hipStream_t s = as_stream(stream);
   switch (nPartials) {
 #define CCN_CASE(Q) \
-  case Q: hipLaunchKernelGGL((mlp_outproj_kernel<Q>), grid, block, 0, s, X, W, tbl, bias, resid, out, M, N, K, ep); break;
+  case Q: hipLaunchKernelGGL((mlp_outproj_kernel<Q>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); break;
     CCN_CASE(0) CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
 #undef CCN_CASE
   }
