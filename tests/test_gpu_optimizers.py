@@ -715,3 +715,17 @@ def test_scattered_lamb(ccn, mode, lamb_variant):
         assert_f32_parity(host(vd), v, "scattered lamb v")
         got = np.concatenate([host(x) for x in wd])
         assert np.max(np.abs(got.astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
+
+
+@pytest.mark.parametrize("which,ranks", [("adam", 2), ("adam", 8), ("lamb", 2), ("lamb", 3)])
+def test_cpp_harness_in_the_shape_of_the_reference_sample(which, ranks):
+    """tests/harness/adam_lamb_scattered.cpp: the flow of the reference's multi-process-adam-scattered.cpp (its buffer
+    list, integer inputs, five checked epochs, its comparator) through the scattered entry points, from C++."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "harness", "build", "adam_lamb_scattered")
+    if not os.path.exists(exe):
+        pytest.skip("harness not built (make -C tests/harness)")
+    r = subprocess.run([exe, which, str(ranks)], capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0 and "Success" in r.stdout, (r.stdout[-1500:], r.stderr[-500:])
+    assert r.stdout.count("weights match the checker") == 5
