@@ -32,7 +32,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adam_f32",
-                    choices=["adam_f32", "adam_f32_scattered", "sgd_f32", "adam_f16g", "lamb_f32", "mlp_outproj", "copy"])
+                    choices=["adam_f32", "adam_f32_scattered", "sgd_f32", "adam_f16g", "adam_bf16g", "lamb_f32",
+                             "mlp_outproj", "copy"])
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -168,15 +169,17 @@ def main():
         units = N
         config = {"workload": f"adam_f32 over {nbuff} scattered buffers, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,
                   "algorithmic_bytes_per_param": per_param, "allocator": a.allocator}
-    elif wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g"):
+    elif wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g", "adam_bf16g"):
         P = a.ranks or (4 if wl == "sgd_f32" else 8)
         N = 1 << (a.log2n or (20 if wl == "sgd_f32" else 28))
-        gbytes = 2 if wl == "adam_f16g" else 4
+        gbytes = 2 if wl in ("adam_f16g", "adam_bf16g") else 4
+        half = torch.bfloat16 if wl == "adam_bf16g" else torch.float16
+        gscale = 2.0 ** 7 if wl == "adam_bf16g" else 2.0 ** 16
         bufs = Buffers(capi, torch, a.allocator == "torch")
         g = []
         for p in range(P):
             if gbytes == 2:
-                t = (torch.randn(N, device="cuda", generator=gen) * (1e-3 * 65536.0)).to(torch.float16)
+                t = (torch.randn(N, device="cuda", generator=gen) * (1e-3 * gscale)).to(half)
                 if p == 0:
                     t[::1 << 20] = float("inf")        # benchmark configuration 3: one entry in 2^20 overflows
             else:
@@ -194,12 +197,14 @@ def main():
             per_param = (P + 1) * 4 + 4
             step = lambda t: capi.sgd_f32(g, w, N, 0.01, stream)
             kernel = "fused_stream_kernel<SgdMath, %d, 4, 1, %d>" % (P if P <= 8 else 0, 256 if P + 2 <= 3 else 64)
-        elif wl == "adam_f16g":
-            w16 = bufs.from_tensor(torch.empty(N, dtype=torch.float16, device="cuda"))
+        elif gbytes == 2:
+            w16 = bufs.from_tensor(torch.empty(N, dtype=half, device="cuda"))
             flag = torch.zeros(1, dtype=torch.int32, device="cuda")
             per_param = P * 2 + 12 + 12 + 2
-            step = lambda t: capi.adam_f16g(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, t, 2.0 ** -16, flag, stream)
-            kernel = "fused_stream_kernel<Adam16Math, %d, 4, 1, 64>" % (P if P <= 8 else 0)
+            call = capi.adam_bf16g if wl == "adam_bf16g" else capi.adam_f16g
+            step = lambda t: call(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, t, 1.0 / gscale, flag, stream)
+            kernel = "fused_stream_kernel<Adam16MathT<%s>, %d, 4, 1, 64>" % ("true" if wl == "adam_bf16g" else "false",
+                                                                             P if P <= 8 else 0)
         else:
             nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
             plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
@@ -269,7 +274,8 @@ def main():
         "metric": METRIC if wl == "adam_f32" else f"{wl} algorithmic GB/s",
         "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"adam_f16g": "f16 gradients, f32 state", "mlp_outproj": "bf16 x bf16 -> f32"}.get(wl, "f32"),
+        "dtype": {"adam_f16g": "f16 gradients, f32 state", "adam_bf16g": "bf16 gradients, f32 state",
+                  "mlp_outproj": "bf16 x bf16 -> f32"}.get(wl, "f32"),
         "data": "synthetic", "config": config,
         "params_per_s": round(units / (wall_ms * 1e-3), 1),
         "device": info,

@@ -33,7 +33,7 @@ SYMBOLS = [
     "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
     "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
     "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
-    "ccn_lamb_f32_scattered",
+    "ccn_lamb_f32_scattered", "ccn_adam_bf16g",
 ]
 
 
@@ -92,6 +92,7 @@ def _declare(L):
     sig("ccn_pseudo_adam_f32", [_pp, _i, _vp, _vp, _vp, _sz, _f, _f, _f, _vp])
     sig("ccn_adam_f32", [_pp, _i, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _vp])
     sig("ccn_adam_f16g", [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _f, _vp, _vp])
+    sig("ccn_adam_bf16g", [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _f, _vp, _vp])
     sig("ccn_overflow_check_f16", [_pp, _i, _sz, _vp, _vp])
     sig("ccn_fused_adam_ref_f16g", [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _vp])
     sig("ccn_lamb_plan_create", [C.POINTER(_sz), _i, _pp])
@@ -316,6 +317,12 @@ def adam_f16g(g, w, m, v, w16, n, lr, beta1, beta2, eps, step, inv_scale, overfl
     p, _keep = ptr_table(g)
     _check(load().ccn_adam_f16g(p, len(g), addr(w), addr(m), addr(v), addr(w16), n, lr, beta1, beta2, eps, step,
                                 inv_scale, addr(overflow_flag), stream), "ccn_adam_f16g")
+
+
+def adam_bf16g(g, w, m, v, w16, n, lr, beta1, beta2, eps, step, inv_scale, overflow_flag, stream=None):
+    p, _keep = ptr_table(g)
+    _check(load().ccn_adam_bf16g(p, len(g), addr(w), addr(m), addr(v), addr(w16), n, lr, beta1, beta2, eps, step,
+                                 inv_scale, addr(overflow_flag), stream), "ccn_adam_bf16g")
 
 
 def overflow_check_f16(g, n, overflow_flag, stream=None):

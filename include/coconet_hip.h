@@ -137,6 +137,11 @@ int  ccn_adam_f32_scattered(ccn_scatter_plan* plan, const float* const* g, int P
 int  ccn_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16, size_t N,
                    float lr, float beta1, float beta2, float eps, int step, float inv_scale,
                    uint32_t* overflow_flag, void* stream);
+/* The same step with bfloat16 gradients and a bfloat16 copy of the weights (overflow = exponent 0xFF).  No counterpart in
+ * the reference, whose mixed-precision path is fp16 only; same contract as ccn_adam_f16g otherwise. */
+int  ccn_adam_bf16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16,
+                    size_t N, float lr, float beta1, float beta2, float eps, int step, float inv_scale,
+                    uint32_t* overflow_flag, void* stream);
 
 /* ---- overflow pre-check for callers that want all-or-nothing steps: *overflow_flag <- any(!isfinite(g)). ---- */
 int  ccn_overflow_check_f16(const uint16_t* const* g, int P, size_t N, uint32_t* overflow_flag, void* stream);

@@ -71,6 +71,8 @@ def _declare(L):
     L.orc_adam_f32.argtypes = [_pp, _i, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i]
     L.orc_adam_f16g.restype = C.c_uint32
     L.orc_adam_f16g.argtypes = [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _f]
+    L.orc_adam_bf16g.restype = C.c_uint32
+    L.orc_adam_bf16g.argtypes = [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _f]
     L.orc_overflow_f16.restype = C.c_uint32
     L.orc_overflow_f16.argtypes = [_pp, _i, _sz]
     L.orc_lamb_f32.restype = None
@@ -179,6 +181,12 @@ def adam_f16g(g16, w, m, v, w16, lr, beta1, beta2, eps, step, inv_scale):
     p, _k = _ptrs(g16, u16)
     return int(lib().orc_adam_f16g(p, len(g16), _ptr(w, f32), _ptr(m, f32), _ptr(v, f32), _ptr(w16, u16), w.size,
                                    lr, beta1, beta2, eps, step, inv_scale))
+
+
+def adam_bf16g(g16, w, m, v, w16, lr, beta1, beta2, eps, step, inv_scale):
+    p, _k = _ptrs(g16, u16)
+    return int(lib().orc_adam_bf16g(p, len(g16), _ptr(w, f32), _ptr(m, f32), _ptr(v, f32), _ptr(w16, u16), w.size,
+                                    lr, beta1, beta2, eps, step, inv_scale))
 
 
 def overflow_f16(g16):

@@ -237,6 +237,40 @@ uint32_t orc_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, floa
   return flag;
 }
 
+/* The same step with bfloat16 gradients and a bfloat16 copy of the weights (no counterpart in the reference, which has
+ * fp16 only): overflow = exponent 0xFF; conversions round to nearest even. */
+uint32_t orc_adam_bf16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16,
+                        size_t N, float lr, float beta1, float beta2, float eps, int step, float inv_scale) {
+  const double bc1 = 1 - pow((double)beta1, (double)step);
+  const double bc2 = 1 - pow((double)beta2, (double)step);
+  const float stepsize = -lr;
+  uint32_t flag = 0;
+  for (size_t i = 0; i < N; i++) {
+    int bad = 0;
+    float gs = 0.0f;
+    for (int p = 0; p < P; p++) {
+      uint16_t h = g[p][i];
+      if ((h & 0x7f80u) == 0x7f80u) bad = 1;
+      float t = orc_bf16_to_f32(h) * inv_scale;
+      gs = (p == 0) ? t : gs + t;
+    }
+    if (bad) {
+      flag = 1;
+    } else {
+      float mi = beta1 * m[i] + (1 - beta1) * gs;
+      float vi = beta2 * v[i] + (1 - beta2) * gs * gs;
+      float m_ = (float)((double)mi / bc1);
+      float v_ = (float)((double)vi / bc2);
+      float x = stepsize * m_ / (sqrtf(v_) + eps);
+      w[i] = w[i] + x;
+      m[i] = mi;
+      v[i] = vi;
+    }
+    w16[i] = orc_f32_to_bf16(w[i]);
+  }
+  return flag;
+}
+
 uint32_t orc_overflow_f16(const uint16_t* const* g, int P, size_t N) {
   for (int p = 0; p < P; p++)
     for (size_t i = 0; i < N; i++)

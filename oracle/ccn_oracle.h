@@ -24,8 +24,8 @@
  *   orc_lamb_f32          same file :402-449; single-segment/w==0 special cases, float64 brute force  pinned
  *                         (mode 2: nccl/.../reduce_kernel.h:391-452; all-ones closed form, float64 brute force;
  *                          the reference sums its norms in fp32 in no fixed order: norm rounding parity unpinned)
- *   orc_adam_f16g         no counterpart in the reference (it has no loss scaling / overflow detection):
- *                         build-defined, pinned by closed forms only; parity with Apex "parity unpinned"
+ *   orc_adam_f16g,        no counterpart in the reference (it has no loss scaling / overflow detection, and no bfloat16):
+ *   orc_adam_bf16g        build-defined, pinned by closed forms only; parity with Apex "parity unpinned"
  *   orc_philox4x32_10     Random123 known-answer vectors                         pinned
  *   orc_mlp_outproj       no reference test beyond the all-ones C == K check
  *                         (nccl-overlap/samples/matmul-allreduce-bias-dropout-layernorm.cu:520-526);
@@ -77,6 +77,8 @@ void orc_adam_f32(const float* const* g, int P, float* w, float* m, float* v, si
 /* returns the overflow flag (0/1) */
 uint32_t orc_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16,
                        size_t N, float lr, float beta1, float beta2, float eps, int step, float inv_scale);
+uint32_t orc_adam_bf16g(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* w16,
+                        size_t N, float lr, float beta1, float beta2, float eps, int step, float inv_scale);
 uint32_t orc_overflow_f16(const uint16_t* const* g, int P, size_t N);
 
 /* ---- LAMB with per-segment norms.  seg_offsets has nseg+1 entries, seg_offsets[nseg] == N.

@@ -272,6 +272,36 @@ def test_mixed_precision_adam(ccn, P, N, plant):
     assert int(host(flag)[0]) == orc.overflow_f16(g16)
 
 
+@pytest.mark.parametrize("P,N,plant,log2scale", [(8, 1 << 20, 0, 7), (8, 100003, 4, 7), (3, 8, 1, 7), (9, 4099, 2, 7),
+                                                 (1, 1, 1, 7), (8, 65539, 0, 131)])
+def test_mixed_precision_adam_bf16(ccn, P, N, plant, log2scale):
+    """bfloat16 gradients and weight copy; overflow = exponent 0xFF.  At scale 2^131 the finite gradients sit near
+    2^121, where their bits read as fp16 would be inf/nan patterns: the flag must stay 0."""
+    inv = float(np.float32(2.0 ** -min(log2scale, 120)))      # kept a normal number
+    g16 = [orc.f32_to_bf16(x * np.float32(2.0 ** (log2scale - 31)) * np.float32(2.0 ** 31))
+           for x in grads_f32(23, P, N, 1e-3)]
+    r = rng(23, 77)
+    for _ in range(plant):
+        g16[int(r.integers(0, P))][int(r.integers(0, N))] = [0x7F80, 0xFF80, 0x7FC0][int(r.integers(0, 3))]
+    if log2scale > 100:
+        assert any(((x & 0x7C00) == 0x7C00).any() for x in g16)
+        assert all(np.isfinite(orc.bf16_to_f32(x)).all() for x in g16)
+    w0 = weights_f32(23, N, 0.05)
+    wd, md, vd = dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w16d = torch.zeros(N, dtype=torch.int16, device=DEV)
+    flag = torch.full((1,), 123, dtype=torch.int32, device=DEV)
+    gd = [dev_u16(x) for x in g16]
+    w, m, v, w16 = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros(N, np.uint16)
+    for t in (1, 2):
+        ccn.adam_bf16g(gd, wd, md, vd, w16d, N, 1e-3, 0.9, 0.999, 1e-6, t, inv, flag)
+        want = orc.adam_bf16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, t, np.float32(inv))
+        assert int(host(flag)[0]) == want == (1 if plant else 0)
+    assert_f32_parity(host(wd), w, "bf16 w")
+    assert_f32_parity(host(md), m, "bf16 m")
+    assert_f32_parity(host(vd), v, "bf16 v")
+    assert np.array_equal(host_u16(w16d), w16)
+
+
 def test_mixed_precision_full_size_flag_and_skips(ccn):
     """benchmark configuration 3 at full size: one in 2^20 entries forced to inf.  Checked through properties:
     flag == 1, exactly the planted elements keep their state, fp16 copy == fp16(w) everywhere."""

@@ -431,3 +431,49 @@ def test_lamb_nccl_global_float64_brute_force():
     expect = w0 - lr * (W / R / R) * r
     assert np.max(np.abs(w - expect)) < 1e-6 * np.max(np.abs(expect))
     assert np.max(np.abs(m - mm)) < 1e-6 * np.max(np.abs(mm)) and np.max(np.abs(v - vv)) < 1e-6 * np.max(np.abs(vv))
+
+
+def test_adam_bf16g_reduces_to_adam_and_flags():
+    """bfloat16 gradients: same pins as the fp16 variant, with torch's bfloat16 cast as the independent conversion."""
+    import torch
+    P, N = 8, 1 << 13
+    scale = 2.0 ** 7
+    g32 = grads_f32(10, P, N, 1e-3)
+    g16 = [orc.f32_to_bf16(x * np.float32(scale)) for x in g32]
+    for x32, x16 in zip(g32, g16):
+        t = (torch.from_numpy(x32) * scale).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(x16, t)
+    w0 = weights_f32(10, N, 0.05)
+    w, m, v, w16 = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32), np.zeros(N, np.uint16)
+    flag = orc.adam_bf16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, 1, np.float32(1 / scale))
+    dec = [orc.bf16_to_f32(x) * np.float32(1 / scale) for x in g16]
+    wr, mr, vr = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    orc.adam_f32(dec, wr, mr, vr, 1e-3, 0.9, 0.999, 1e-6, 1)
+    assert flag == 0
+    assert np.array_equal(w, wr) and np.array_equal(m, mr) and np.array_equal(v, vr)
+    want16 = torch.from_numpy(w).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(w16, want16)
+    # finite values near 2^121, whose bits read as fp16 would be inf/nan patterns, are not overflows
+    big = [orc.f32_to_bf16(x * np.float32(2.0 ** 100) * np.float32(2.0 ** 31)) for x in g32]
+    assert all(np.isfinite(orc.bf16_to_f32(x)).all() for x in big)
+    assert any(((x & 0x7C00) == 0x7C00).any() for x in big)
+    wb, mb, vb = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    assert orc.adam_bf16g(big, wb, mb, vb, w16, 1e-3, 0.9, 0.999, 1e-6, 1, np.float32(2.0 ** -120)) == 0
+    assert np.isfinite(vb).all() and (mb != 0).any()
+    # +inf, -inf and a nan
+    bad = {17: (0, 0x7F80), 4096: (3, 0xFF80), N - 1: (7, 0x7FC1)}
+    for i, (p, bits) in bad.items():
+        g16[p][i] = bits
+    dec = [orc.bf16_to_f32(x) * np.float32(1 / scale) for x in g16]
+    for i, (p, _) in bad.items():
+        dec[p][i] = 0
+    wr, mr, vr = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    orc.adam_f32(dec, wr, mr, vr, 1e-3, 0.9, 0.999, 1e-6, 1)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    flag = orc.adam_bf16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, 1, np.float32(1 / scale))
+    assert flag == 1
+    keep = np.ones(N, bool)
+    keep[list(bad)] = False
+    assert np.array_equal(w[keep], wr[keep]) and np.array_equal(m[keep], mr[keep]) and np.array_equal(v[keep], vr[keep])
+    assert np.array_equal(w[~keep], w0[~keep]) and np.all(m[~keep] == 0) and np.all(v[~keep] == 0)
+    assert np.all(np.isfinite(w)) and np.isfinite(m).all() and np.isfinite(v).all()
