@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+
+#include <new>
 #include "coconet_hip.h"
 
 namespace ccn {
@@ -19,6 +21,19 @@ int hip_fail(hipError_t e);                        // records e, returns the CCN
     hipError_t _e = (expr);                                                \
     if (_e != hipSuccess) return ::ccn::hip_fail(_e);                      \
   } while (0)
+
+// Runs a host-side body that may allocate host memory (std::vector, std::unordered_map) and turns what it could throw
+// into an error code: no exception leaves an extern "C" entry point.
+template <class Body>
+int guarded(Body&& body) noexcept {
+  try {
+    return body();
+  } catch (const std::bad_alloc&) {
+    return CCN_ENOMEM;
+  } catch (...) {
+    return CCN_EINVAL;
+  }
+}
 
 struct DeviceInfo {
   int device = -1;

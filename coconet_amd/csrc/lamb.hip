@@ -720,10 +720,7 @@ int ccn_lamb_plan_destroy(ccn_lamb_plan* plan) {
   return rc;
 }
 
-int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** out) {
-  if (!out) return CCN_EINVAL;
-  *out = nullptr;
-  if (!seg_offsets || nseg < 1 || seg_offsets[0] != 0) return CCN_EINVAL;
+static int lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** out) {
   for (int b = 0; b < nseg; b++) {
     if (seg_offsets[b + 1] <= seg_offsets[b]) return CCN_EINVAL;   // empty or descending segment
   }
@@ -806,6 +803,10 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
 
   ccn_lamb_plan* p = new (std::nothrow) ccn_lamb_plan();
   if (!p) return CCN_ENOMEM;
+  struct Owner {   // frees the half-built plan on every early exit, a throwing std::vector included
+    ccn_lamb_plan* p;
+    ~Owner() { if (p) ccn_lamb_plan_destroy(p); }
+  } owner{p};
   p->device = di->device;
   p->nseg = nseg;
   p->N = seg_offsets[nseg];
@@ -849,12 +850,17 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   }
   upload(p->rtiles, rtiles.data(), rtiles.size() * sizeof(LambTile));
   upload(p->seg_rtile_begin, rbegin.data(), rbegin.size() * sizeof(uint32_t));
-  if (e != hipSuccess) {
-    ccn_lamb_plan_destroy(p);
-    return hip_fail(e);
-  }
+  if (e != hipSuccess) return hip_fail(e);
+  owner.p = nullptr;
   *out = p;
   return CCN_OK;
+}
+
+int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** out) {
+  if (!out) return CCN_EINVAL;
+  *out = nullptr;
+  if (!seg_offsets || nseg < 1 || seg_offsets[0] != 0) return CCN_EINVAL;
+  return guarded([&] { return lamb_plan_create(seg_offsets, nseg, out); });
 }
 
 }  // extern "C"
@@ -1046,13 +1052,13 @@ extern "C" {
 int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, float* m, float* v, float lr, float beta1,
                  float beta2, float eps, float wd, int step, int mode, void* stream) {
   if (!w) return CCN_EINVAL;
-  return lamb_step(plan, g, P, w, nullptr, m, v, lr, beta1, beta2, eps, wd, step, mode, stream);
+  return guarded([&] { return lamb_step(plan, g, P, w, nullptr, m, v, lr, beta1, beta2, eps, wd, step, mode, stream); });
 }
 
 int ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v, float lr,
                            float beta1, float beta2, float eps, float wd, int step, int mode, void* stream) {
   if (!w) return CCN_EINVAL;
-  return lamb_step(plan, g, P, nullptr, w, m, v, lr, beta1, beta2, eps, wd, step, mode, stream);
+  return guarded([&] { return lamb_step(plan, g, P, nullptr, w, m, v, lr, beta1, beta2, eps, wd, step, mode, stream); });
 }
 
 int ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream) {

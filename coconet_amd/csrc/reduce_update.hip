@@ -289,40 +289,71 @@ __global__ __launch_bounds__(kBlock) void fill_f32_kernel(float* __restrict__ ds
 // ------------------------------------------------------------------------------------------------------------------
 // Scattered layout: gradients and weights live in nbuff separate buffers (one per parameter tensor), the moments in
 // single arrays that follow the buffers' concatenation, as ncclAllReduceScatteredAdam takes them
-// (nccl-overlap/src/nccl.h.in:216-218).  A plan cuts every buffer into tiles of kScatTile elements; one
-// single-wavefront workgroup per tile reads the tile record, then the buffer's pointers from a device table
-// (rank-major gradient pointers, then the weight pointers), then streams exactly like fused_stream_kernel.
-// State array 0 of the policy (w) is scattered, the others (m, v) are contiguous.
+// (nccl-overlap/src/nccl.h.in:216-218).  A plan cuts every buffer into tiles of kScatTile elements, numbered
+// through all buffers; one single-wavefront workgroup per tile finds its buffer, reads the buffer's pointers from a
+// device table (rank-major gradient pointers, then the weight pointers), then streams exactly like
+// fused_stream_kernel.  State array 0 of the policy (w) is scattered, the others (m, v) are contiguous.
+//
+// Finding the buffer costs no trip to HBM: a per-tile record would be read once per launch and so always miss the
+// caches, doubling the time a wavefront waits before it can issue its loads.  Instead one word per group of 32 tiles
+// names the buffer that holds the group's first tile (a 64-byte line of those words serves 512 consecutive
+// workgroups, so it is in L2 for all but the first), and the per-buffer records (first tile, first element), which
+// stay cached, are scanned forward from there: no step at all unless a buffer ends inside the group.  The pointers of
+// the group's buffer are fetched together with its record, and again only if the scan moved on.
 // ------------------------------------------------------------------------------------------------------------------
 constexpr int kScatTile = kWave * 4;   // 256 elements: one 4-element pack per lane
+constexpr int kScatCoarseShift = 5;    // one coarse word per 32 tiles
 
-struct ScatTile {
-  uint64_t off;    // first element inside the buffer
-  uint64_t goff;   // first element in the concatenation (index into the moment arrays)
-  uint32_t buf;
-  uint32_t count;  // elements in the tile (<= kScatTile)
-};
+struct ScatBuf {
+  uint64_t goff;        // first element of the buffer in the concatenation (index into the moment arrays)
+  uint32_t tile_begin;  // number of its first tile
+  uint32_t pad;
+};                      // entry nbuff holds the totals, so that [b + 1] always ends buffer b
 
 template <class M, int P>
-__global__ __launch_bounds__(kWave) void scattered_stream_kernel(const ScatTile* __restrict__ tiles,
+__global__ __launch_bounds__(kWave) void scattered_stream_kernel(const uint32_t* __restrict__ coarse,
+                                                                 const ScatBuf* __restrict__ bufs,
                                                                  const float* const* __restrict__ gtab,
                                                                  float* const* __restrict__ wtab, const int nP,
                                                                  const uint32_t nbuff, const StateTable<M::NS> moments,
                                                                  const typename M::Prm prm) {
   static_assert(M::NS >= 1 && !M::OUT16 && !M::OUTF && !M::FLAG, "fp32 policies with w as state 0");
   constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
-  const ScatTile t = tiles[(size_t)blockIdx.x + (size_t)blockIdx.y * gridDim.x];
+  const uint32_t tile = blockIdx.x + blockIdx.y * gridDim.x;
+  uint32_t buf = coarse[tile >> kScatCoarseShift];
+  ScatBuf r0 = bufs[buf], r1 = bufs[buf + 1];
   const float* gp[PX];
+  float* wp;
+  auto fetch_pointers = [&]() {
+#pragma unroll
+    for (int p = 0; p < PX; p++)
+      if (P > 0 || p < nP) gp[p] = gtab[(size_t)p * nbuff + buf];
+    wp = wtab[buf];
+  };
+  fetch_pointers();
+  if (r1.tile_begin <= tile) {
+    do {   // ends: entry nbuff holds the tile count, above every tile number
+      buf++;
+      r0 = r1;
+      r1 = bufs[buf + 1];
+    } while (r1.tile_begin <= tile);
+    fetch_pointers();
+  }
+  struct { uint64_t off, goff; uint32_t count; } t;
+  t.off = (uint64_t)(tile - r0.tile_begin) * kScatTile;
+  t.goff = r0.goff + t.off;
+  const uint64_t left = (r1.goff - r0.goff) - t.off;
+  t.count = left < (uint64_t)kScatTile ? (uint32_t)left : (uint32_t)kScatTile;
   uintptr_t bits = 0;
 #pragma unroll
   for (int p = 0; p < PX; p++) {
     if (P > 0 || p < nP) {
-      gp[p] = gtab[(size_t)p * nbuff + t.buf] + t.off;
+      gp[p] += t.off;
       bits |= reinterpret_cast<uintptr_t>(gp[p]);
     }
   }
   float* sp[M::NS];
-  sp[0] = wtab[t.buf] + t.off;
+  sp[0] = wp + t.off;
 #pragma unroll
   for (int k = 1; k < M::NS; k++) sp[k] = moments.p[k] + t.goff;
 #pragma unroll
@@ -464,7 +495,8 @@ struct ccn_scatter_plan {
   uint32_t nbuff = 0;
   size_t total = 0;
   size_t ntiles = 0;
-  ScatTile* tiles = nullptr;
+  uint32_t* coarse = nullptr;          // [ceil(ntiles / 2^kScatCoarseShift)] buffer of the group's first tile
+  ScatBuf* bufs = nullptr;             // [nbuff + 1]
   const void** table_dev = nullptr;    // [CCN_MAX_RANKS * nbuff] gradient pointers, rank-major, then [nbuff] weight pointers
   const void** table_pinned = nullptr; // staging copy in pinned host memory
   std::vector<const void*> shadow;     // what the device table holds
@@ -514,24 +546,24 @@ int launch_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float
   if (rc != CCN_OK) return rc;
   const float* const* gtab = reinterpret_cast<const float* const*>(plan->table_dev);
   float* const* wtab = reinterpret_cast<float* const*>(const_cast<void**>(plan->table_dev) + (size_t)CCN_MAX_RANKS * plan->nbuff);
-  // A wavefront here reads its tile record, then the buffer's pointers, and only then its data: two more round trips
-  // than the flat kernels, so more wavefronts per CU are needed to keep loads in flight (measured at P = 8: 10-16 per
-  // CU give 76 % of HBM peak, the flat kernels' 7 give 73 %).  The tuning override of stream_shape still applies.
-  const StreamShape sh = stream_shape((P + M::NS) * 16, M::NS * 16);
-  unsigned lds = lds_for_residency(10);
-  if (sh.lds_bytes != 0 && sh.lds_bytes < lds) lds = sh.lds_bytes;
+  // A wavefront here first finds its buffer and reads the buffer's pointers, and only then its data: two short round
+  // trips (cache hits) more than the flat kernels.  Measured at P = 8: 8 to 10 wavefronts per CU give 78 % of HBM peak,
+  // 7 give 76 %, 13 give 77 %.  CCN_LDS_KB overrides, as for the flat kernels.
+  static const int f_lds = [] { const char* e = std::getenv("CCN_LDS_KB"); return e ? std::atoi(e) : -1; }();
+  const unsigned lds = f_lds >= 0 && f_lds <= 64 ? (unsigned)f_lds * 1024u : lds_for_residency(8);
   const size_t gx = plan->ntiles < 0x40000000ull ? plan->ntiles : 0x40000000ull;
   const dim3 grid((unsigned)gx, (unsigned)((plan->ntiles + gx - 1) / gx));
   if (grid.x * (size_t)grid.y != plan->ntiles) return CCN_ERANGE;   // the kernel has no bounds check on the tile index
   switch (P) {
 #define CCN_CASE(K) \
-  case K: hipLaunchKernelGGL((scattered_stream_kernel<M, K>), grid, dim3(kWave), lds, s, (const ScatTile*)plan->tiles, gtab, \
+  case K: hipLaunchKernelGGL((scattered_stream_kernel<M, K>), grid, dim3(kWave), lds, s, (const uint32_t*)plan->coarse, \
+                             (const ScatBuf*)plan->bufs, gtab, \
                              wtab, P, plan->nbuff, st, prm); break;
     CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
 #undef CCN_CASE
     default:
-      hipLaunchKernelGGL((scattered_stream_kernel<M, 0>), grid, dim3(kWave), lds, s, (const ScatTile*)plan->tiles, gtab, wtab, P,
-                         plan->nbuff, st, prm);
+      hipLaunchKernelGGL((scattered_stream_kernel<M, 0>), grid, dim3(kWave), lds, s, (const uint32_t*)plan->coarse,
+                         (const ScatBuf*)plan->bufs, gtab, wtab, P, plan->nbuff, st, prm);
   }
   CCN_HIP(hipGetLastError());
   return CCN_OK;
@@ -608,45 +640,46 @@ int ccn_fused_adam_ref_f16g(const uint16_t* const* g, int P, float* w, uint16_t*
 int ccn_scatter_plan_destroy(ccn_scatter_plan* plan) {
   if (!plan) return CCN_OK;
   int rc = CCN_OK;
-  if (plan->tiles && hipFree(plan->tiles) != hipSuccess) rc = CCN_EHIP;
+  if (plan->coarse && hipFree(plan->coarse) != hipSuccess) rc = CCN_EHIP;
+  if (plan->bufs && hipFree(plan->bufs) != hipSuccess) rc = CCN_EHIP;
   if (plan->table_dev && hipFree(plan->table_dev) != hipSuccess) rc = CCN_EHIP;
   if (plan->table_pinned && hipHostFree(plan->table_pinned) != hipSuccess) rc = CCN_EHIP;
   delete plan;
   return rc;
 }
 
-int ccn_scatter_plan_create(const size_t* counts, int nbuff, ccn_scatter_plan** out) {
-  if (!out) return CCN_EINVAL;
-  *out = nullptr;
-  if (!counts || nbuff < 1) return CCN_EINVAL;
+static int scatter_plan_create(const size_t* counts, int nbuff, ccn_scatter_plan** out) {
   const DeviceInfo* di = nullptr;
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
-  std::vector<ScatTile> tiles;
-  size_t total = 0;
+  std::vector<ScatBuf> bufs((size_t)nbuff + 1);
+  std::vector<uint32_t> coarse;
+  size_t total = 0, ntiles = 0;
   for (int b = 0; b < nbuff; b++) {
     if (counts[b] == 0) return CCN_EINVAL;
-    for (size_t off = 0; off < counts[b]; off += kScatTile) {
-      ScatTile t;
-      t.off = off;
-      t.goff = total + off;
-      t.buf = (uint32_t)b;
-      t.count = (uint32_t)(counts[b] - off < (size_t)kScatTile ? counts[b] - off : (size_t)kScatTile);
-      tiles.push_back(t);
-    }
+    const size_t nt = (counts[b] + kScatTile - 1) / kScatTile;
+    if (ntiles + nt >= 0xffffffffull) return CCN_ERANGE;          // tile numbers are 32-bit
+    bufs[b] = ScatBuf{(uint64_t)total, (uint32_t)ntiles, 0u};
+    // every group of tiles whose first tile falls into this buffer
+    for (size_t grp = (ntiles + (1u << kScatCoarseShift) - 1) >> kScatCoarseShift; (grp << kScatCoarseShift) < ntiles + nt; grp++)
+      coarse.push_back((uint32_t)b);
     total += counts[b];
+    ntiles += nt;
   }
+  bufs[nbuff] = ScatBuf{(uint64_t)total, (uint32_t)ntiles, 0u};
   ccn_scatter_plan* p = new (std::nothrow) ccn_scatter_plan();
   if (!p) return CCN_ENOMEM;
   p->device = di->device;
   p->nbuff = (uint32_t)nbuff;
   p->total = total;
-  p->ntiles = tiles.size();
+  p->ntiles = ntiles;
   const size_t words = (size_t)(CCN_MAX_RANKS + 1) * (size_t)nbuff;
-  hipError_t e = hipMalloc((void**)&p->tiles, tiles.size() * sizeof(ScatTile));
+  hipError_t e = hipMalloc((void**)&p->coarse, coarse.size() * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipMalloc((void**)&p->bufs, bufs.size() * sizeof(ScatBuf));
   if (e == hipSuccess) e = hipMalloc((void**)&p->table_dev, words * sizeof(void*));
   if (e == hipSuccess) e = hipHostMalloc((void**)&p->table_pinned, words * sizeof(void*), hipHostMallocDefault);
-  if (e == hipSuccess) e = hipMemcpy(p->tiles, tiles.data(), tiles.size() * sizeof(ScatTile), hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(p->coarse, coarse.data(), coarse.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMemcpy(p->bufs, bufs.data(), bufs.size() * sizeof(ScatBuf), hipMemcpyHostToDevice);
   if (e != hipSuccess) {
     ccn_scatter_plan_destroy(p);
     return hip_fail(e);
@@ -655,15 +688,23 @@ int ccn_scatter_plan_create(const size_t* counts, int nbuff, ccn_scatter_plan** 
   return CCN_OK;
 }
 
+int ccn_scatter_plan_create(const size_t* counts, int nbuff, ccn_scatter_plan** out) {
+  if (!out) return CCN_EINVAL;
+  *out = nullptr;
+  if (!counts || nbuff < 1) return CCN_EINVAL;
+  return guarded([&] { return scatter_plan_create(counts, nbuff, out); });
+}
+
 int ccn_sgd_f32_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, float lr, void* stream) {
-  return launch_scattered<SgdMath>(plan, g, P, w, nullptr, SgdMath::Prm{lr}, stream);
+  return guarded([&] { return launch_scattered<SgdMath>(plan, g, P, w, nullptr, SgdMath::Prm{lr}, stream); });
 }
 
 int ccn_adam_f32_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v,
                            float lr, float beta1, float beta2, float eps, int step, void* stream) {
   if (step < 1) return CCN_EINVAL;
   float* mom[2] = {m, v};
-  return launch_scattered<AdamMath>(plan, g, P, w, mom, make_adam_prm(lr, beta1, beta2, eps, step, 1.0f), stream);
+  const AdamPrm prm = make_adam_prm(lr, beta1, beta2, eps, step, 1.0f);
+  return guarded([&] { return launch_scattered<AdamMath>(plan, g, P, w, mom, prm, stream); });
 }
 
 }  // extern "C"

@@ -149,12 +149,20 @@ int ccn_malloc(void** p, size_t bytes) {
   }
   void* base = nullptr;
   CCN_HIP(hipMalloc(&base, bytes + kStaggerPad));
-  std::lock_guard<std::mutex> lock(g_alloc_mu);
-  const size_t slot = (size_t)(g_alloc_count++) % kStaggerSlots;
-  void* user = static_cast<char*>(base) + slot * kStaggerStep;
-  g_alloc_base[user] = base;
-  *p = user;
-  return CCN_OK;
+  const int rc = guarded([&] {
+    std::lock_guard<std::mutex> lock(g_alloc_mu);
+    // Allocation c takes slot (c + c/16 + c/256 + c/4096) mod 16: allocations 1, 16, 256 or 4096 apart in the
+    // sequence all land in different slots, so the arrays walked in lock step differ whether the caller allocated
+    // rank by rank or tensor by tensor.
+    const size_t c = g_alloc_count++;
+    const size_t slot = (c + c / 16 + c / 256 + c / 4096) % kStaggerSlots;
+    void* user = static_cast<char*>(base) + slot * kStaggerStep;
+    g_alloc_base[user] = base;
+    *p = user;
+    return CCN_OK;
+  });
+  if (rc != CCN_OK) (void)hipFree(base);
+  return rc;
 }
 
 int ccn_free(void* p) {

@@ -668,10 +668,12 @@ def test_lamb_resident_kernel_shares_the_gpu(ccn):
 
 # ---------------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("P", [1, 3, 8, 11])
-def test_scattered_adam_and_sgd(ccn, P):
+@pytest.mark.parametrize("counts", [[1, 255, 256, 257, 1000, 4096, 70001, 3],
+                                    [1] * 70 + [300] + [2] * 40 + [9000, 8192, 5] + [256] * 33])
+def test_scattered_adam_and_sgd(ccn, P, counts):
     """Gradients and weights in separate buffers of ragged sizes (two of them misaligned by 4 bytes), moments in single
-    arrays over the concatenation: the same results, bit for bit, as the oracle on the concatenated arrays."""
-    counts = [1, 255, 256, 257, 1000, 4096, 70001, 3]
+    arrays over the concatenation: the same results, bit for bit, as the oracle on the concatenated arrays.  The second
+    list has runs of buffers smaller than a tile, so that many buffers end inside one group of tiles."""
     offs = np.concatenate([[0], np.cumsum(counts)])
     N = int(offs[-1])
     g = grads_f32(95 + P, P, N, 1e-3)
