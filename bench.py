@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adam_f32",
                     choices=["adam_f32", "adam_f32_scattered", "sgd_f32", "adam_f16g", "adam_bf16g", "lamb_f32",
-                             "mlp_outproj", "copy"])
+                             "lamb_nccl_f16g", "mlp_outproj", "copy"])
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -169,10 +169,10 @@ def main():
         units = N
         config = {"workload": f"adam_f32 over {nbuff} scattered buffers, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,
                   "algorithmic_bytes_per_param": per_param, "allocator": a.allocator}
-    elif wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g", "adam_bf16g"):
+    elif wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g", "adam_bf16g", "lamb_nccl_f16g"):
         P = a.ranks or (4 if wl == "sgd_f32" else 8)
         N = 1 << (a.log2n or (20 if wl == "sgd_f32" else 28))
-        gbytes = 2 if wl in ("adam_f16g", "adam_bf16g") else 4
+        gbytes = 2 if wl in ("adam_f16g", "adam_bf16g", "lamb_nccl_f16g") else 4
         half = torch.bfloat16 if wl == "adam_bf16g" else torch.float16
         gscale = 2.0 ** 7 if wl == "adam_bf16g" else 2.0 ** 16
         bufs = Buffers(capi, torch, a.allocator == "torch")
@@ -180,7 +180,7 @@ def main():
         for p in range(P):
             if gbytes == 2:
                 t = (torch.randn(N, device="cuda", generator=gen) * (1e-3 * gscale)).to(half)
-                if p == 0:
+                if p == 0 and wl != "lamb_nccl_f16g":
                     t[::1 << 20] = float("inf")        # benchmark configuration 3: one entry in 2^20 overflows
             else:
                 t = torch.empty(N, device="cuda").normal_(0.0, 1e-3 if wl != "sgd_f32" else 1e-2, generator=gen)
@@ -197,6 +197,14 @@ def main():
             per_param = (P + 1) * 4 + 4
             step = lambda t: capi.sgd_f32(g, w, N, 0.01, stream)
             kernel = "fused_stream_kernel<SgdMath, %d, 4, 1, %d>" % (P if P <= 8 else 0, 256 if P + 2 <= 3 else 64)
+        elif wl == "lamb_nccl_f16g":
+            # the modified NCCL's mixed-precision LAMB, 256 segments; runs the two-pass kernels
+            w16 = bufs.from_tensor(torch.empty(N, dtype=torch.float16, device="cuda"))
+            nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
+            plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
+            per_param = P * 2 + 12 + 12 + 2
+            step = lambda t: plan.step_nccl_f16g(g, w, w16, m, v, 1e-3, 0.9, 0.999, 1.0, stream)
+            kernel = "lamb_pass1_f16g_kernel<%d> + lamb_finalize_kernel + lamb_pass2_f16w_kernel" % (P if P <= 8 else 0)
         elif gbytes == 2:
             w16 = bufs.from_tensor(torch.empty(N, dtype=half, device="cuda"))
             flag = torch.zeros(1, dtype=torch.int32, device="cuda")
@@ -268,6 +276,16 @@ def main():
     wall_ms = (t1 - t0) * 1e3 / K
     ev_ms = e0.elapsed_ms(e1) / K
 
+    # the spread of single launches, each bracketed by its own pair of events (outside the timed region)
+    n_single = 0 if a.graph_steps > 0 else min(K, 50)
+    pairs = [(capi.Event(), capi.Event()) for _ in range(n_single)]
+    for i, (s0, s1) in enumerate(pairs):
+        s0.record(stream)
+        step(W + K + 1 + i)
+        s1.record(stream)
+    torch.cuda.synchronize()
+    singles = sorted(s0.elapsed_ms(s1) for s0, s1 in pairs)
+
     gbps = alg_bytes / (wall_ms * 1e-3) / 1e9
     ach = alg_bytes / (ev_ms * 1e-3) / 1e9
     line = {
@@ -275,13 +293,16 @@ def main():
         "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"adam_f16g": "f16 gradients, f32 state", "adam_bf16g": "bf16 gradients, f32 state",
+                  "lamb_nccl_f16g": "f16 gradients (f16 sum), f32 state",
                   "mlp_outproj": "bf16 x bf16 -> f32"}.get(wl, "f32"),
         "data": "synthetic", "config": config,
         "params_per_s": round(units / (wall_ms * 1e-3), 1),
         "device": info,
         "roofline": {"bound": "hbm", "achieved": round(ach, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": traffic_from_profiles(f"{wl}.pmc.txt"),
-                     "kernel": kernel, "avg_launch_ms": round(ev_ms, 5), "algorithmic_bytes_per_launch": alg_bytes},
+                     "kernel": kernel, "avg_launch_ms": round(ev_ms, 5), "algorithmic_bytes_per_launch": alg_bytes,
+                     "median_launch_ms": round(singles[len(singles) // 2], 5) if singles else None,
+                     "min_launch_ms": round(singles[0], 5) if singles else None},
     }
     if flops:
         line["mfma"] = {"achieved": round(flops / (ev_ms * 1e-3) / 1e12, 2), "peak": MFMA_BF16_PEAK_TFLOPS,

@@ -33,7 +33,7 @@ SYMBOLS = [
     "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
     "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
     "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
-    "ccn_lamb_f32_scattered", "ccn_adam_bf16g",
+    "ccn_lamb_f32_scattered", "ccn_adam_bf16g", "ccn_lamb_nccl_f16g",
 ]
 
 
@@ -100,6 +100,7 @@ def _declare(L):
     sig("ccn_lamb_f32", [_vp, _pp, _i, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
     sig("ccn_lamb_plan_norms", [_vp, _vp, _vp])
     sig("ccn_lamb_f32_scattered", [_vp, _pp, _i, _pp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
+    sig("ccn_lamb_nccl_f16g", [_vp, _pp, _i, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _vp])
     sig("ccn_mlp_outproj_bf16", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _vp])
     sig("ccn_bias_dropout_residual", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _vp])
     sig("ccn_scatter_plan_create", [C.POINTER(_sz), _i, _pp])
@@ -359,6 +360,12 @@ class LambPlan:
         wt = (C.c_void_p * self.nseg)(*[addr(x) for x in w])
         _check(load().ccn_lamb_f32_scattered(self.h, gt, len(g), wt, addr(m), addr(v), lr, beta1, beta2, eps, wd, step, mode,
                                              stream), "ccn_lamb_f32_scattered")
+
+    def step_nccl_f16g(self, g, w, halfw, m, v, lr, beta1, beta2, wd, stream=None):
+        """The modified NCCL's mixed-precision LAMB: g are fp16 bit patterns, halfw receives fp16(w)."""
+        p, _keep = ptr_table(g)
+        _check(load().ccn_lamb_nccl_f16g(self.h, p, len(g), addr(w), addr(halfw), addr(m), addr(v), lr, beta1, beta2, wd,
+                                         stream), "ccn_lamb_nccl_f16g")
 
     def norms(self, stream=None):
         import numpy as np

@@ -97,43 +97,58 @@ __device__ __forceinline__ float lamb_r(float mi, float vi, float w, const LambP
 
 // One pack of VEC elements starting at element e0.
 // Everything pass 1 reads for one pack of VEC elements.
-template <int P, int VEC>
+// G = float, or uint16_t for fp16 gradients (the modified NCCL's mixed-precision LAMB, CCN_LAMB_NCCL_GLOBAL only).
+template <int P, int VEC, class G = float>
 struct LambIn {
-  Pack<float, VEC> g[P > 0 ? P : CCN_MAX_RANKS];
+  Pack<G, VEC> g[P > 0 ? P : CCN_MAX_RANKS];
   Pack<float, VEC> w, m, v;
 };
 
 // Issues the pack's loads, all of them before anything waits (P = 0: the first nP of CCN_MAX_RANKS, wave-uniform).
-template <int P, int VEC>
-__device__ __forceinline__ void lamb_pass1_load(LambIn<P, VEC>& in, const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, int nP,
+template <int P, int VEC, class G = float>
+__device__ __forceinline__ void lamb_pass1_load(LambIn<P, VEC, G>& in, const SrcTable<G, (P ? P : CCN_MAX_RANKS)>& g, int nP,
                                                 const float* w, const float* m, const float* v, size_t e0) {
   constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
 #pragma unroll
   for (int p = 0; p < PX; p++) {
-    if (P > 0 || p < nP) in.g[p] = load_stream<float, VEC>(g.p[p] + e0);
+    if (P > 0 || p < nP) in.g[p] = load_stream<G, VEC>(g.p[p] + e0);
   }
   in.w = load_stream<float, VEC>(w + e0);   // w is read again by pass 2, 12 GB later
   in.m = load_stream<float, VEC>(m + e0);
   in.v = load_stream<float, VEC>(v + e0);
 }
 
-template <int P, int VEC>
-__device__ __forceinline__ void lamb_pass1_math(const LambIn<P, VEC>& in, int nP, float* m, float* v, size_t e0, float nf,
+template <int P, int VEC, class G = float>
+__device__ __forceinline__ void lamb_pass1_math(const LambIn<P, VEC, G>& in, int nP, float* m, float* v, size_t e0, float nf,
                                                 const LambPrm& k, double& accW, double& accR, Pack<float, VEC>& r_out,
                                                 Pack<float, VEC>& w_out) {
   constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
   Pack<float, VEC> mv, vv;
 #pragma unroll
   for (int e = 0; e < VEC; e++) {
-    float ge = in.g[0].d[e];
+    float ge, gsq;   // the gradient sum and its square
+    if constexpr (std::is_same<G, uint16_t>::value) {
+      // nccl/src/collectives/device/common_kernel.h:2460-2472 and reduce_kernel.h:391-399: the sum is carried in fp16
+      // and the square is taken in fp16
+      uint16_t S0 = in.g[0].d[e];
 #pragma unroll
-    for (int p = 1; p < PX; p++) {
-      if (P > 0 || p < nP) ge = ge + in.g[p].d[e];
+      for (int p = 1; p < PX; p++) {
+        if (P > 0 || p < nP) S0 = f32_to_f16_bits(f16_bits_to_f32(S0) + f16_bits_to_f32(in.g[p].d[e]));
+      }
+      ge = f16_bits_to_f32(S0);
+      gsq = f16_bits_to_f32(f32_to_f16_bits(ge * ge));
+    } else {
+      ge = in.g[0].d[e];
+#pragma unroll
+      for (int p = 1; p < PX; p++) {
+        if (P > 0 || p < nP) ge = ge + in.g[p].d[e];
+      }
+      gsq = ge * ge;
     }
     const float we = in.w.d[e];
     float mi, vi;
-    if (k.mode == CCN_LAMB_NCCL_GLOBAL) {
-      vi = ((in.v.d[e] * k.b2) + ((ge * ge) * k.omb2));
+    if (std::is_same<G, uint16_t>::value || k.mode == CCN_LAMB_NCCL_GLOBAL) {
+      vi = ((in.v.d[e] * k.b2) + (gsq * k.omb2));
       mi = ((in.m.d[e] * k.b1) + (ge * k.omb1));
     } else {
       mi = k.b1 * in.m.d[e] + k.omb1 * ge;
@@ -152,13 +167,13 @@ __device__ __forceinline__ void lamb_pass1_math(const LambIn<P, VEC>& in, int nP
 }
 
 // One pack of VEC elements starting at element e0.
-template <int P, int VEC>
-__device__ __forceinline__ void lamb_pass1_pack(const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, int nP, const float* w,
+template <int P, int VEC, class G = float>
+__device__ __forceinline__ void lamb_pass1_pack(const SrcTable<G, (P ? P : CCN_MAX_RANKS)>& g, int nP, const float* w,
                                                 float* m, float* v, size_t e0, float nf, const LambPrm& k, double& accW,
                                                 double& accR, Pack<float, VEC>& r_out, Pack<float, VEC>& w_out) {
-  LambIn<P, VEC> in;
-  lamb_pass1_load<P, VEC>(in, g, nP, w, m, v, e0);
-  lamb_pass1_math<P, VEC>(in, nP, m, v, e0, nf, k, accW, accR, r_out, w_out);
+  LambIn<P, VEC, G> in;
+  lamb_pass1_load<P, VEC, G>(in, g, nP, w, m, v, e0);
+  lamb_pass1_math<P, VEC, G>(in, nP, m, v, e0, nf, k, accW, accR, r_out, w_out);
 }
 
 template <int P, bool SCAT>
@@ -181,6 +196,34 @@ __global__ __launch_bounds__(kBlock) void lamb_pass1_kernel(const SrcTable<float
       const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
       Pack<float, 1> r1, w1;
       for (uint32_t j = j0; j < j1; j++) lamb_pass1_pack<P, 1>(gt, nP, wt, m, v, t.start + j, t.nf, k, accW, accR, r1, w1);
+    }
+  }
+  const double sW = block_sum(accW, lds);
+  const double sR = block_sum(accR, lds + kBlock / kWave);
+  if (threadIdx.x == 0) {
+    partials[2 * (size_t)blockIdx.x] = sW;
+    partials[2 * (size_t)blockIdx.x + 1] = sR;
+  }
+}
+
+// Pass 1 for fp16 gradients in flat arrays (the two-pass path only).
+template <int P>
+__global__ __launch_bounds__(kBlock) void lamb_pass1_f16g_kernel(const SrcTable<uint16_t, (P ? P : CCN_MAX_RANKS)> g, const int nP,
+                                                                 const float* w, float* m, float* v, const LambLayout lay,
+                                                                 double* __restrict__ partials, const int vec_ok,
+                                                                 const LambPrm k) {
+  __shared__ double lds[2 * kBlock / kWave];
+  const LambTile t = lamb_tile_of(lay, blockIdx.x);
+  double accW = 0.0, accR = 0.0;
+  const uint32_t j0 = threadIdx.x * 4;
+  if (j0 < t.count) {
+    if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+      Pack<float, 4> r4, w4;
+      lamb_pass1_pack<P, 4, uint16_t>(g, nP, w, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
+    } else {
+      const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
+      Pack<float, 1> r1, w1;
+      for (uint32_t j = j0; j < j1; j++) lamb_pass1_pack<P, 1, uint16_t>(g, nP, w, m, v, t.start + j, t.nf, k, accW, accR, r1, w1);
     }
   }
   const double sW = block_sum(accW, lds);
@@ -302,20 +345,24 @@ __global__ __launch_bounds__(kBlock) void lamb_fold_kernel(const double* __restr
   }
 }
 
-template <int VEC>
+// HALF: also writes the fp16 copy of the new weights (nccl/src/collectives/device/common_kernel.h:2695).
+template <int VEC, bool HALF = false>
 __device__ __forceinline__ void lamb_pass2_pack(float* w, const float* m, const float* v, size_t e0, float step_scale,
-                                                const LambPrm& k) {
+                                                const LambPrm& k, uint16_t* halfw = nullptr) {
   Pack<float, VEC> wv = load_stream<float, VEC>(w + e0);
   const Pack<float, VEC> mv = load_stream<float, VEC>(m + e0);
   const Pack<float, VEC> vv = load_stream<float, VEC>(v + e0);
+  Pack<uint16_t, VEC> hv;
 #pragma unroll
   for (int e = 0; e < VEC; e++) {
     const float we = wv.d[e];
     const float r = lamb_r(mv.d[e], vv.d[e], we, k);
     const float x = step_scale * r;
     wv.d[e] = we - x;
+    hv.d[e] = HALF ? f32_to_f16_bits(wv.d[e]) : (uint16_t)0;
   }
   store_stream<float, VEC>(w + e0, wv);
+  if constexpr (HALF) store_stream<uint16_t, VEC>(halfw + e0, hv);
 }
 
 template <bool SCAT>
@@ -332,6 +379,21 @@ __global__ __launch_bounds__(kBlock) void lamb_pass2_kernel(float* w, const floa
   } else {
     const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
     for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(wt, m, v, t.start + j, step_scale, k);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void lamb_pass2_f16w_kernel(float* w, uint16_t* halfw, const float* m, const float* v,
+                                                                 const LambLayout lay, const float* __restrict__ scale,
+                                                                 const int vec_ok, const LambPrm k) {
+  const LambTile t = lamb_tile_of(lay, blockIdx.x);
+  const float step_scale = k.lr * scale[t.seg];
+  const uint32_t j0 = threadIdx.x * 4;
+  if (j0 >= t.count) return;
+  if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+    lamb_pass2_pack<4, true>(w, m, v, t.start + j0, step_scale, k, halfw);
+  } else {
+    const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
+    for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1, true>(w, m, v, t.start + j, step_scale, k, halfw);
   }
 }
 
@@ -635,6 +697,8 @@ struct ccn_lamb_plan {
   const void** ptr_pinned = nullptr;
   std::vector<const void*> ptr_shadow;  // what the device table holds
   int ptr_ranks = 0;
+  // fp16 gradients: a plan over the same segments with every segment on the two-pass path; made on first use
+  ccn_lamb_plan* two_pass_twin = nullptr;
 };
 
 namespace {
@@ -716,11 +780,12 @@ int ccn_lamb_plan_destroy(ccn_lamb_plan* plan) {
     if (b && hipFree(b) != hipSuccess) rc = CCN_EHIP;
   }
   if (plan->ptr_pinned && hipHostFree(plan->ptr_pinned) != hipSuccess) rc = CCN_EHIP;
+  if (plan->two_pass_twin && ccn_lamb_plan_destroy(plan->two_pass_twin) != CCN_OK) rc = CCN_EHIP;
   delete plan;
   return rc;
 }
 
-static int lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** out) {
+static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_only, ccn_lamb_plan** out) {
   for (int b = 0; b < nseg; b++) {
     if (seg_offsets[b + 1] <= seg_offsets[b]) return CCN_EINVAL;   // empty or descending segment
   }
@@ -730,7 +795,7 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan**
 
   // Shape of the resident kernel.  CCN_LAMB_RESIDENT=0 sends every segment down the two-pass path;
   // CCN_LAMB_RES_BLOCK (64 | 256), CCN_LAMB_RES_WGS (workgroups per CU) and CCN_LAMB_SPIN are for tuning and tests.
-  const bool resident_wanted = env_long("CCN_LAMB_RESIDENT", 1) != 0;
+  const bool resident_wanted = !two_pass_only && env_long("CCN_LAMB_RESIDENT", 1) != 0;
   int res_block = (int)env_long("CCN_LAMB_RES_BLOCK", kBlock);
   if (res_block != kWave && res_block != kBlock) res_block = kBlock;
   const int res_sub = kResSub;
@@ -860,7 +925,7 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   if (!out) return CCN_EINVAL;
   *out = nullptr;
   if (!seg_offsets || nseg < 1 || seg_offsets[0] != 0) return CCN_EINVAL;
-  return guarded([&] { return lamb_plan_create(seg_offsets, nseg, out); });
+  return guarded([&] { return lamb_plan_create(seg_offsets, nseg, false, out); });
 }
 
 }  // extern "C"
@@ -1045,6 +1110,74 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
   return CCN_OK;
 }
 
+// One step of the modified NCCL's mixed-precision LAMB: fp16 gradients in flat arrays, fp32 w, m, v, fp16 copy of w.
+int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v, float lr,
+                   float beta1, float beta2, float wd, void* stream) {
+  if (!plan || !g || !w || !halfw || !m || !v || P < 1 || P > CCN_MAX_RANKS) return CCN_EINVAL;
+  for (int p = 0; p < P; p++) if (!g[p]) return CCN_EINVAL;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  if (di->device != plan->device) return CCN_EINVAL;
+  if (!plan->two_pass_twin) {
+    std::vector<size_t> offs(plan->seg_start.begin(), plan->seg_start.end());
+    offs.push_back(plan->N);
+    rc = lamb_plan_create(offs.data(), plan->nseg, true, &plan->two_pass_twin);
+    if (rc != CCN_OK) return rc;
+  }
+  ccn_lamb_plan* tp = plan->two_pass_twin;
+
+  LambPrm k;
+  k.b1 = beta1;
+  k.omb1 = 1 - beta1;
+  k.b2 = beta2;
+  k.omb2 = 1 - beta2;
+  k.eps = 0.0f;
+  k.wd = wd;
+  k.lr = lr;
+  k.mode = CCN_LAMB_NCCL_GLOBAL;
+  k.bc1 = k.bc2 = 1.0;
+
+  bool al = aligned16(w) && aligned16(m) && aligned16(v) && (reinterpret_cast<uintptr_t>(halfw) & 7u) == 0;
+  for (int p = 0; p < P; p++) al = al && (reinterpret_cast<uintptr_t>(g[p]) & 7u) == 0;
+  const int vec_ok = al ? 1 : 0;
+  hipStream_t s = as_stream(stream);
+  const dim3 grid((unsigned)tp->ntiles), block(kBlock);
+  LambLayout lay;
+  lay.tiles = tp->tiles;
+  lay.seg_len = vec_ok ? tp->uniform_seg_len : 0;
+  lay.seg_len_f = (float)tp->uniform_seg_len;
+  lay.tile = kLambTile;
+  lay.gtab = nullptr;
+  lay.wtab = nullptr;
+  lay.nseg = (uint32_t)tp->nseg;
+  with_rank_count(P, [&](auto ptag) {
+    constexpr int PP = decltype(ptag)::value;
+    SrcTable<uint16_t, (PP ? PP : CCN_MAX_RANKS)> tbl;
+    for (int p = 0; p < (PP ? PP : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < P ? p : 0];
+    hipLaunchKernelGGL((lamb_pass1_f16g_kernel<PP>), grid, block, lds_for_residency(P >= 2 ? 4 : 0), s, tbl, P, (const float*)w, m,
+                       v, lay, tp->partials, vec_ok, k);
+  });
+  CCN_HIP(hipGetLastError());
+  const double* sums = tp->partials;
+  const uint32_t* seg_begin = tp->seg_tile_begin;
+  if (tp->ngroups) {
+    hipLaunchKernelGGL(lamb_fold_kernel, dim3(tp->ngroups), block, 0, s, (const double*)tp->partials,
+                       (const uint32_t*)tp->group_begin, tp->folded);
+    CCN_HIP(hipGetLastError());
+    sums = tp->folded;
+    seg_begin = tp->seg_group_begin;
+  }
+  // the norms and scales land in the caller's plan, where ccn_lamb_plan_norms reads them
+  hipLaunchKernelGGL(lamb_finalize_kernel, dim3((unsigned)tp->nseg), block, 0, s, sums, seg_begin, (const uint64_t*)tp->seg_len,
+                     plan->norms, plan->scale, k.mode);
+  CCN_HIP(hipGetLastError());
+  hipLaunchKernelGGL(lamb_pass2_f16w_kernel, grid, block, 0, s, w, halfw, (const float*)m, (const float*)v, lay,
+                     (const float*)plan->scale, vec_ok, k);
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1059,6 +1192,11 @@ int ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, fl
                            float beta1, float beta2, float eps, float wd, int step, int mode, void* stream) {
   if (!w) return CCN_EINVAL;
   return guarded([&] { return lamb_step(plan, g, P, nullptr, w, m, v, lr, beta1, beta2, eps, wd, step, mode, stream); });
+}
+
+int ccn_lamb_nccl_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
+                       float lr, float beta1, float beta2, float wd, void* stream) {
+  return guarded([&] { return lamb_step_f16g(plan, g, P, w, halfw, m, v, lr, beta1, beta2, wd, stream); });
 }
 
 int ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream) {

@@ -173,7 +173,16 @@ int  ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, f
  * device pointers.  The plan keeps a device copy of the pointers, refreshed (one stream synchronisation) when they change. */
 int  ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v,
                             float lr, float beta1, float beta2, float eps, float wd, int step, int mode, void* stream);
-/* copies W_b, R_b of the last ccn_lamb_f32 on this plan to a HOST array of 2*nseg doubles (synchronises) */
+/* The modified NCCL's mixed-precision LAMB: fp16 gradients (their sum carried in fp16, the square taken in fp16), fp32
+ * w, m, v, and an fp16 copy of the new weights in halfw; arithmetic of CCN_LAMB_NCCL_GLOBAL otherwise (per segment,
+ * wd in place of the hard-coded 1.0f, no eps, no step).  g: HOST array of P device pointers to fp16 bit patterns.
+ * Replaces AllReduce_pipe(lr, beta1, beta2, (half*)g, w, halfw, m, v, r, ...) of nccl/src/nccl.h.in:211-216 for the
+ * LAMB build (phase 1 nccl/src/collectives/device/common_kernel.h:2438-2535, phase 2 :2657-2700); the caller's r
+ * buffer is not needed: phase 2 recomputes r from the stored m and v.  Runs the two-pass kernels (a second tile table
+ * over the same segments is made on the first call, which therefore allocates and cannot be recorded). */
+int  ccn_lamb_nccl_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
+                        float lr, float beta1, float beta2, float wd, void* stream);
+/* copies W_b, R_b of the last LAMB step on this plan to a HOST array of 2*nseg doubles (synchronises) */
 int  ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream);
 
 /* ---- model-parallel MLP out-projection, one rank's K-slice, epilogue fused into the GEMM write-back:

@@ -75,6 +75,8 @@ def _declare(L):
     L.orc_adam_bf16g.argtypes = [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _f, _i, _f]
     L.orc_overflow_f16.restype = C.c_uint32
     L.orc_overflow_f16.argtypes = [_pp, _i, _sz]
+    L.orc_lamb_nccl_f16g.restype = None
+    L.orc_lamb_nccl_f16g.argtypes = [_pp, _i, _vp, _vp, _vp, _vp, _vp, _i, _f, _f, _f, _f, _vp]
     L.orc_lamb_f32.restype = None
     L.orc_lamb_f32.argtypes = [_pp, _i, _vp, _vp, _vp, _vp, _i, _f, _f, _f, _f, _f, _i, _i, _vp]
     L.orc_philox4x32_10.restype = None
@@ -203,6 +205,19 @@ def lamb_f32(g, w, m, v, seg_offsets, lr, beta1, beta2, eps, wd, step, mode=0):
     norms = np.zeros((nseg, 2), np.float64)
     lib().orc_lamb_f32(p, len(g), _ptr(w, f32), _ptr(m, f32), _ptr(v, f32), so.ctypes.data_as(C.c_void_p), nseg,
                        lr, beta1, beta2, eps, wd, step, mode, norms.ctypes.data_as(C.c_void_p))
+    return norms
+
+
+def lamb_nccl_f16g(g16, w, halfw, m, v, seg_offsets, lr, beta1, beta2, wd):
+    """The modified NCCL's mixed-precision LAMB (fp16 gradients, fp16 weight copy).  Returns norms (nseg, 2)."""
+    p, _k = _ptrs(g16, u16)
+    so = np.ascontiguousarray(seg_offsets, dtype=np.uint64)
+    nseg = so.size - 1
+    assert so[-1] == w.size and so[0] == 0
+    norms = np.zeros((nseg, 2), np.float64)
+    lib().orc_lamb_nccl_f16g(p, len(g16), _ptr(w, f32), _ptr(halfw, u16), _ptr(m, f32), _ptr(v, f32),
+                             so.ctypes.data_as(C.c_void_p), nseg, lr, beta1, beta2, wd,
+                             norms.ctypes.data_as(C.c_void_p))
     return norms
 
 

@@ -325,6 +325,46 @@ static void lamb_nccl_segment(const float* const* g, int P, float* w, float* m, 
   }
 }
 
+/* The modified NCCL's LAMB with fp16 gradients (its mixed-precision path), per segment:
+ *   phase 1 nccl/src/collectives/device/common_kernel.h:2438-2535: gradient sum carried in fp16 (FuncSumHalf chain,
+ *   :2460-2472); functors nccl/src/collectives/device/reduce_kernel.h:391-399 mixedbinOp1 (square taken in fp16),
+ *   mixedbinOp3 (here with beta1, :2509), binOp2, binOp4, rOp :425-432; phase 2 common_kernel.h:2677-2700 with the
+ *   fp16 copy of the new weights (float4ToHalf4, :2695).
+ *   S0 = fp16 sum;  v = (v*b2) + (float(S0*S0 in fp16)*(1-b2));  S4 = v/b2;  m = (m*b1) + (float(S0)*(1-b1));  S3 = m/b1;
+ *   r = S3/sqrtf(S4) + 1.0f*w;  norms, scale and the update as in lamb_nccl_segment;  halfw = fp16(w).
+ * The kernel keeps r in a caller's buffer between the phases; recomputing it from the stored m, v and the old w
+ * gives the same bits.  wd takes the place of the hard-coded 1.0f. */
+void orc_lamb_nccl_f16g(const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
+                        const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2, float wd,
+                        double* norms_out) {
+  for (int b = 0; b < nseg; b++) {
+    const size_t lo = seg_offsets[b], hi = seg_offsets[b + 1];
+    double rr = 0.0, ww = 0.0;
+    for (size_t i = lo; i < hi; i++) {
+      uint16_t S0 = g[0][i];
+      for (int p = 1; p < P; p++) S0 = hadd(S0, g[p][i]);
+      float vi = ((v[i] * beta2) + ((orc_f16_to_f32(hmul(S0, S0))) * (1 - beta2)));
+      float S4 = (vi / beta2);
+      float mi = ((m[i] * beta1) + ((orc_f16_to_f32(S0)) * (1 - beta1)));
+      float S3 = (mi / beta1);
+      float r = (S3) / sqrtf(S4) + wd * w[i];
+      ww += (double)(w[i] * w[i]);
+      rr += (double)(r * r);
+      v[i] = vi;
+      m[i] = mi;
+    }
+    const float wNorm = sqrtf((float)ww), rNorm = sqrtf((float)rr);
+    if (norms_out) { norms_out[2 * b] = wNorm; norms_out[2 * b + 1] = rNorm; }
+    const float scale = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f) / rNorm;
+    for (size_t i = lo; i < hi; i++) {
+      float r = ((m[i] / beta1)) / sqrtf((v[i] / beta2)) + wd * w[i];
+      float delta = (lr * scale) * r;
+      w[i] = w[i] - delta;
+      halfw[i] = orc_f32_to_f16(w[i]);
+    }
+  }
+}
+
 void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
                   const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2,
                   float eps, float wd, int step, int mode, double* norms_out) {

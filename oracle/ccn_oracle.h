@@ -24,6 +24,9 @@
  *   orc_lamb_f32          same file :402-449; single-segment/w==0 special cases, float64 brute force  pinned
  *                         (mode 2: nccl/.../reduce_kernel.h:391-452; all-ones closed form, float64 brute force;
  *                          the reference sums its norms in fp32 in no fixed order: norm rounding parity unpinned)
+ *   orc_lamb_nccl_f16g    nccl/.../common_kernel.h:2438-2535, 2677-2700; equals orc_lamb_f32 mode 2 bit for bit where
+ *                         the fp16 sums and squares are exact; numpy float16 restatement of the fp16 chain   pinned
+ *                         (rounding of the fp32 norm sums unpinned, as for mode 2)
  *   orc_adam_f16g,        no counterpart in the reference (it has no loss scaling / overflow detection, and no bfloat16):
  *   orc_adam_bf16g        build-defined, pinned by closed forms only; parity with Apex "parity unpinned"
  *   orc_philox4x32_10     Random123 known-answer vectors                         pinned
@@ -85,6 +88,9 @@ uint32_t orc_overflow_f16(const uint16_t* const* g, int P, size_t N);
  *      mode 0: scale = trust ratio W/R;  mode 1 (reference): scale = (W/R)/R;
  *      mode 2: the modified NCCL's global-norm LAMB arithmetic (divide by beta, L2 norms, no eps).
  *      norms_out (optional, 2*nseg doubles): W_b, R_b after the square root. ---- */
+void orc_lamb_nccl_f16g(const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
+                        const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2, float wd,
+                        double* norms_out);
 void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
                   const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2,
                   float eps, float wd, int step, int mode, double* norms_out);

@@ -667,6 +667,47 @@ def test_lamb_resident_kernel_shares_the_gpu(ccn):
 
 
 # ---------------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("P,segs,shift", [(8, [0, 1 << 18], 0), (3, [0, 700, 701, 5000, 8192 + 3], 0),
+                                          (8, [0, 4096, 8192, 12288], 0), (11, [0, 1000, 70001], 0),
+                                          (2, [0, 4099], 1), (1, [0, 1], 0), (8, [0, 5 * 1024 * 4096 + 17], 0)])
+def test_lamb_nccl_mixed_precision(ccn, P, segs, shift):
+    """The modified NCCL's LAMB with fp16 gradients: m and v bit for bit, w within the fp32 bar (the order of the
+    float64 norm sums differs), the fp16 weight copy within one fp16 ulp and equal to fp16 of the kernel's own w.
+    shift = 1: every array starts one element past an aligned address (scalar path).  The last case has a segment of
+    more than 4096 tiles (the partial sums are folded in two levels)."""
+    N = segs[-1]
+    g16 = [orc.f32_to_f16(x) for x in grads_f32(71 + P, P, N, 0.5)]
+    w0 = weights_f32(71, N, 0.05)
+    m0 = weights_f32(72, N, 0.01)
+    v0 = np.abs(weights_f32(73, N, 1e-2)) + np.float32(1e-3)
+
+    def place(a, dt):
+        if not shift:
+            return dev(a) if dt == "f" else dev_u16(a)
+        pad = np.concatenate([np.zeros(1, a.dtype), a])
+        return (dev(pad) if dt == "f" else dev_u16(pad))[1:]
+
+    gd = [place(x, "h") for x in g16]
+    wd, md, vd = place(w0, "f"), place(m0, "f"), place(v0, "f")
+    hwd = place(np.zeros(N, np.uint16), "h")
+    w, m, v, hw = w0.copy(), m0.copy(), v0.copy(), np.zeros(N, np.uint16)
+    plan = ccn.LambPlan(segs)
+    for _ in range(2):
+        plan.step_nccl_f16g(gd, wd, hwd, md, vd, 0.01, 0.9, 0.999, 1.0)
+        want_norms = orc.lamb_nccl_f16g(g16, w, hw, m, v, segs, 0.01, 0.9, 0.999, 1.0)
+    got_norms = plan.norms()
+    plan.close()
+    assert_f32_parity(host(md), m, "mixed lamb m")
+    assert_f32_parity(host(vd), v, "mixed lamb v")
+    got_w = host(wd)
+    assert np.max(np.abs(got_w.astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
+    assert np.max(np.abs(got_norms - want_norms) / want_norms) <= 1e-6
+    got_hw = host_u16(hwd)
+    assert np.array_equal(got_hw, got_w.astype(np.float16).view(np.uint16))
+    assert rel_err(orc.f16_to_f32(got_hw), orc.f16_to_f32(hw)) <= 1e-3
+
+
+# ---------------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("P", [1, 3, 8, 11])
 @pytest.mark.parametrize("counts", [[1, 255, 256, 257, 1000, 4096, 70001, 3],
                                     [1] * 70 + [300] + [2] * 40 + [9000, 8192, 5] + [256] * 33])

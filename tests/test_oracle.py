@@ -477,3 +477,53 @@ def test_adam_bf16g_reduces_to_adam_and_flags():
     assert np.array_equal(w[keep], wr[keep]) and np.array_equal(m[keep], mr[keep]) and np.array_equal(v[keep], vr[keep])
     assert np.array_equal(w[~keep], w0[~keep]) and np.all(m[~keep] == 0) and np.all(v[~keep] == 0)
     assert np.all(np.isfinite(w)) and np.isfinite(m).all() and np.isfinite(v).all()
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the modified NCCL's mixed-precision LAMB (fp16 gradients)
+# ---------------------------------------------------------------------------------------------------------------------
+def test_lamb_nccl_f16g_equals_fp32_variant_where_fp16_is_exact():
+    """Small-integer gradients: the fp16 sum and the fp16 square are exact, so every bit of m, v, w and the norms must
+    equal the fp32 variant (mode 2) on the same values; a wrong beta, a dropped term or a swapped operand shows."""
+    P, segs = 8, [0, 700, 701, 5000, 8192]
+    N = segs[-1]
+    r = rng(61)
+    gi = [r.integers(-2, 3, N).astype(np.float32) for _ in range(P)]        # |sum| <= 16, square <= 256
+    g16 = [orc.f32_to_f16(x) for x in gi]
+    w0 = weights_f32(61, N, 0.05)
+    m0 = weights_f32(62, N, 0.01)
+    v0 = np.abs(weights_f32(63, N, 1e-2)) + np.float32(1e-3)
+    w, m, v, hw = w0.copy(), m0.copy(), v0.copy(), np.zeros(N, np.uint16)
+    n16 = orc.lamb_nccl_f16g(g16, w, hw, m, v, segs, 0.01, 0.9, 0.999, 1.0)
+    wr, mr, vr = w0.copy(), m0.copy(), v0.copy()
+    n32 = orc.lamb_f32(gi, wr, mr, vr, segs, 0.01, 0.9, 0.999, 0.0, 1.0, 1, mode=2)
+    assert np.array_equal(m, mr) and np.array_equal(v, vr) and np.array_equal(w, wr)
+    assert np.array_equal(n16, n32)
+    assert np.array_equal(hw, w.astype(np.float16).view(np.uint16))
+
+
+def test_lamb_nccl_f16g_half_chain_against_numpy_float16():
+    """Where fp16 rounds: the sum chain and the square, restated with numpy's float16 (correctly rounded, an
+    independent implementation), must give the same m and v."""
+    P, N = 5, 4096
+    g32 = grads_f32(64, P, N, 3.0)
+    g16 = [orc.f32_to_f16(x) for x in g32]
+    w0 = weights_f32(64, N, 0.05)
+    m0 = weights_f32(65, N, 0.01)
+    v0 = np.abs(weights_f32(66, N, 1e-2)) + np.float32(1e-3)
+    w, m, v, hw = w0.copy(), m0.copy(), v0.copy(), np.zeros(N, np.uint16)
+    orc.lamb_nccl_f16g(g16, w, hw, m, v, [0, N], 0.01, 0.9, 0.999, 1.0)
+    S0 = g16[0].view(np.float16).copy()
+    for x in g16[1:]:
+        S0 = (S0 + x.view(np.float16)).astype(np.float16)
+    sq = (S0 * S0).astype(np.float16)
+    assert np.any(sq.astype(np.float32) != S0.astype(np.float32) ** 2)      # the square does round somewhere
+    b1, b2 = np.float32(0.9), np.float32(0.999)
+    want_v = (v0 * b2) + (sq.astype(np.float32) * (np.float32(1) - b2))
+    want_m = (m0 * b1) + (S0.astype(np.float32) * (np.float32(1) - b1))
+    assert np.array_equal(v, want_v.astype(np.float32)) and np.array_equal(m, want_m.astype(np.float32))
+    # and the update, in float64, from those m and v
+    r = (want_m.astype(np.float64) / 0.9) / np.sqrt(want_v.astype(np.float64) / np.float64(b2)) + w0
+    scale = (np.sqrt(np.sum(w0.astype(np.float64) ** 2)) / np.sqrt(np.sum(r ** 2))) / np.sqrt(np.sum(r ** 2))
+    assert np.max(np.abs(w - (w0 - 0.01 * scale * r))) <= 1e-6 * np.max(np.abs(w0))
+    assert np.array_equal(hw, w.astype(np.float16).view(np.uint16))
