@@ -65,6 +65,14 @@ def test_argument_validation_happens_before_any_device_work():
     offs = (C.c_size_t * 3)(1, 10, 20)
     assert lib.ccn_lamb_plan_create(offs, 2, C.byref(plan)) == capi.CCN_EINVAL      # does not start at 0
     assert lib.ccn_lamb_f32(None, p, 2, 0x1000, 0x1000, 0x1000, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, 0, None) == capi.CCN_EINVAL
+    assert lib.ccn_lamb_nccl_f16g(None, p, 2, 0x1000, 0x1000, 0x1000, 0x1000, 1e-3, 0.9, 0.999, 1.0, None) == capi.CCN_EINVAL
+    tbl[3] = 0x1000
+    assert lib.ccn_adam_bf16g(p, 8, 0x1000, 0x1000, 0x1000, 0x1000, 16, 1e-3, 0.9, 0.999, 1e-6, 0, 1.0, 0x1000, None) == capi.CCN_EINVAL
+    assert lib.ccn_adam_bf16g(p, 8, 0x1000, 0x1000, 0x1000, None, 16, 1e-3, 0.9, 0.999, 1e-6, 1, 1.0, 0x1000, None) == capi.CCN_EINVAL
+    assert lib.ccn_scatter_plan_create(None, 4, C.byref(plan)) == capi.CCN_EINVAL
+    counts = (C.c_size_t * 2)(10, 0)
+    assert lib.ccn_scatter_plan_create(counts, 0, C.byref(plan)) == capi.CCN_EINVAL
+    assert lib.ccn_adam_f32_scattered(None, p, 2, p, 0x1000, 0x1000, 1e-3, 0.9, 0.999, 1e-6, 1, None) == capi.CCN_EINVAL
 
 
 def test_missing_library_fails_loudly(monkeypatch):
