@@ -89,3 +89,23 @@ def test_product_package_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".hpp", ".cpp", ".h")):
                 text = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+
+
+def test_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 on its own, and a C program must link against the library."""
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no C compiler")
+    src = tmp_path / "c_abi.c"
+    src.write_text('#include "coconet_hip.h"\n'
+                   'int main(void) { return (ccn_version() > 0 && ccn_strerror(CCN_EINVAL) != 0) ? 0 : 1; }\n')
+    inc = os.path.join(ROOT, "include")
+    obj = tmp_path / "c_abi.o"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, "-c", str(src), "-o", str(obj)],
+                   check=True)
+    libdir = os.path.dirname(capi.LIB_PATH)
+    exe = tmp_path / "c_abi"
+    subprocess.run(["gcc", str(obj), "-o", str(exe), "-L", libdir, "-lcoconet_hip", "-Wl,-rpath," + libdir,
+                    "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"], check=True)
+    assert subprocess.run([str(exe)]).returncode == 0
