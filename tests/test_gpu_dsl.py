@@ -18,6 +18,14 @@ REF = ["ref-sgd-ar-c", "ref-sgd-rs-c-ag", "ref-sgd-fuse-rs-c-ag", "ref-adam-ar-c
        "ref-adam-fuse-rs-c-ag", "ref-lamb-ar-c", "ref-lamb-rs-c-ag", "ref-lamb-fuse-rs-c-ag"]
 
 
+def as_the_reference_scraper_reads(line):
+    """The reference's result scraper quotes the keys of every {...} line and evaluates it as a dict literal
+    (experiments/generate-pdf/process_hypercluster_data.py:41-54); the emitted lines must survive that."""
+    import ast
+    quoted = line.replace("{", '{"').replace(":", '":').replace(",", ',"')
+    return {k.strip(): v for k, v in ast.literal_eval(quoted).items()}
+
+
 def run_program(name, *args):
     exe = os.path.join(GEN, name)
     if not os.path.exists(exe):
@@ -31,6 +39,8 @@ def run_program(name, *args):
         if m:
             fields = dict(re.findall(r"(\w+): ([0-9.eE+-]+)", m.group(3)))
             rows.append((int(m.group(1)), int(m.group(2)), {k: float(v) for k, v in fields.items()}))
+            d = as_the_reference_scraper_reads(line.strip())
+            assert d["SZ"] == rows[-1][0] and d["Epochs"] == rows[-1][1] and abs(d["Total"] - rows[-1][2]["Total"]) < 1e-9
     return rows
 
 
