@@ -78,17 +78,15 @@ StreamShape stream_shape(int load_bytes, int store_bytes) {
   StreamShape sh;
   // Single-wavefront workgroups, and fewer of them per CU the more 16-byte loads each thread has in flight.
   // Measured optima on MI355X at N = 2^28 (2^27 beyond 8 ranks), fp32 Adam unless said otherwise, as
-  // loads per thread -> wavefronts per CU (% of HBM peak): 4 -> 13+ (83), 5 -> 11-14 (84), 7 -> 12-13 (83; fp16-gradient
-  // Adam at 8 ranks: 81), 9 -> 8 (86; SGD at 8 ranks: 84), 11 -> 7 (85.5; 6 or 8 give 82-83), 15 -> 8 (82), 19 -> 6-10 (79).
+  // loads per thread -> wavefronts per CU (% of HBM peak): 2 -> 26 (SGD at 1 rank: 85.5; 256-thread workgroups at full
+  // occupancy 82.5), 3 -> 16-20 (SGD at 2 ranks: 84.6; 13: 79), 4 -> 17 (SGD at 3 ranks: 84.6; 13: 81), 5 -> 11-14 (84),
+  // 7 -> 12-13 (83; fp16-gradient Adam at 8 ranks: 81), 9 -> 8 (86; SGD at 8 ranks: 84), 11 -> 7 (85.5; 6 or 8 give
+  // 82-83), 15 -> 8 (82), 19 -> 6-10 (79).
   const int loads = (load_bytes + 15) / 16;
-  if (loads + (store_bytes + 15) / 16 <= 3) {
-    sh.block = 256;                 // copy-like kernels want all the occupancy they can get
-    sh.lds_bytes = 0;
-  } else {
-    const int waves = loads <= 7 ? 13 : (loads <= 10 ? 8 : (loads <= 13 ? 7 : 8));
-    sh.block = 64;
-    sh.lds_bytes = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
-  }
+  (void)store_bytes;
+  const int waves = loads <= 2 ? 26 : (loads <= 4 ? 17 : (loads <= 7 ? 13 : (loads <= 10 ? 8 : (loads <= 13 ? 7 : 8))));
+  sh.block = 64;
+  sh.lds_bytes = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
   if (f_block == 64 || f_block == 256) sh.block = f_block;
   if (f_lds >= 0 && f_lds <= 64) sh.lds_bytes = (unsigned)f_lds * 1024u;
   return sh;

@@ -294,10 +294,9 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // Launch shape for a kernel whose threads load `loads` and store `stores` 16-byte packs, from measurements on MI355X
 // at 2^28 elements: single-wavefront workgroups, and fewer of them per CU the more loads a thread has in flight
-// (13 up to 7 loads, 7 up to 10, 6 up to 13, 8 beyond: one fewer than the library's kernels of the same shape, whose
-// double-precision bias correction keeps a wavefront busy for longer), the cap expressed as unused dynamic LDS;
-// copy-like kernels want 256-thread workgroups and all the occupancy they can get.  Scalar (unaligned) launches keep
-// 256 threads.
+// (26 up to 2 loads, 20 up to 4, 13 up to 7, 7 up to 10, 6 up to 13, 8 beyond: from 8 loads on one fewer than the
+// library's kernels of the same shape, whose double-precision bias correction keeps a wavefront busy for longer), the
+// cap expressed as unused dynamic LDS.  Scalar (unaligned) launches keep 256 threads.
 struct LaunchShape {
   int block;
   unsigned lds;
@@ -307,8 +306,10 @@ inline LaunchShape shape_for(int loads, int stores, int vec, bool has_sums = fal
   static const int f_block = [] { const char* e = getenv("CCN_BLOCK"); return e ? atoi(e) : 0; }();
   static const int f_lds = [] { const char* e = getenv("CCN_LDS_KB"); return e ? atoi(e) : -1; }();
   LaunchShape sh{kBlock, 0};
-  if (vec == 1 || loads + stores <= 3) return sh;
-  const int waves = loads <= 7 ? 13 : (loads <= 10 ? 7 : (loads <= 13 ? 6 : 8));
+  (void)stores;
+  if (vec == 1) return sh;
+  // wavefronts per CU by 16-byte loads per thread, measured at N = 2^28: 2 -> 26, 3-4 -> 20, 5-7 -> 13, 8-10 -> 7, 11-13 -> 6
+  const int waves = loads <= 2 ? 26 : (loads <= 4 ? 20 : (loads <= 7 ? 13 : (loads <= 10 ? 7 : (loads <= 13 ? 6 : 8))));
   sh.block = kWave;
   sh.lds = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
   if (has_sums) {   // float64 sums and a workgroup reduction: four 256-thread workgroups per CU hide them better
