@@ -218,7 +218,7 @@ def main():
             plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
             per_param = (P + 3) * 4 + 3 * 4
             step = lambda t: plan.step(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, capi.LAMB_TRUST_RATIO, stream)
-            kernel = "lamb_reset_kernel + lamb_resident_kernel<%d, 256, 4> + lamb_deferred_kernel<256, 4>" % (P if P <= 8 else 0)
+            kernel = "lamb_reset_kernel + lamb_oneshot_kernel<%d, 256, 8> + lamb_deferred_kernel<256, 8>" % (P if P <= 8 else 0)
         alg_bytes = float(per_param) * N
         units = N
         config = {"workload": f"{wl} fused reduce+update, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,

@@ -1,12 +1,14 @@
 // LAMB with per-segment trust ratio.  The update of a segment needs the segment's two norms, which need every element
 // of the segment first, so each element is visited twice.  A plan sorts the segments into two groups:
 //
-// resident segments (short enough for the chip to hold between the visits: 2 tiles per workgroup of a grid that fills
-//   the GPU once, 4 M elements at the default shape) go through one persistent kernel.  A workgroup runs pass 1 on a
-//   tile (P-way gradient reduce, m/v update, r, the tile's float64 sums of w^2 and r^2), parks r and the old w in
-//   LDS, and one round later, when the workgroup that finished the segment's last tile has published the scale,
-//   writes w from what it parked: 56 bytes per element instead of 68.  No sum is an atomic accumulation: tile sums
-//   are stored one by one and added in a fixed order, so results do not depend on scheduling.
+// resident segments (short enough for the chip to hold between the visits: half the tiles the GPU runs at once, 3 M
+//   elements at the default shape) go through lamb_oneshot_kernel, one tile per workgroup.  A workgroup runs pass 1
+//   on its tile (P-way gradient reduce, m/v update, r, the tile's float64 sums of w^2 and r^2), keeps r in registers
+//   and the old w in LDS, waits until the workgroup that finished the segment's last tile has published the scale,
+//   and writes w from what it kept: 56 bytes per element instead of 68.  (lamb_resident_kernel, a persistent grid that
+//   parks tiles in LDS and retires them a round later, is the older form of the same thing; CCN_LAMB_ONESHOT=0 selects
+//   it.)  No sum is an atomic accumulation: tile sums are stored one by one and added in a fixed order, so results do
+//   not depend on scheduling.
 // the other segments take two streaming passes with a finalize kernel between them:
 //   pass 1   one workgroup per tile of kLambTile elements, one 4-element pack per thread
 //   finalize one workgroup per segment: fixed-order sum of the segment's tile pairs, norms, scale
@@ -397,7 +399,7 @@ __global__ __launch_bounds__(kBlock) void lamb_pass2_f16w_kernel(float* w, uint1
   }
 }
 
-// ---- segment-resident variant ----------------------------------------------------------------------------------------
+// ---- segment-resident variant, persistent form ----------------------------------------------------------------------
 // A persistent grid that is resident as a whole walks the tiles of the "resident" segments round-robin.  A workgroup
 // runs pass 1 on a tile, parks the tile's r and old w in LDS, and retires the tile one round later, when the
 // segment's scale is known: pass 2 then reads nothing from memory.  The workgroup that finishes a segment's last tile
@@ -408,6 +410,8 @@ __global__ __launch_bounds__(kBlock) void lamb_pass2_f16w_kernel(float* w, uint1
 // with tiles of a segment whose other tiles it has yet to start.
 constexpr int kResDepth = 2;   // parking slots per workgroup
 constexpr int kResSub = 4;     // packs per thread per tile
+constexpr int kOneshotSub = 8;
+constexpr int kOneshotBlock = 256; // the same for the one-tile-per-workgroup kernel
 // Arrival counters.  Device-scope atomics on one address are served one after the other (some 15 ns each, measured),
 // so a segment's tiles count into kResFan counters, each on a cache line of its own, and the tile that completes one
 // of them counts into the segment's top counter.
@@ -630,6 +634,134 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
   }
 }
 
+// ---- one tile per workgroup, no persistent loop ----------------------------------------------------------------------
+// The same protocol with the hardware's dispatcher in place of the round-robin walk: workgroup b runs pass 1 on tile b
+// (SUB packs per thread), keeps the tile's r in registers and its old w in LDS, counts itself in, waits (within the spin
+// limit) for the segment's scale and writes w.  Workgroups are dispatched in tile order, so the tiles a waiting
+// workgroup depends on are already running; a tile that runs out of patience goes onto the deferred list as above.
+template <int P, int BS, int SUB, bool SCAT>
+__global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void lamb_oneshot_kernel(const SrcTable<float, (P ? P : CCN_MAX_RANKS)> g, const int nP,
+                                                          float* w, float* m, float* v, const LambLayout lay,
+                                                          double* partials, const uint64_t* __restrict__ seg_len,
+                                                          double* norms, float* scale, const LambResident rs,
+                                                          const int vec_ok, const LambPrm k) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  Pack<float, 4>* wpark = reinterpret_cast<Pack<float, 4>*>(smem);
+  double* red = reinterpret_cast<double*>(smem + (size_t)SUB * BS * sizeof(Pack<float, 4>));
+  uint32_t* bc = reinterpret_cast<uint32_t*>(red + 2 * kBlock / kWave);   // [0] last tile of its segment, [1] ready, [2] scale
+  const unsigned tile = blockIdx.x;
+  const LambTile t = lamb_tile_of(lay, tile);
+  SrcTable<float, (P ? P : CCN_MAX_RANKS)> gt;
+  float* wt;
+  lamb_buffers_of<P, SCAT>(lay, g, w, nP, t.seg, gt, wt);
+  Pack<float, 4> rpark[SUB];
+  double accW = 0.0, accR = 0.0;
+  const bool fast = P > 0 && vec_ok && (t.start & 3u) == 0 && t.count == (uint32_t)(BS * 4 * SUB);
+  if (fast) {
+    LambIn<P, 4> cur;
+    lamb_pass1_load<P, 4>(cur, gt, nP, wt, m, v, t.start + threadIdx.x * 4);
+#pragma unroll
+    for (int u = 0; u < SUB; u++) {
+      const size_t e0 = t.start + (size_t)(u * BS + threadIdx.x) * 4;
+      LambIn<P, 4> nxt;
+      if (u + 1 < SUB) lamb_pass1_load<P, 4>(nxt, gt, nP, wt, m, v, e0 + BS * 4);
+      Pack<float, 4> w4;
+      lamb_pass1_math<P, 4>(cur, nP, m, v, e0, t.nf, k, accW, accR, rpark[u], w4);
+      wpark[u * BS + threadIdx.x] = w4;
+      if (u + 1 < SUB) cur = nxt;
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < SUB; u++) {
+      const uint32_t j0 = (u * BS + threadIdx.x) * 4;
+      Pack<float, 4> r4 = {}, w4 = {};
+      if (j0 < t.count) {
+        if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+          lamb_pass1_pack<P, 4>(gt, nP, wt, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (j0 + e < t.count) {
+              Pack<float, 1> r1, w1;
+              lamb_pass1_pack<P, 1>(gt, nP, wt, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
+              r4.d[e] = r1.d[0];
+              w4.d[e] = w1.d[0];
+            }
+          }
+        }
+      }
+      rpark[u] = r4;
+      wpark[u * BS + threadIdx.x] = w4;
+    }
+  }
+  const double sW = group_sum<BS>(accW, red);
+  const double sR = group_sum<BS>(accR, red + kBlock / kWave);
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile,
+                       (unsigned long long)__double_as_longlong(sW), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile + 1,
+                       (unsigned long long)__double_as_longlong(sR), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    drain_vector_memory();   // the sums are in place before the count says so
+    const uint32_t seg_lo = rs.seg_tile_begin[t.seg];
+    const uint32_t seg_tiles = rs.seg_tile_begin[t.seg + 1] - seg_lo;
+    const uint32_t f = (tile - seg_lo) % kResFan;
+    const uint32_t fan_target = (seg_tiles - f + kResFan - 1) / kResFan;
+    const uint32_t arrived = __hip_atomic_fetch_add(&rs.cnt[(size_t)t.seg * kResCntStride + (1 + f) * kResCntLine], 1u,
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+    uint32_t last = 0;
+    if (arrived == fan_target) {
+      const uint32_t fans = seg_tiles < (uint32_t)kResFan ? seg_tiles : (uint32_t)kResFan;
+      last = __hip_atomic_fetch_add(&rs.cnt[(size_t)t.seg * kResCntStride], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 ==
+             fans;
+    }
+    bc[0] = last;
+  }
+  __syncthreads();
+  if (bc[0]) {
+    const float sc = lamb_finalize_segment<BS, true>(partials, rs.seg_tile_begin[t.seg], rs.seg_tile_begin[t.seg + 1],
+                                                     seg_len[t.seg], (int)t.seg, norms, scale, k.mode, red);
+    if (threadIdx.x == 0)
+      __hip_atomic_store(&rs.ready[t.seg], (1ull << 32) | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (threadIdx.x == 0) {
+    uint32_t budget = rs.spin_limit;
+    unsigned long long word;
+    while (((word = __hip_atomic_load(&rs.ready[t.seg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
+      if (budget == 0) break;
+      budget--;
+      __builtin_amdgcn_s_sleep(32);
+    }
+    if ((word >> 32) == 0) {
+      const uint32_t at = __hip_atomic_fetch_add(rs.ndeferred, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      rs.deferred[at] = tile;
+    }
+    bc[1] = (uint32_t)(word >> 32);
+    bc[2] = (uint32_t)word;
+  }
+  __syncthreads();
+  if (!bc[1]) return;
+  const float step_scale = k.lr * __uint_as_float(bc[2]);
+#pragma unroll
+  for (int u = 0; u < SUB; u++) {
+    const uint32_t j0 = (u * BS + threadIdx.x) * 4;
+    if (j0 >= t.count) continue;
+    Pack<float, 4> wv = wpark[u * BS + threadIdx.x];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float x = step_scale * rpark[u].d[e];
+      wv.d[e] = wv.d[e] - x;
+    }
+    if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
+      store_stream<float, 4>(wt + t.start + j0, wv);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (j0 + e < t.count) wt[t.start + j0 + e] = wv.d[e];
+      }
+    }
+  }
+}
+
 // Finishes the deferred tiles: pass 2 from the stored m and v, as the two-pass path does.
 template <int BS, int SUB, bool SCAT>
 __global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, const float* m, const float* v, const LambLayout lay,
@@ -699,6 +831,7 @@ struct ccn_lamb_plan {
   int ptr_ranks = 0;
   // fp16 gradients: a plan over the same segments with every segment on the two-pass path; made on first use
   ccn_lamb_plan* two_pass_twin = nullptr;
+  bool oneshot = false;   // resident segments run lamb_oneshot_kernel (one tile per workgroup) instead of the persistent kernel
 };
 
 namespace {
@@ -753,6 +886,18 @@ int resident_occupancy(int P, int block, int sub, unsigned lds) {
   return occ;
 }
 
+int oneshot_occupancy(int P, unsigned lds) {
+  int occ = 0;
+  with_rank_count(P, [&](auto ptag) {
+    auto* fn = lamb_oneshot_kernel<decltype(ptag)::value, kOneshotBlock, kOneshotSub, false>;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, kOneshotBlock, lds) != hipSuccess) {
+      (void)hipGetLastError();
+      occ = 0;
+    }
+  });
+  return occ;
+}
+
 // Cuts segment b into tiles of `tile` elements appended to `out`.
 void cut_segment(std::vector<LambTile>& out, const size_t* seg_offsets, int b, uint64_t tile) {
   const uint64_t n = seg_offsets[b + 1] - seg_offsets[b];
@@ -793,16 +938,20 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
 
-  // Shape of the resident kernel.  CCN_LAMB_RESIDENT=0 sends every segment down the two-pass path;
-  // CCN_LAMB_RES_BLOCK (64 | 256), CCN_LAMB_RES_WGS (workgroups per CU) and CCN_LAMB_SPIN are for tuning and tests.
+  // Shape of the resident kernels.  CCN_LAMB_RESIDENT=0 sends every segment down the two-pass path; CCN_LAMB_ONESHOT=0
+  // selects the persistent kernel instead of the one-tile-per-workgroup kernel; CCN_LAMB_RES_BLOCK (64 | 256) and
+  // CCN_LAMB_RES_WGS (workgroups per CU) shape the persistent kernel; CCN_LAMB_SPIN bounds the waits of both.  All of
+  // them are for tuning and tests.
   const bool resident_wanted = !two_pass_only && env_long("CCN_LAMB_RESIDENT", 1) != 0;
   int res_block = (int)env_long("CCN_LAMB_RES_BLOCK", kBlock);
   if (res_block != kWave && res_block != kBlock) res_block = kBlock;
-  const int res_sub = kResSub;
+  const bool oneshot = resident_wanted && env_long("CCN_LAMB_ONESHOT", 1) != 0;
+  if (oneshot) res_block = kOneshotBlock;
+  const int res_sub = oneshot ? kOneshotSub : kResSub;
   int lds_limit = 0;
   if (hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, di->device) != hipSuccess) lds_limit = 65536;
-  auto lds_need = [&](int bs) {
-    return (size_t)kResDepth * bs * 4 * res_sub * 8 + 2 * (kBlock / kWave) * sizeof(double) + 16;
+  auto lds_need = [&](int bs) {   // parked packs (r and w in two slots, or w alone), the reduction scratch, three flags
+    return (oneshot ? (size_t)bs * res_sub * 16 : (size_t)kResDepth * bs * 4 * res_sub * 8) + 2 * (kBlock / kWave) * sizeof(double) + 16;
   };
   if (lds_need(res_block) > (size_t)lds_limit) res_block = kWave;
   const uint64_t res_tile = (uint64_t)res_block * 4 * res_sub;
@@ -819,15 +968,24 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   // in blocks): shrink the request until res_wgs fit, or settle for the workgroups that do.
   unsigned res_lds = (unsigned)((kLdsPerCu / (size_t)res_wgs) & ~(size_t)1023);
   if (res_lds > (unsigned)lds_limit) res_lds = (unsigned)lds_limit;
-  int occ = resident_occupancy(8, res_block, res_sub, res_lds);
-  while (occ > 0 && occ < res_wgs && res_lds >= res_need + 1024) {
-    res_lds -= 1024;
+  int occ = 0;
+  if (oneshot) {   // registers, not LDS, decide how many of these share a CU
+    res_lds = (unsigned)((res_need + 1023) & ~(size_t)1023);
+    occ = oneshot_occupancy(8, res_lds);
+    res_wgs = occ;
+  } else {
     occ = resident_occupancy(8, res_block, res_sub, res_lds);
+    while (occ > 0 && occ < res_wgs && res_lds >= res_need + 1024) {
+      res_lds -= 1024;
+      occ = resident_occupancy(8, res_block, res_sub, res_lds);
+    }
+    if (occ > 0 && occ < res_wgs) res_wgs = occ;
   }
-  if (occ > 0 && occ < res_wgs) res_wgs = occ;
   const bool resident_ok = occ > 0;
   const unsigned res_grid_full = (unsigned)di->cu_count * (unsigned)res_wgs;
-  const uint64_t res_cap_tiles = (uint64_t)kResDepth * res_grid_full;
+  // Tiles a resident segment may have: what the persistent grid can park, or half of what the GPU runs at once of the
+  // one-tile workgroups (a segment's waiting tiles must leave room for the ones that complete it).
+  const uint64_t res_cap_tiles = oneshot ? res_grid_full / 2 : (uint64_t)kResDepth * res_grid_full;
 
   std::vector<LambTile> tiles, rtiles;
   std::vector<uint32_t> begin((size_t)nseg + 1), rbegin((size_t)nseg + 1);
@@ -884,6 +1042,7 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   p->res_uniform_seg_len = (all_resident && uniform % res_tile == 0) ? uniform : 0;
   p->res_grid = p->res_ntiles < res_grid_full ? p->res_ntiles : res_grid_full;
   p->res_lds = res_lds;
+  p->oneshot = oneshot;
   p->spin_limit = (uint32_t)env_long("CCN_LAMB_SPIN", 1 << 15);
   hipError_t e = hipSuccess;
   auto alloc = [&](void** ptr, size_t bytes) { if (e == hipSuccess) e = hipMalloc(ptr, bytes ? bytes : 16); };
@@ -1035,6 +1194,21 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
     hipLaunchKernelGGL(lamb_reset_kernel, dim3((unsigned)((plan->nseg + kBlock - 1) / kBlock)), block, 0, s, rs.cnt, rs.ready,
                        plan->nseg, rs.ndeferred);
     CCN_HIP(hipGetLastError());
+    if (plan->oneshot) {
+      with_ranks([&](auto ptag) {
+        constexpr int PP = decltype(ptag)::value;
+        const auto tbl = table(ptag);
+        hipLaunchKernelGGL((scattered ? lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, true> : lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, false>),
+                           dim3(plan->res_ntiles), dim3(kOneshotBlock), plan->res_lds, s, tbl, P, w, m, v, lay, plan->rpartials,
+                           (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
+      });
+      CCN_HIP(hipGetLastError());
+      const unsigned dg = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
+      hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<kOneshotBlock, kOneshotSub, true> : lamb_deferred_kernel<kOneshotBlock, kOneshotSub, false>),
+                         dim3(dg), dim3(kOneshotBlock), 0, s, w, (const float*)m, (const float*)v, lay, (const float*)plan->scale,
+                         (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred, vec_ok, k);
+      CCN_HIP(hipGetLastError());
+    } else {
     // The wait in the kernel is bounded either way, but it only pays when the whole grid is resident.
     if (plan->occupancy[P] == 0) plan->occupancy[P] = resident_occupancy(P, plan->res_block, plan->res_sub, plan->res_lds);
     const int occ = plan->occupancy[P];
@@ -1067,6 +1241,7 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
                          vec_ok, k);
     });
     CCN_HIP(hipGetLastError());
+    }
   }
 
   if (plan->ntiles) {

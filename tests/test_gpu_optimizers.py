@@ -395,21 +395,24 @@ def _lamb_compare(ccn, g, w0, segs, lr, b1, b2, eps, wd_, steps, mode, what, m0=
     return ulp_diff_f32(gw, w)
 
 
-# How a plan runs its segments is fixed when the plan is created, from these variables: the segment-resident kernel
-# with 256-thread or single-wavefront workgroups, the same with a spin limit of zero (every tile whose segment is
-# not ready at the first poll goes through the deferred list), or the two-pass kernels only.
+# How a plan runs its segments is fixed when the plan is created, from these variables: the one-tile-per-workgroup
+# kernel (the default), the persistent segment-resident kernel with 256-thread or single-wavefront workgroups, each of
+# them also with a spin limit of zero (every tile whose segment is not ready at the first poll goes through the
+# deferred list), or the two-pass kernels only.
 LAMB_VARIANTS = {
-    "resident": {},
-    "resident-wave": {"CCN_LAMB_RES_BLOCK": "64"},
-    "deferred": {"CCN_LAMB_SPIN": "0"},
-    "deferred-wave": {"CCN_LAMB_SPIN": "0", "CCN_LAMB_RES_BLOCK": "64"},
+    "one-tile": {},
+    "one-tile-deferred": {"CCN_LAMB_SPIN": "0"},
+    "resident": {"CCN_LAMB_ONESHOT": "0"},
+    "resident-wave": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_RES_BLOCK": "64"},
+    "deferred": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0"},
+    "deferred-wave": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0", "CCN_LAMB_RES_BLOCK": "64"},
     "two-pass": {"CCN_LAMB_RESIDENT": "0"},
 }
 
 
 @pytest.fixture(params=list(LAMB_VARIANTS))
 def lamb_variant(request, monkeypatch):
-    for k in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS"):
+    for k in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT"):
         monkeypatch.delenv(k, raising=False)
     for k, val in LAMB_VARIANTS[request.param].items():
         monkeypatch.setenv(k, val)
@@ -457,12 +460,16 @@ def test_lamb_unaligned_buffers(ccn, lamb_variant):
     assert ulp_diff_f32(host(wd), w) <= 2
 
 
-def test_lamb_mixed_resident_and_two_pass(ccn, monkeypatch):
-    """One segment too long to stay on chip (one workgroup per CU: 2 * 256 tiles of 4096 elements at most) between
-    short ones: the long one takes the two-pass kernels, the others the resident kernel, in one call."""
-    monkeypatch.setenv("CCN_LAMB_RES_WGS", "1")
+@pytest.mark.parametrize("kernel,long_seg", [("one-tile", 4_000_000), ("persistent", 2_500_000)])
+def test_lamb_mixed_resident_and_two_pass(ccn, monkeypatch, kernel, long_seg):
+    """One segment too long to stay on chip between short ones: the long one takes the two-pass kernels, the others
+    the resident kernel, in one call.  The one-tile kernel keeps segments of up to half the tiles the GPU runs at once
+    (384 tiles of 8192 elements); the persistent kernel, held to one workgroup per CU here, 2 * 256 tiles of 4096."""
+    if kernel == "persistent":
+        monkeypatch.setenv("CCN_LAMB_ONESHOT", "0")
+        monkeypatch.setenv("CCN_LAMB_RES_WGS", "1")
     P = 2
-    segs = [0, 3000, 3000 + 2_500_000, 3000 + 2_500_000 + 8192, 3000 + 2_500_000 + 8192 + 100_001]
+    segs = [0, 3000, 3000 + long_seg, 3000 + long_seg + 8192, 3000 + long_seg + 8192 + 100_001]
     N = segs[-1]
     g = grads_f32(72, P, N, 1e-3)
     w0 = weights_f32(72, N, 0.05)
