@@ -198,13 +198,13 @@ def main():
             step = lambda t: capi.sgd_f32(g, w, N, 0.01, stream)
             kernel = "fused_stream_kernel<SgdMath, %d, 4, 1, %d>" % (P if P <= 8 else 0, 256 if P + 2 <= 3 else 64)
         elif wl == "lamb_nccl_f16g":
-            # the modified NCCL's mixed-precision LAMB, 256 segments; runs the two-pass kernels
+            # the modified NCCL's mixed-precision LAMB, 256 segments
             w16 = bufs.from_tensor(torch.empty(N, dtype=torch.float16, device="cuda"))
             nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
             plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
             per_param = P * 2 + 12 + 12 + 2
             step = lambda t: plan.step_nccl_f16g(g, w, w16, m, v, 1e-3, 0.9, 0.999, 1.0, stream)
-            kernel = "lamb_pass1_f16g_kernel<%d> + lamb_finalize_kernel + lamb_pass2_f16w_kernel" % (P if P <= 8 else 0)
+            kernel = "lamb_reset_kernel + lamb_oneshot_kernel<%d, 256, 8, false, uint16_t> + lamb_deferred_kernel<256, 8, false, true>" % (P if P <= 8 else 0)
         elif gbytes == 2:
             w16 = bufs.from_tensor(torch.empty(N, dtype=half, device="cuda"))
             flag = torch.zeros(1, dtype=torch.int32, device="cuda")

@@ -639,9 +639,10 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
 // (SUB packs per thread), keeps the tile's r in registers and its old w in LDS, counts itself in, waits (within the spin
 // limit) for the segment's scale and writes w.  Workgroups are dispatched in tile order, so the tiles a waiting
 // workgroup depends on are already running; a tile that runs out of patience goes onto the deferred list as above.
-template <int P, int BS, int SUB, bool SCAT>
-__global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void lamb_oneshot_kernel(const SrcTable<float, (P ? P : CCN_MAX_RANKS)> g, const int nP,
-                                                          float* w, float* m, float* v, const LambLayout lay,
+// G = uint16_t: fp16 gradients and an fp16 copy of the new weights in halfw (flat arrays only).
+template <int P, int BS, int SUB, bool SCAT, class G = float>
+__global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void lamb_oneshot_kernel(const SrcTable<G, (P ? P : CCN_MAX_RANKS)> g, const int nP,
+                                                          float* w, uint16_t* halfw, float* m, float* v, const LambLayout lay,
                                                           double* partials, const uint64_t* __restrict__ seg_len,
                                                           double* norms, float* scale, const LambResident rs,
                                                           const int vec_ok, const LambPrm k) {
@@ -651,22 +652,29 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
   uint32_t* bc = reinterpret_cast<uint32_t*>(red + 2 * kBlock / kWave);   // [0] last tile of its segment, [1] ready, [2] scale
   const unsigned tile = blockIdx.x;
   const LambTile t = lamb_tile_of(lay, tile);
-  SrcTable<float, (P ? P : CCN_MAX_RANKS)> gt;
+  constexpr bool kHalf = std::is_same<G, uint16_t>::value;
+  static_assert(!(kHalf && SCAT), "fp16 gradients come in flat arrays");
+  SrcTable<G, (P ? P : CCN_MAX_RANKS)> gt;
   float* wt;
-  lamb_buffers_of<P, SCAT>(lay, g, w, nP, t.seg, gt, wt);
+  if constexpr (SCAT) {
+    lamb_buffers_of<P, SCAT>(lay, g, w, nP, t.seg, gt, wt);
+  } else {
+    gt = g;
+    wt = w;
+  }
   Pack<float, 4> rpark[SUB];
   double accW = 0.0, accR = 0.0;
   const bool fast = P > 0 && vec_ok && (t.start & 3u) == 0 && t.count == (uint32_t)(BS * 4 * SUB);
   if (fast) {
-    LambIn<P, 4> cur;
-    lamb_pass1_load<P, 4>(cur, gt, nP, wt, m, v, t.start + threadIdx.x * 4);
+    LambIn<P, 4, G> cur;
+    lamb_pass1_load<P, 4, G>(cur, gt, nP, wt, m, v, t.start + threadIdx.x * 4);
 #pragma unroll
     for (int u = 0; u < SUB; u++) {
       const size_t e0 = t.start + (size_t)(u * BS + threadIdx.x) * 4;
-      LambIn<P, 4> nxt;
-      if (u + 1 < SUB) lamb_pass1_load<P, 4>(nxt, gt, nP, wt, m, v, e0 + BS * 4);
+      LambIn<P, 4, G> nxt;
+      if (u + 1 < SUB) lamb_pass1_load<P, 4, G>(nxt, gt, nP, wt, m, v, e0 + BS * 4);
       Pack<float, 4> w4;
-      lamb_pass1_math<P, 4>(cur, nP, m, v, e0, t.nf, k, accW, accR, rpark[u], w4);
+      lamb_pass1_math<P, 4, G>(cur, nP, m, v, e0, t.nf, k, accW, accR, rpark[u], w4);
       wpark[u * BS + threadIdx.x] = w4;
       if (u + 1 < SUB) cur = nxt;
     }
@@ -677,13 +685,13 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
       Pack<float, 4> r4 = {}, w4 = {};
       if (j0 < t.count) {
         if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-          lamb_pass1_pack<P, 4>(gt, nP, wt, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
+          lamb_pass1_pack<P, 4, G>(gt, nP, wt, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; e++) {
             if (j0 + e < t.count) {
               Pack<float, 1> r1, w1;
-              lamb_pass1_pack<P, 1>(gt, nP, wt, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
+              lamb_pass1_pack<P, 1, G>(gt, nP, wt, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
               r4.d[e] = r1.d[0];
               w4.d[e] = w1.d[0];
             }
@@ -753,18 +761,27 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
     }
     if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
       store_stream<float, 4>(wt + t.start + j0, wv);
+      if constexpr (kHalf) {
+        Pack<uint16_t, 4> hv;
+#pragma unroll
+        for (int e = 0; e < 4; e++) hv.d[e] = f32_to_f16_bits(wv.d[e]);
+        store_stream<uint16_t, 4>(halfw + t.start + j0, hv);
+      }
     } else {
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        if (j0 + e < t.count) wt[t.start + j0 + e] = wv.d[e];
+        if (j0 + e < t.count) {
+          wt[t.start + j0 + e] = wv.d[e];
+          if constexpr (kHalf) halfw[t.start + j0 + e] = f32_to_f16_bits(wv.d[e]);
+        }
       }
     }
   }
 }
 
 // Finishes the deferred tiles: pass 2 from the stored m and v, as the two-pass path does.
-template <int BS, int SUB, bool SCAT>
-__global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, const float* m, const float* v, const LambLayout lay,
+template <int BS, int SUB, bool SCAT, bool HALF = false>
+__global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, uint16_t* halfw, const float* m, const float* v, const LambLayout lay,
                                                            const float* __restrict__ scale,
                                                            const uint32_t* __restrict__ deferred,
                                                            const uint32_t* __restrict__ ndeferred, const int vec_ok,
@@ -778,10 +795,10 @@ __global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, const float
       const uint32_t j0 = (u * BS + threadIdx.x) * 4;
       if (j0 >= t.count) continue;
       if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-        lamb_pass2_pack<4>(wt, m, v, t.start + j0, step_scale, k);
+        lamb_pass2_pack<4, HALF>(wt, m, v, t.start + j0, step_scale, k, halfw);
       } else {
         const uint32_t j1 = j0 + 4 < t.count ? j0 + 4 : t.count;
-        for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1>(wt, m, v, t.start + j, step_scale, k);
+        for (uint32_t j = j0; j < j1; j++) lamb_pass2_pack<1, HALF>(wt, m, v, t.start + j, step_scale, k, halfw);
       }
     }
   }
@@ -1199,13 +1216,13 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
         constexpr int PP = decltype(ptag)::value;
         const auto tbl = table(ptag);
         hipLaunchKernelGGL((scattered ? lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, true> : lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, false>),
-                           dim3(plan->res_ntiles), dim3(kOneshotBlock), plan->res_lds, s, tbl, P, w, m, v, lay, plan->rpartials,
+                           dim3(plan->res_ntiles), dim3(kOneshotBlock), plan->res_lds, s, tbl, P, w, (uint16_t*)nullptr, m, v, lay, plan->rpartials,
                            (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
       });
       CCN_HIP(hipGetLastError());
       const unsigned dg = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
       hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<kOneshotBlock, kOneshotSub, true> : lamb_deferred_kernel<kOneshotBlock, kOneshotSub, false>),
-                         dim3(dg), dim3(kOneshotBlock), 0, s, w, (const float*)m, (const float*)v, lay, (const float*)plan->scale,
+                         dim3(dg), dim3(kOneshotBlock), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v, lay, (const float*)plan->scale,
                          (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred, vec_ok, k);
       CCN_HIP(hipGetLastError());
     } else {
@@ -1236,7 +1253,7 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
       constexpr int BS = decltype(bstag)::value;
       constexpr int SUB = decltype(subtag)::value;
       hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<BS, SUB, true> : lamb_deferred_kernel<BS, SUB, false>), dim3(dgrid),
-                         dim3(BS), 0, s, w, (const float*)m, (const float*)v,
+                         dim3(BS), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v,
                          lay, (const float*)plan->scale, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
                          vec_ok, k);
     });
@@ -1294,14 +1311,6 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
   if (di->device != plan->device) return CCN_EINVAL;
-  if (!plan->two_pass_twin) {
-    std::vector<size_t> offs(plan->seg_start.begin(), plan->seg_start.end());
-    offs.push_back(plan->N);
-    rc = lamb_plan_create(offs.data(), plan->nseg, true, &plan->two_pass_twin);
-    if (rc != CCN_OK) return rc;
-  }
-  ccn_lamb_plan* tp = plan->two_pass_twin;
-
   LambPrm k;
   k.b1 = beta1;
   k.omb1 = 1 - beta1;
@@ -1312,12 +1321,58 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
   k.lr = lr;
   k.mode = CCN_LAMB_NCCL_GLOBAL;
   k.bc1 = k.bc2 = 1.0;
-
   bool al = aligned16(w) && aligned16(m) && aligned16(v) && (reinterpret_cast<uintptr_t>(halfw) & 7u) == 0;
   for (int p = 0; p < P; p++) al = al && (reinterpret_cast<uintptr_t>(g[p]) & 7u) == 0;
   const int vec_ok = al ? 1 : 0;
   hipStream_t s = as_stream(stream);
-  const dim3 grid((unsigned)tp->ntiles), block(kBlock);
+  const dim3 block(kBlock);
+
+  // Every segment short enough to stay on chip: the one-tile kernel, as for fp32 gradients.
+  if (plan->oneshot && plan->ntiles == 0 && plan->res_ntiles) {
+    LambLayout lay;
+    lay.tiles = plan->rtiles;
+    lay.seg_len = plan->res_uniform_seg_len;
+    lay.seg_len_f = (float)plan->res_uniform_seg_len;
+    lay.tile = (uint32_t)(plan->res_block * 4 * plan->res_sub);
+    lay.gtab = nullptr;
+    lay.wtab = nullptr;
+    lay.nseg = (uint32_t)plan->nseg;
+    LambResident rs;
+    rs.cnt = plan->sync;
+    rs.ndeferred = plan->sync + (size_t)plan->nseg * kResCntStride;
+    rs.ready = plan->ready;
+    rs.seg_tile_begin = plan->seg_rtile_begin;
+    rs.deferred = plan->deferred;
+    rs.ntiles = plan->res_ntiles;
+    rs.spin_limit = plan->spin_limit;
+    hipLaunchKernelGGL(lamb_reset_kernel, dim3((unsigned)((plan->nseg + kBlock - 1) / kBlock)), block, 0, s, rs.cnt, rs.ready,
+                       plan->nseg, rs.ndeferred);
+    CCN_HIP(hipGetLastError());
+    with_rank_count(P, [&](auto ptag) {
+      constexpr int PP = decltype(ptag)::value;
+      SrcTable<uint16_t, (PP ? PP : CCN_MAX_RANKS)> tbl;
+      for (int p = 0; p < (PP ? PP : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < P ? p : 0];
+      hipLaunchKernelGGL((lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, false, uint16_t>), dim3(plan->res_ntiles),
+                         dim3(kOneshotBlock), plan->res_lds, s, tbl, P, w, halfw, m, v, lay, plan->rpartials,
+                         (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
+    });
+    CCN_HIP(hipGetLastError());
+    const unsigned dg = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
+    hipLaunchKernelGGL((lamb_deferred_kernel<kOneshotBlock, kOneshotSub, false, true>), dim3(dg), dim3(kOneshotBlock), 0, s, w,
+                       halfw, (const float*)m, (const float*)v, lay, (const float*)plan->scale,
+                       (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred, vec_ok, k);
+    CCN_HIP(hipGetLastError());
+    return CCN_OK;
+  }
+
+  if (!plan->two_pass_twin) {
+    std::vector<size_t> offs(plan->seg_start.begin(), plan->seg_start.end());
+    offs.push_back(plan->N);
+    rc = lamb_plan_create(offs.data(), plan->nseg, true, &plan->two_pass_twin);
+    if (rc != CCN_OK) return rc;
+  }
+  ccn_lamb_plan* tp = plan->two_pass_twin;
+  const dim3 grid((unsigned)tp->ntiles);
   LambLayout lay;
   lay.tiles = tp->tiles;
   lay.seg_len = vec_ok ? tp->uniform_seg_len : 0;

@@ -178,8 +178,9 @@ int  ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, f
  * wd in place of the hard-coded 1.0f, no eps, no step).  g: HOST array of P device pointers to fp16 bit patterns.
  * Replaces AllReduce_pipe(lr, beta1, beta2, (half*)g, w, halfw, m, v, r, ...) of nccl/src/nccl.h.in:211-216 for the
  * LAMB build (phase 1 nccl/src/collectives/device/common_kernel.h:2438-2535, phase 2 :2657-2700); the caller's r
- * buffer is not needed: phase 2 recomputes r from the stored m and v.  Runs the two-pass kernels (a second tile table
- * over the same segments is made on the first call, which therefore allocates and cannot be recorded). */
+ * buffer is not needed: r stays on chip, or phase 2 recomputes it from the stored m and v.  A plan whose segments all fit
+ * on chip runs the one-tile kernel, as for fp32 gradients; any other plan runs the two-pass kernels over all its
+ * segments (a second tile table is then made on the first call, which therefore allocates and cannot be recorded). */
 int  ccn_lamb_nccl_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
                         float lr, float beta1, float beta2, float wd, void* stream);
 /* copies W_b, R_b of the last LAMB step on this plan to a HOST array of 2*nseg doubles (synchronises) */

@@ -677,11 +677,20 @@ def test_lamb_resident_kernel_shares_the_gpu(ccn):
 @pytest.mark.parametrize("P,segs,shift", [(8, [0, 1 << 18], 0), (3, [0, 700, 701, 5000, 8192 + 3], 0),
                                           (8, [0, 4096, 8192, 12288], 0), (11, [0, 1000, 70001], 0),
                                           (2, [0, 4099], 1), (1, [0, 1], 0), (8, [0, 5 * 1024 * 4096 + 17], 0)])
-def test_lamb_nccl_mixed_precision(ccn, P, segs, shift):
+@pytest.mark.parametrize("path", ["one-tile", "one-tile-deferred", "two-pass"])
+def test_lamb_nccl_mixed_precision(ccn, monkeypatch, P, segs, shift, path):
     """The modified NCCL's LAMB with fp16 gradients: m and v bit for bit, w within the fp32 bar (the order of the
     float64 norm sums differs), the fp16 weight copy within one fp16 ulp and equal to fp16 of the kernel's own w.
     shift = 1: every array starts one element past an aligned address (scalar path).  The last case has a segment of
-    more than 4096 tiles (the partial sums are folded in two levels)."""
+    more than 4096 tiles: it takes the two-pass kernels whatever the path, with its partial sums folded in two levels."""
+    for name in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT"):
+        monkeypatch.delenv(name, raising=False)
+    if path == "one-tile-deferred":
+        monkeypatch.setenv("CCN_LAMB_SPIN", "0")
+    if path == "two-pass":
+        monkeypatch.setenv("CCN_LAMB_RESIDENT", "0")
+    if path != "one-tile" and segs[-1] > (1 << 22):
+        pytest.skip("the long segment takes the two-pass kernels in every path: run once")
     N = segs[-1]
     g16 = [orc.f32_to_f16(x) for x in grads_f32(71 + P, P, N, 0.5)]
     w0 = weights_f32(71, N, 0.05)
