@@ -732,7 +732,7 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
       __hip_atomic_store(&rs.ready[t.seg], (1ull << 32) | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (threadIdx.x == 0) {
-    uint32_t budget = rs.spin_limit;
+    uint32_t budget = rs.spin_limit / 4;   // polls are four times as far apart as in the persistent kernel
     unsigned long long word;
     while (((word = __hip_atomic_load(&rs.ready[t.seg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
       if (budget == 0) break;
