@@ -430,6 +430,25 @@ def test_lamb_ragged_segments(ccn, mode, lamb_variant):
     assert ulps <= 2
 
 
+@pytest.mark.parametrize("P", [1, 5, 7, 9, 16])
+@pytest.mark.parametrize("path", ["one-tile", "persistent", "two-pass"])
+def test_lamb_rank_counts(ccn, monkeypatch, P, path):
+    """Every rank count has its own instantiation up to 8 and a looped one beyond; segments around the 8192-element
+    tile of the one-tile kernel."""
+    for name in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT"):
+        monkeypatch.delenv(name, raising=False)
+    if path == "persistent":
+        monkeypatch.setenv("CCN_LAMB_ONESHOT", "0")
+    if path == "two-pass":
+        monkeypatch.setenv("CCN_LAMB_RESIDENT", "0")
+    segs = [0, 8192, 8192 + 8191, 3 * 8192 + 5, 5 * 8192 + 5]
+    N = segs[-1]
+    g = grads_f32(40 + P, P, N, 1e-3)
+    w0 = weights_f32(40, N, 0.05)
+    ulps = _lamb_compare(ccn, g, w0, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, 2, 0, f"ranks {P} {path}")
+    assert ulps <= 2
+
+
 def test_lamb_config4_reduced(ccn, lamb_variant):
     # benchmark configuration 4 layout at reduced size: 16 segments of 2^16, P = 8, wd = 0.01, two-pass norm + update
     P, nseg, seglen = 8, 16, 1 << 16
