@@ -837,3 +837,122 @@ def test_cpp_harness_in_the_shape_of_the_reference_sample(which, ranks):
     r = subprocess.run([exe, which, str(ranks)], capture_output=True, text=True, timeout=240)
     assert r.returncode == 0 and "Success" in r.stdout, (r.stdout[-1500:], r.stderr[-500:])
     assert r.stdout.count("weights match the checker") == 5
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+def _placed(a, shift, kind):
+    """Device copy of `a` that starts `shift` elements past an aligned address."""
+    if shift == 0:
+        return dev(a) if kind == "f" else dev_u16(a)
+    pad = np.concatenate([np.zeros(shift, a.dtype), a])
+    return (dev(pad) if kind == "f" else dev_u16(pad))[shift:]
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_seeded_random_shapes(ccn, case):
+    """Seeded random rank counts, sizes, starting alignments and segmentations through every optimizer entry point:
+    the same bits as the oracle (LAMB: m, v the same bits, w within 2 ulp)."""
+    r = rng(1000 + case)
+    P = int(r.integers(1, 17))
+    N = int(r.choice([1, 2, 3, 5, 63, 64, 65, 255, 257, 1023, 4097, 8191, 8193, 40_000, 100_003, 262_147]))
+    shifts = [int(x) for x in r.integers(0, 4, P + 3)] if case % 3 else [0] * (P + 3)
+    op = ["sgd", "adam", "adam16", "lamb", "lamb16"][case % 5]
+    w0 = weights_f32(2000 + case, N, 0.05)
+    m0 = weights_f32(3000 + case, N, 0.01)
+    v0 = np.abs(weights_f32(4000 + case, N, 1e-2)) + np.float32(1e-4)
+    g = grads_f32(5000 + case, P, N, 1e-3)
+    w, m, v = w0.copy(), m0.copy(), v0.copy()
+    wd, md, vd = _placed(w0, shifts[P], "f"), _placed(m0, shifts[P + 1], "f"), _placed(v0, shifts[P + 2], "f")
+    what = f"case {case}: {op} P={P} N={N} shifts={shifts}"
+    if op in ("sgd", "adam", "lamb"):
+        gd = [_placed(x, shifts[p], "f") for p, x in enumerate(g)]
+    else:
+        g16 = [orc.f32_to_f16(x * np.float32(256.0)) for x in g]
+        gd = [_placed(x, shifts[p], "h") for p, x in enumerate(g16)]
+    if op == "sgd":
+        ccn.sgd_f32(gd, wd, N, 0.01)
+        orc.sgd_f32(g, w, 0.01)
+        assert_f32_parity(host(wd), w, what)
+        return
+    if op == "adam":
+        for t in (1, 2):
+            ccn.adam_f32(gd, wd, md, vd, N, 1e-3, 0.9, 0.999, 1e-6, t)
+            orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t)
+    elif op == "adam16":
+        w16d = _placed(np.zeros(N, np.uint16), shifts[0], "h")
+        w16 = np.zeros(N, np.uint16)
+        flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+        for t in (1, 2):
+            ccn.adam_f16g(gd, wd, md, vd, w16d, N, 1e-3, 0.9, 0.999, 1e-6, t, 1.0 / 256.0, flag)
+            want = orc.adam_f16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, t, np.float32(1.0 / 256.0))
+            assert int(host(flag)[0]) == want == 0
+        assert np.array_equal(host_u16(w16d), w16), what
+    else:
+        cuts = sorted(set(int(x) for x in r.integers(1, max(N, 2), min(5, N)) if 0 < x < N))
+        segs = [0] + cuts + [N]
+        plan = ccn.LambPlan(segs)
+        if op == "lamb":
+            mode = int(r.integers(0, 3))
+            eps, wdec = (1e-6, 0.01) if mode != 2 else (0.0, 1.0)
+            for t in (1, 2):
+                plan.step(gd, wd, md, vd, 1e-3, 0.9, 0.999, eps, wdec, t, mode)
+                orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, eps, wdec, t, mode)
+        else:
+            hwd = _placed(np.zeros(N, np.uint16), shifts[0], "h")
+            hw = np.zeros(N, np.uint16)
+            for _ in (1, 2):
+                plan.step_nccl_f16g(gd, wd, hwd, md, vd, 0.01, 0.9, 0.999, 1.0)
+                orc.lamb_nccl_f16g(g16, w, hw, m, v, segs, 0.01, 0.9, 0.999, 1.0)
+            got_w = host(wd)
+            assert np.array_equal(host_u16(hwd), got_w.astype(np.float16).view(np.uint16)), what
+        plan.close()
+        assert_f32_parity(host(md), m, what + " m")
+        assert_f32_parity(host(vd), v, what + " v")
+        got_w = host(wd)
+        assert np.max(np.abs(got_w.astype(np.float64) - w)) <= FP32_TOL * max(float(np.max(np.abs(w))), 1e-30), what
+        return
+    assert_f32_parity(host(wd), w, what + " w")
+    assert_f32_parity(host(md), m, what + " m")
+    assert_f32_parity(host(vd), v, what + " v")
+
+
+@pytest.mark.parametrize("case", range(8))
+def test_seeded_random_scattered_buffers(ccn, case):
+    """Seeded random buffer lists (sizes from one element to a few tiles, some buffers misaligned) through the scattered
+    Adam, SGD and LAMB entry points: the same bits as the oracle on the concatenation."""
+    r = rng(7000 + case)
+    P = int(r.integers(1, 12))
+    nbuff = int(r.integers(1, 60))
+    counts = [int(x) for x in r.choice([1, 2, 3, 4, 100, 255, 256, 257, 1000, 5000, 8192, 20_001], nbuff)]
+    offs = np.concatenate([[0], np.cumsum(counts)])
+    N = int(offs[-1])
+    g = grads_f32(7100 + case, P, N, 1e-3)
+    w0 = weights_f32(7200 + case, N, 0.05)
+    shift = [int(x) for x in r.integers(0, 2, nbuff)]
+
+    def pieces(flat):
+        return [_placed(flat[int(offs[b]):int(offs[b + 1])], shift[b], "f") for b in range(nbuff)]
+
+    gd, wd = [pieces(x) for x in g], pieces(w0)
+    md, vd = torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    plan = ccn.ScatterPlan(counts)
+    for t in (1, 2):
+        plan.adam(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, t)
+        orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t)
+    plan.sgd(gd, wd, 0.01)
+    orc.sgd_f32(g, w, 0.01)
+    plan.close()
+    what = f"case {case}: P={P} counts={counts}"
+    assert_f32_parity(np.concatenate([host(x) for x in wd]), w, what + " w")
+    assert_f32_parity(host(md), m, what + " m")
+    assert_f32_parity(host(vd), v, what + " v")
+    lplan = ccn.LambPlan([int(x) for x in offs])
+    for t in (3, 4):
+        lplan.step_scattered(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+        orc.lamb_f32(g, w, m, v, [int(x) for x in offs], 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+    lplan.close()
+    assert_f32_parity(host(md), m, what + " lamb m")
+    assert_f32_parity(host(vd), v, what + " lamb v")
+    got = np.concatenate([host(x) for x in wd])
+    assert np.max(np.abs(got.astype(np.float64) - w)) <= FP32_TOL * float(np.max(np.abs(w))), what
