@@ -149,3 +149,26 @@ def test_outproj_config5_full_size(ccn):
     # the residual only when the scaled sum rounds away, which is rare)
     dropped = float((out == resid).float().mean())
     assert abs(dropped - 0.1) < 2e-3
+
+
+@pytest.mark.parametrize("case", range(8))
+def test_seeded_random_shapes(ccn, case):
+    """Seeded random tile counts, depths, partial counts, drop rates and seeds through the fused kernel (every count of
+    partial buffers has an instantiation of its own), without a residual in some cases."""
+    r = rng(900 + case)
+    M, N, K = 128 * int(r.integers(1, 4)), 128 * int(r.integers(1, 4)), 64 * int(r.integers(1, 6))
+    nP = case % 9 if case < 8 else 8
+    p = float(r.choice([0.0, 0.1, 0.5]))
+    seed = int(r.integers(0, 1 << 40))
+    with_resid = case % 3 != 0
+    X, W, parts, bias, resid = make_case(950 + case, M, N, K, nP)
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(bf16_dev(X), bf16_dev(W), [torch.from_numpy(q).to(DEV) for q in parts], torch.from_numpy(bias).to(DEV),
+                         bf16_dev(resid) if with_resid else None, out, M, N, K, p, seed)
+    got = bf16_host(out).reshape(M, N)
+    zero = np.zeros_like(resid)
+    want, want_f32 = orc.mlp_outproj(X, W, parts, bias, resid if with_resid else zero, M, N, K, p, seed)
+    keep = orc.dropout_mask(seed, 0, M * N, p).reshape(M, N).astype(bool)
+    assert np.array_equal(got[~keep], (resid if with_resid else zero)[~keep])
+    d = bf16_ulp_distance(got, want)
+    assert d.max() <= 1 and (d > 0).mean() < 0.02, f"case {case}: M={M} N={N} K={K} nP={nP} p={p}: {d.max()} {(d > 0).mean():.4f}"
