@@ -83,19 +83,70 @@ def traffic_from_profiles(name):
     return None
 
 
-def cpu_baseline_adam(P, budget_s=8.0):
-    """The oracle's restatement of the reference checker loop (multi-process-adam-scattered.cpp:112-136 with a
+def cpu_baseline(wl, P, budget_s=8.0):
+    """The oracle's restatement of the reference loops (for Adam: multi-process-adam-scattered.cpp:112-136 with a
     fixed-order P-way sum) on a bounded sample of the same workload: once on one thread, as the reference runs it, and
-    once with the index range cut into one slice per host thread (the loop is elementwise, so the results are the same)."""
+    once with the work cut into one slice per host thread (index ranges, whole segments for LAMB, rows for the MLP:
+    the loops are independent across those, so the results are the same)."""
     import oracle as orc
     from concurrent.futures import ThreadPoolExecutor
-    n = 1 << 24
+    threads = max(1, min(16, os.cpu_count() or 1))     # a one-GPU box gives a job 16 host threads
     r = np.random.Generator(np.random.Philox(key=[5, 0]))
-    g = [(r.standard_normal(n, dtype=np.float32) * np.float32(1e-3)) for _ in range(P)]
-    w = r.uniform(-0.05, 0.05, n).astype(np.float32)
-    m = np.zeros(n, np.float32)
-    v = np.zeros(n, np.float32)
-    orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 1)          # warm the pages
+    f32 = np.float32
+    if wl == "mlp_outproj":
+        # a band of rows of the 8192 x 1024 x 8192 product with its 7 partial buffers
+        rows, Nn, Kd, nP = 8 * threads, 8192, 1024, 7
+        X = orc.f32_to_bf16(r.standard_normal((rows, Kd), dtype=f32))
+        Wm = orc.f32_to_bf16(r.standard_normal((Kd, Nn), dtype=f32) * f32(0.02))
+        parts = [r.standard_normal((rows, Nn), dtype=f32) for _ in range(nP)]
+        bias = r.standard_normal(Nn, dtype=f32)
+        resid = orc.f32_to_bf16(r.standard_normal((rows, Nn), dtype=f32))
+        units, per_unit = rows * Nn, (7 * 4 + 2 + 2) + (Kd * 2 * 2.0) / 8192   # bytes per output, X and W amortised
+        what = f"oracle orc_mlp_outproj on {rows} of the 8192 rows (K=1024, 7 partials, p=0.1)"
+
+        def piece(lo, hi, t):
+            orc.mlp_outproj(X[lo:hi], Wm, [q[lo:hi] for q in parts], bias, resid[lo:hi], hi - lo, Nn, Kd, 0.1, 0)
+        cuts = [rows * k // threads for k in range(threads + 1)]
+    else:
+        n = 1 << 24
+        nseg = 16
+        segs = [k * (n // nseg) for k in range(nseg + 1)]
+        half = wl in ("adam_f16g", "adam_bf16g", "lamb_nccl_f16g")
+        scale = f32(2.0 ** 7 if wl == "adam_bf16g" else 2.0 ** 16 if wl == "adam_f16g" else 1.0)
+        g = [(r.standard_normal(n, dtype=f32) * f32(1e-3)) for _ in range(P)]
+        if half:
+            g = [(orc.f32_to_bf16 if wl == "adam_bf16g" else orc.f32_to_f16)(x * scale) for x in g]
+        w = r.uniform(-0.05, 0.05, n).astype(f32)
+        m = np.zeros(n, f32)
+        v = np.full(n, 1e-6, f32) if wl == "lamb_nccl_f16g" else np.zeros(n, f32)
+        w16 = np.zeros(n, np.uint16)
+        units = n
+        per_unit = {"sgd_f32": (P + 1) * 4 + 4, "adam_f32": (P + 3) * 4 + 12, "adam_f32_scattered": (P + 3) * 4 + 12,
+                    "lamb_f32": (P + 3) * 4 + 12}.get(wl, P * 2 + 12 + 12 + 2)
+        what = f"oracle loop of {wl}, P={P}, N=2^24 sample of the 2^28 workload" + (" in 16 segments" if "lamb" in wl else "")
+
+        def piece(lo, hi, t):
+            gs = [x[lo:hi] for x in g]
+            if wl == "sgd_f32":
+                orc.sgd_f32(gs, w[lo:hi], 0.01)
+            elif wl in ("adam_f32", "adam_f32_scattered"):
+                orc.adam_f32(gs, w[lo:hi], m[lo:hi], v[lo:hi], 1e-3, 0.9, 0.999, 1e-6, t)
+            elif wl == "adam_f16g":
+                orc.adam_f16g(gs, w[lo:hi], m[lo:hi], v[lo:hi], w16[lo:hi], 1e-3, 0.9, 0.999, 1e-6, t, f32(1.0) / scale)
+            elif wl == "adam_bf16g":
+                orc.adam_bf16g(gs, w[lo:hi], m[lo:hi], v[lo:hi], w16[lo:hi], 1e-3, 0.9, 0.999, 1e-6, t, f32(1.0) / scale)
+            else:
+                local = [x - lo for x in segs if lo <= x <= hi]
+                if wl == "lamb_f32":
+                    orc.lamb_f32(gs, w[lo:hi], m[lo:hi], v[lo:hi], local, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+                else:
+                    orc.lamb_nccl_f16g(gs, w[lo:hi], w16[lo:hi], m[lo:hi], v[lo:hi], local, 1e-3, 0.9, 0.999, 1.0)
+        if "lamb" in wl:      # whole segments per thread
+            cuts = [segs[nseg * k // threads] for k in range(threads + 1)]
+        else:
+            cuts = [n * k // threads for k in range(threads + 1)]
+    top = cuts[-1]
+    piece(0, top, 1)          # warm the pages
 
     def timed(step_fn):
         t0 = time.perf_counter()
@@ -105,27 +156,24 @@ def cpu_baseline_adam(P, budget_s=8.0):
             reps += 1
             el = time.perf_counter() - t0
             if el > budget_s or reps >= 400:
-                return el / (reps * n), reps
+                return el / (reps * units), reps
 
-    one, reps1 = timed(lambda t: orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t))
-    threads = max(1, min(16, os.cpu_count() or 1))     # a one-GPU box gives a job 16 host threads
-    cuts = [n * k // threads for k in range(threads + 1)]
+    one, reps1 = timed(lambda t: piece(0, top, t))
     pool = ThreadPoolExecutor(threads)
 
     def sliced(t):
-        jobs = [pool.submit(orc.adam_f32, [x[a:b] for x in g], w[a:b], m[a:b], v[a:b], 1e-3, 0.9, 0.999, 1e-6, t)
-                for a, b in zip(cuts[:-1], cuts[1:])]
+        jobs = [pool.submit(piece, a, b, t) for a, b in zip(cuts[:-1], cuts[1:]) if b > a]
         for j in jobs:
             j.result()
 
     many, repsT = timed(sliced)
     pool.shutdown()
     return {
-        "value": round(56.0 / many / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        "value": round(per_unit / many / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
         "params_per_s": round(1.0 / many, 1),
-        "single_thread": {"value": round(56.0 / one / 1e9, 3), "unit": "GB/s", "params_per_s": round(1.0 / one, 1)},
-        "sample": f"oracle orc_adam_f32, P={P}, N=2^24 sample of the 2^28 workload; {repsT} steps on {threads} threads "
-                  f"(one index slice each), {reps1} steps on 1 thread ({os.cpu_count()} host cpus visible)",
+        "single_thread": {"value": round(per_unit / one / 1e9, 3), "unit": "GB/s", "params_per_s": round(1.0 / one, 1)},
+        "sample": f"{what}; {repsT} steps on {threads} threads (one slice each), {reps1} steps on 1 thread "
+                  f"({os.cpu_count()} host cpus visible)",
     }
 
 
@@ -307,8 +355,8 @@ def main():
     if flops:
         line["mfma"] = {"achieved": round(flops / (ev_ms * 1e-3) / 1e12, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                         "unit": "TFLOP/s", "frac": round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
-    if wl == "adam_f32" and not a.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline_adam(8)
+    if wl != "copy" and not a.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(wl, P if wl != "mlp_outproj" else 8)
     print(json.dumps(line), flush=True)
 
 
