@@ -71,5 +71,33 @@ def main():
     print("wrote", os.path.join(HERE, "fixtures.npz"), {k: v.shape for k, v in out.items()})
 
 
+def main_16bit():
+    """fixtures_16bit.npz: the bfloat16-gradient Adam step and the modified NCCL's mixed-precision LAMB."""
+    out = {}
+    P, N = 8, 515
+    g16 = [orc.f32_to_bf16(x * np.float32(128.0)) for x in grads_f32(105, P, N, 1e-3)]
+    g16[1][40] = 0x7F80
+    g16[6][511] = 0xFFC0
+    w, m, v = weights_f32(105, N, 0.05), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    w16 = np.zeros(N, np.uint16)
+    out["bf16_g16"], out["bf16_w0"] = np.stack(g16), w.copy()
+    out["bf16_flag"] = np.array([orc.adam_bf16g(g16, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, 1, np.float32(2.0 ** -7))], np.uint32)
+    out["bf16_w1"], out["bf16_m1"], out["bf16_v1"], out["bf16_w16"] = w, m, v, w16
+    P = 4
+    segs = np.array([0, 7, 1031, 2048, 9000], np.uint64)
+    N = int(segs[-1])
+    g16 = [orc.f32_to_f16(x) for x in grads_f32(106, P, N, 0.5)]
+    w = weights_f32(106, N, 0.05)
+    m = weights_f32(107, N, 0.01)
+    v = np.abs(weights_f32(108, N, 1e-2)) + np.float32(1e-3)
+    hw = np.zeros(N, np.uint16)
+    out.update(lamb16_g16=np.stack(g16), lamb16_segs=segs, lamb16_w0=w.copy(), lamb16_m0=m.copy(), lamb16_v0=v.copy())
+    out["lamb16_norms"] = orc.lamb_nccl_f16g(g16, w, hw, m, v, segs, 0.01, 0.9, 0.999, 1.0)
+    out.update(lamb16_w1=w, lamb16_m1=m, lamb16_v1=v, lamb16_hw=hw)
+    np.savez_compressed(os.path.join(HERE, "fixtures_16bit.npz"), **out)
+    print("wrote", os.path.join(HERE, "fixtures_16bit.npz"), {k: v.shape for k, v in out.items()})
+
+
 if __name__ == "__main__":
     main()
+    main_16bit()
