@@ -33,7 +33,7 @@ SYMBOLS = [
     "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
     "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
     "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
-    "ccn_lamb_f32_scattered", "ccn_adam_bf16g", "ccn_lamb_nccl_f16g",
+    "ccn_lamb_f32_scattered", "ccn_adam_bf16g", "ccn_lamb_nccl_f16g", "ccn_lamb_f32_static",
 ]
 
 
@@ -99,6 +99,7 @@ def _declare(L):
     sig("ccn_lamb_plan_destroy", [_vp])
     sig("ccn_lamb_f32", [_vp, _pp, _i, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
     sig("ccn_lamb_plan_norms", [_vp, _vp, _vp])
+    sig("ccn_lamb_f32_static", [_pp, _i, _vp, _vp, _vp, _sz, _sz, _f, _f, _f, _f, _f, _i, _i, _vp, _vp])
     sig("ccn_lamb_f32_scattered", [_vp, _pp, _i, _pp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
     sig("ccn_lamb_nccl_f16g", [_vp, _pp, _i, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _vp])
     sig("ccn_mlp_outproj_bf16", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _vp])
@@ -383,6 +384,17 @@ class LambPlan:
             self.close()
         except Exception:
             pass
+
+
+LAMB_STATIC_MAX_N = 1 << 28
+LAMB_STATIC_MAX_SEGS = 4096
+
+
+def lamb_f32_static(g, w, m, v, n, seg_len, lr, beta1, beta2, eps, wd, step, mode=LAMB_TRUST_RATIO, norms=None, stream=None):
+    """ccn_lamb_f32_static: the two-pass LAMB step on uniform segments, scratch in the library's static device array."""
+    p, _keep = ptr_table(g)
+    _check(load().ccn_lamb_f32_static(p, len(g), addr(w), addr(m), addr(v), n, seg_len, lr, beta1, beta2, eps, wd, step,
+                                      mode, addr(norms), stream), "ccn_lamb_f32_static")
 
 
 def mlp_outproj_bf16(X, W, partials, bias, resid, out, M, N, K, p_drop, seed, stream=None):

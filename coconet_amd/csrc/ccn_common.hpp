@@ -191,6 +191,10 @@ StreamShape stream_shape(int load_bytes, int store_bytes);
 // Dynamic LDS request that keeps at most `per_cu` workgroups on a CU (0 = no request).
 unsigned lds_for_residency(int per_cu);
 
+// Looks up, once per device and with that device current, the device address of the static scratch array behind
+// ccn_lamb_f32_static, so that the entry point itself never has to (it may run under stream capture).
+int lamb_static_setup();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace ccn

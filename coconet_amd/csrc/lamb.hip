@@ -19,6 +19,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <type_traits>
 #include <vector>
@@ -804,6 +805,40 @@ __global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, uint16_t* h
   }
 }
 
+// ---- the two-pass step without a plan, for callers that cannot allocate ------------------------------------------------
+// Everything a plan would hold in allocated device memory (tile sums, group sums, norms, scales and the small index
+// tables of the finalize kernels) lives in one file-scope device array instead.  Every GPU the library runs on holds its
+// own copy of the array at its own address until the process ends; host code never uses the array's name as an address
+// (on the host it is a stand-in, not device memory) but the pointer hipGetSymbolAddress returns for the current device.
+constexpr size_t kStaticMaxTiles = (size_t)1 << 18;                       // N <= 2^28 elements in tiles of kLambTile
+constexpr size_t kStaticMaxSegs = CCN_LAMB_STATIC_MAX_SEGS;
+constexpr size_t kStaticMaxGroups = kStaticMaxTiles / kLambFold + 64;      // groups only exist when segments are long
+static_assert(kStaticMaxTiles * kLambTile == CCN_LAMB_STATIC_MAX_N, "header and kernel limits agree");
+
+struct LambStaticScratch {
+  double partials[2 * kStaticMaxTiles];
+  double folded[2 * kStaticMaxGroups];
+  double norms[2 * kStaticMaxSegs];
+  uint64_t seg_len[kStaticMaxSegs];
+  float scale[kStaticMaxSegs];
+  uint32_t seg_begin[kStaticMaxSegs + 1];      // first tile (or first group, when sums go through groups) of a segment
+  uint32_t group_begin[kStaticMaxGroups + 1];  // first tile of a group
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(LambStaticScratch)];
+
+// Fills the index tables for nseg segments of tps tiles each.  gps = 0: the finalize kernel reads tile sums, seg_begin
+// counts tiles.  gps > 0: segment sums go through gps groups of at most kLambFold tiles, seg_begin counts groups.
+__global__ void lamb_static_tables_kernel(LambStaticScratch* sc, const uint32_t nseg, const uint32_t tps, const uint32_t gps,
+                                          const uint64_t seg_len) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < nseg) sc->seg_len[i] = seg_len;
+  if (i <= nseg) sc->seg_begin[i] = gps ? i * gps : i * tps;
+  if (gps && i <= nseg * gps) {
+    const uint32_t b = i / gps, q = i % gps;
+    sc->group_begin[i] = i == nseg * gps ? nseg * tps : b * tps + q * kLambFold;
+  }
+}
+
 }  // namespace ccn
 
 using namespace ccn;
@@ -1411,6 +1446,35 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
 
 }  // namespace
 
+namespace ccn {
+
+// Device address of `scratch` on each device, asked for once per device with that device current.
+namespace {
+constexpr int kStaticMaxDevices = 16;
+LambStaticScratch* g_static_ptr[kStaticMaxDevices];
+int g_static_rc[kStaticMaxDevices];
+std::once_flag g_static_once[kStaticMaxDevices];
+}  // namespace
+
+int lamb_static_setup(LambStaticScratch** out) {
+  int dev = -1;
+  CCN_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kStaticMaxDevices) return CCN_ENODEV;
+  std::call_once(g_static_once[dev], [dev] {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    g_static_rc[dev] = e == hipSuccess ? (ptr ? CCN_OK : CCN_EHIP) : hip_fail(e);
+    g_static_ptr[dev] = static_cast<LambStaticScratch*>(ptr);
+  });
+  if (g_static_rc[dev] != CCN_OK) return g_static_rc[dev];
+  if (out) *out = g_static_ptr[dev];
+  return CCN_OK;
+}
+
+int lamb_static_setup() { return lamb_static_setup(nullptr); }
+
+}  // namespace ccn
+
 extern "C" {
 
 int ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, float* m, float* v, float lr, float beta1,
@@ -1428,6 +1492,77 @@ int ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, fl
 int ccn_lamb_nccl_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
                        float lr, float beta1, float beta2, float wd, void* stream) {
   return guarded([&] { return lamb_step_f16g(plan, g, P, w, halfw, m, v, lr, beta1, beta2, wd, stream); });
+}
+
+int ccn_lamb_f32_static(const float* const* g, int P, float* w, float* m, float* v, size_t N, size_t seg_len, float lr,
+                        float beta1, float beta2, float eps, float wd, int step, int mode, double* norms, void* stream) {
+  if (!g || !w || !m || !v || P < 1 || P > CCN_MAX_RANKS || step < 1 || N == 0 || seg_len == 0) return CCN_EINVAL;
+  if (mode != CCN_LAMB_TRUST_RATIO && mode != CCN_LAMB_REFERENCE && mode != CCN_LAMB_NCCL_GLOBAL) return CCN_EINVAL;
+  for (int p = 0; p < P; p++) if (!g[p]) return CCN_EINVAL;
+  if (seg_len % kLambTile || N % seg_len) return CCN_EINVAL;   // whole tiles per segment, whole segments
+  if (N > CCN_LAMB_STATIC_MAX_N || N / seg_len > CCN_LAMB_STATIC_MAX_SEGS) return CCN_ERANGE;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  LambStaticScratch* sc = nullptr;
+  rc = lamb_static_setup(&sc);
+  if (rc != CCN_OK) return rc;
+
+  LambPrm k;
+  k.b1 = beta1;
+  k.omb1 = 1 - beta1;
+  k.b2 = beta2;
+  k.omb2 = 1 - beta2;
+  k.eps = eps;
+  k.wd = wd;
+  k.lr = lr;
+  k.mode = mode;
+  k.bc1 = 1 - std::pow((double)beta1, (double)step);
+  k.bc2 = 1 - std::pow((double)beta2, (double)step);
+
+  const uint32_t nseg = (uint32_t)(N / seg_len), tps = (uint32_t)(seg_len / kLambTile), ntiles = nseg * tps;
+  const uint32_t gps = tps > kLambFold ? (tps + kLambFold - 1) / kLambFold : 0;   // the plan's rule for going through groups
+  bool al = aligned16(w) && aligned16(m) && aligned16(v);
+  for (int p = 0; p < P; p++) al = al && aligned16(g[p]);
+  const int vec_ok = al ? 1 : 0;
+  LambLayout lay;
+  lay.tiles = nullptr;
+  lay.seg_len = seg_len;
+  lay.seg_len_f = (float)seg_len;
+  lay.tile = kLambTile;
+  lay.gtab = nullptr;
+  lay.wtab = nullptr;
+  lay.nseg = nseg;
+  hipStream_t s = as_stream(stream);
+  const dim3 block(kBlock), grid(ntiles);
+  double* const norms_dst = norms ? norms : sc->norms;
+
+  const uint32_t entries = (gps ? nseg * gps : nseg) + 1;
+  hipLaunchKernelGGL(lamb_static_tables_kernel, dim3((entries + kBlock - 1) / kBlock), block, 0, s, sc, nseg, tps, gps,
+                     (uint64_t)seg_len);
+  CCN_HIP(hipGetLastError());
+  with_rank_count(P, [&](auto ptag) {
+    constexpr int PP = decltype(ptag)::value;
+    SrcTable<float, (PP ? PP : CCN_MAX_RANKS)> tbl;
+    for (int p = 0; p < (PP ? PP : CCN_MAX_RANKS); p++) tbl.p[p] = g[p < P ? p : 0];
+    hipLaunchKernelGGL((lamb_pass1_kernel<PP, false>), grid, block, lds_for_residency(P >= 2 ? 4 : 0), s, tbl, P, (const float*)w, m,
+                       v, lay, sc->partials, vec_ok, k);
+  });
+  CCN_HIP(hipGetLastError());
+  const double* sums = sc->partials;
+  if (gps) {
+    hipLaunchKernelGGL(lamb_fold_kernel, dim3(nseg * gps), block, 0, s, (const double*)sc->partials,
+                       (const uint32_t*)sc->group_begin, sc->folded);
+    CCN_HIP(hipGetLastError());
+    sums = sc->folded;
+  }
+  hipLaunchKernelGGL(lamb_finalize_kernel, dim3(nseg), block, 0, s, sums, (const uint32_t*)sc->seg_begin,
+                     (const uint64_t*)sc->seg_len, norms_dst, sc->scale, mode);
+  CCN_HIP(hipGetLastError());
+  hipLaunchKernelGGL((lamb_pass2_kernel<false>), grid, block, 0, s, w, (const float*)m, (const float*)v, lay,
+                     (const float*)sc->scale, vec_ok, k);
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
 }
 
 int ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream) {

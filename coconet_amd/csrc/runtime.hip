@@ -106,7 +106,9 @@ int ccn_init(int device) {
   if (device < 0 || device >= count) return CCN_ENODEV;
   CCN_HIP(hipSetDevice(device));
   const DeviceInfo* di = nullptr;
-  return current_device_info(&di);
+  const int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  return lamb_static_setup();
 }
 
 int ccn_device_info(int* cu_count, size_t* hbm_bytes, char* arch, size_t arch_len) {

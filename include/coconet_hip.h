@@ -183,6 +183,21 @@ int  ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, f
  * segments (a second tile table is then made on the first call, which therefore allocates and cannot be recorded). */
 int  ccn_lamb_nccl_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
                         float lr, float beta1, float beta2, float wd, void* stream);
+/* The two-pass step of ccn_lamb_f32 for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  It takes no plan: the tile sums, norms,
+ * scales and index tables a plan would own live in a static device array inside the library (about 4.2 MiB, held by every
+ * GPU the library runs on until the process ends), and the call makes no hipMalloc, hipFree or other allocating call.
+ * Segments are uniform: N / seg_len segments of seg_len elements each; seg_len must be a multiple of 1024 and divide N
+ * (CCN_EINVAL otherwise).  Limits: N <= CCN_LAMB_STATIC_MAX_N and N / seg_len <= CCN_LAMB_STATIC_MAX_SEGS, beyond which
+ * the call returns CCN_ERANGE and does nothing.  norms: DEVICE array of 2 * (N / seg_len) doubles receiving W_b, R_b, or
+ * NULL.  Same arithmetic, kernels and results as ccn_lamb_f32 on a plan whose segments take the two-pass path.
+ * All calls on one GPU share the one array: calls that overlap in time on the same GPU (two streams, two threads)
+ * race; order them.  ccn_init looks the array's address up; without ccn_init the first call on a device does. */
+#define CCN_LAMB_STATIC_MAX_N    ((size_t)1 << 28)
+#define CCN_LAMB_STATIC_MAX_SEGS 4096
+int  ccn_lamb_f32_static(const float* const* g, int P, float* w, float* m, float* v, size_t N, size_t seg_len,
+                         float lr, float beta1, float beta2, float eps, float wd, int step, int mode,
+                         double* norms, void* stream);
 /* copies W_b, R_b of the last LAMB step on this plan to a HOST array of 2*nseg doubles (synchronises) */
 int  ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream);
 
