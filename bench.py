@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", action="store_true",
+                    help="default run only: leave out the short runs of the other benchmark configurations")
     ap.add_argument("--graph-steps", type=int, default=0,
                     help="record this many steps once (ccn_graph_*) and time replays of the recording: for launch-bound "
                          "sizes such as config 1; a recorded step keeps its step number")
@@ -177,33 +179,21 @@ def cpu_baseline(wl, P, budget_s=8.0):
     }
 
 
-def main():
-    a = parse()
-    if a.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the reduce over P rank buffers is local); "
-              "run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-    import torch
-    from coconet_amd import capi
-    capi.load()
-    capi.init(0)
-    torch.cuda.set_device(0)
-    info = capi.device_info()
-    K, W = a.steps, a.warmup
-    wl = a.workload
-    own_stream = capi.Stream() if a.graph_steps > 0 else None      # the null stream cannot be recorded
-    stream = own_stream.h if own_stream else torch.cuda.current_stream().cuda_stream
+def build_workload(a, wl, capi, torch, stream, allocator):
+    """Allocates the synthetic inputs of one workload in HBM.  Returns (step, alg_bytes, units, kernel, config, flops, P, keep)
+    where step(t) enqueues one pass of the hot path on `stream` and `keep` holds what must stay alive."""
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
-
     flops = None
+    P = 8
+    keep = []
     if wl == "adam_f32_scattered":
         # the same step with gradients and weights in 256 separate buffers (one per "parameter tensor")
         P = a.ranks or 8
         N = 1 << (a.log2n or 28)
         nbuff = 256
         per = N // nbuff
-        bufs = Buffers(capi, torch, a.allocator == "torch")
+        bufs = Buffers(capi, torch, allocator == "torch")
         mk = lambda scale: bufs.from_tensor(torch.empty(per, device="cuda").normal_(0.0, scale, generator=gen))
         g = [[mk(1e-3) for _ in range(nbuff)] for _ in range(P)]
         w = [mk(0.05) for _ in range(nbuff)]
@@ -216,14 +206,18 @@ def main():
         alg_bytes = float(per_param) * N
         units = N
         config = {"workload": f"adam_f32 over {nbuff} scattered buffers, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,
-                  "algorithmic_bytes_per_param": per_param, "allocator": a.allocator}
-    elif wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g", "adam_bf16g", "lamb_nccl_f16g"):
+                  "algorithmic_bytes_per_param": per_param, "allocator": allocator}
+        keep = [bufs, plan]
+    elif wl in ("adam_f32", "sgd_f32", "lamb_f32", "adam_f16g", "adam_bf16g", "lamb_nccl_f16g", "sgd_f32_large"):
+        large_sgd = wl == "sgd_f32_large"       # configuration 1's shape at a size that leaves the caches
+        if large_sgd:
+            wl = "sgd_f32"
         P = a.ranks or (4 if wl == "sgd_f32" else 8)
-        N = 1 << (a.log2n or (20 if wl == "sgd_f32" else 28))
+        N = 1 << (a.log2n or (28 if large_sgd else 20 if wl == "sgd_f32" else 28))
         gbytes = 2 if wl in ("adam_f16g", "adam_bf16g", "lamb_nccl_f16g") else 4
         half = torch.bfloat16 if wl == "adam_bf16g" else torch.float16
         gscale = 2.0 ** 7 if wl == "adam_bf16g" else 2.0 ** 16
-        bufs = Buffers(capi, torch, a.allocator == "torch")
+        bufs = Buffers(capi, torch, allocator == "torch")
         g = []
         for p in range(P):
             if gbytes == 2:
@@ -237,6 +231,7 @@ def main():
         w = bufs.from_tensor(torch.empty(N, device="cuda").uniform_(-0.05, 0.05, generator=gen))
         m = bufs.from_tensor(torch.zeros(N, device="cuda"))
         v = bufs.from_tensor(torch.zeros(N, device="cuda"))
+        keep = [bufs]
         if wl == "adam_f32":
             per_param = (P + 3) * 4 + 3 * 4
             step = lambda t: capi.adam_f32(g, w, m, v, N, 1e-3, 0.9, 0.999, 1e-6, t, stream)
@@ -250,12 +245,14 @@ def main():
             w16 = bufs.from_tensor(torch.empty(N, dtype=torch.float16, device="cuda"))
             nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
             plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
+            keep.append(plan)
             per_param = P * 2 + 12 + 12 + 2
             step = lambda t: plan.step_nccl_f16g(g, w, w16, m, v, 1e-3, 0.9, 0.999, 1.0, stream)
             kernel = "lamb_reset_kernel + lamb_oneshot_kernel<%d, 256, 8, false, uint16_t> + lamb_deferred_kernel<256, 8, false, true>" % (P if P <= 8 else 0)
         elif gbytes == 2:
             w16 = bufs.from_tensor(torch.empty(N, dtype=half, device="cuda"))
             flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+            keep.append(flag)
             per_param = P * 2 + 12 + 12 + 2
             call = capi.adam_bf16g if wl == "adam_bf16g" else capi.adam_f16g
             step = lambda t: call(g, w, m, v, w16, N, 1e-3, 0.9, 0.999, 1e-6, t, 1.0 / gscale, flag, stream)
@@ -264,13 +261,14 @@ def main():
         else:
             nseg = 256 if N >= (1 << 20) * 256 else max(1, N >> 20)
             plan = capi.LambPlan([i * (N // nseg) for i in range(nseg + 1)])
+            keep.append(plan)
             per_param = (P + 3) * 4 + 3 * 4
             step = lambda t: plan.step(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, capi.LAMB_TRUST_RATIO, stream)
             kernel = "lamb_reset_kernel + lamb_oneshot_kernel<%d, 256, 8> + lamb_deferred_kernel<256, 8>" % (P if P <= 8 else 0)
         alg_bytes = float(per_param) * N
         units = N
         config = {"workload": f"{wl} fused reduce+update, N=2^{int(np.log2(N))}, P={P}", "N": N, "P": P,
-                  "algorithmic_bytes_per_param": per_param, "allocator": a.allocator}
+                  "algorithmic_bytes_per_param": per_param, "allocator": allocator}
     elif wl == "mlp_outproj":
         M = Nn = 8192
         Kd = 1024
@@ -296,6 +294,101 @@ def main():
         units = N
         kernel = "torch copy"
         config = {"workload": f"device copy of 2^{int(np.log2(N))} fp32"}
+    return step, alg_bytes, units, kernel, config, flops, P, keep
+
+
+def release(keep, capi, torch):
+    """Gives a workload's device memory back before the next one is allocated."""
+    for k in keep:
+        if isinstance(k, Buffers):
+            for x in k.keep:
+                if isinstance(x, int):
+                    capi.free(x)
+            k.keep = []
+        elif hasattr(k, "close"):
+            k.close()
+    keep.clear()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+
+
+def timed_steps(step, K, W, capi, torch, stream):
+    """W untimed steps, then K steps bracketed by a device synchronisation on both sides.  Returns the wall-clock and the
+    HIP-event time per step (events recorded on the launch stream)."""
+    for t in range(1, W + 1):
+        step(t)
+    torch.cuda.synchronize()
+    e0, e1 = capi.Event(), capi.Event()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for t in range(W + 1, W + K + 1):
+        step(t)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / K, e0.elapsed_ms(e1) / K
+
+
+def other_workloads(a, capi, torch, stream):
+    """Short runs of the other benchmark configurations, and of the headline kernel on plain (unstaggered) allocations,
+    so that every configuration's figure comes from the same command as the headline.  Few steps each: these are HBM-bound
+    kernels of a few milliseconds whose launch times spread by about a percent."""
+    rows = []
+    # The headline kernel on plain allocations, in a process of its own: same-sized blocks straight from a fresh
+    # allocator are the case a caller that does not use ccn_malloc starts from (what an allocator hands out after other
+    # buffers have come and gone in the same process is placed differently and measures differently).
+    import subprocess
+    child = subprocess.run([sys.executable, os.path.abspath(__file__), "--allocator", "torch", "--steps", "30", "--warmup", "10",
+                            "--no-cpu-baseline", "--no-others"], capture_output=True, text=True, timeout=300)
+    try:
+        c = json.loads(child.stdout.strip().splitlines()[-1])
+        rows.append({"workload": c["config"]["workload"], "allocator": "torch (fresh process)", "steps": c["steps"],
+                     "warmup": c["warmup"], "ms_per_step": c["ms_per_step"], "avg_launch_ms": c["roofline"]["avg_launch_ms"],
+                     "algorithmic_GBps": c["roofline"]["achieved"], "frac_of_hbm_peak": c["roofline"]["frac"],
+                     "kernel": c["roofline"]["kernel"],
+                     "algorithmic_bytes_per_launch": c["roofline"]["algorithmic_bytes_per_launch"], "traffic": None})
+    except (ValueError, KeyError, IndexError):
+        rows.append({"workload": "adam_f32 on plain allocations", "error": (child.stderr or child.stdout)[-300:]})
+    for wl, allocator in (("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_large", "ccn"), ("adam_f16g", "ccn"),
+                          ("lamb_f32", "ccn"), ("mlp_outproj", "ccn")):
+        step, alg_bytes, units, kernel, config, flops, P, keep = build_workload(a, wl, capi, torch, stream, allocator)
+        steps, warm = (200, 20) if alg_bytes < 1e9 else (30, 10)
+        wall_ms, ev_ms = timed_steps(step, steps, warm, capi, torch, stream)
+        ach = alg_bytes / (ev_ms * 1e-3) / 1e9
+        row = {"workload": config["workload"], "allocator": allocator, "steps": steps, "warmup": warm,
+               "ms_per_step": round(wall_ms, 5), "avg_launch_ms": round(ev_ms, 5), "algorithmic_GBps": round(ach, 2),
+               "frac_of_hbm_peak": round(ach / HBM_PEAK_GBPS, 4), "kernel": kernel,
+               "algorithmic_bytes_per_launch": alg_bytes,
+               "traffic": traffic_from_profiles(f"{'sgd_f32' if wl == 'sgd_f32_large' else wl}.pmc.txt") if allocator == "ccn" else None}
+        if alg_bytes < 1e9:
+            row["note"] = "fits the caches and is bound by launches: not a roofline figure"
+        if flops:
+            row["mfma_TFLOPs"] = round(flops / (ev_ms * 1e-3) / 1e12, 2)
+            row["frac_of_mfma_peak"] = round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+        rows.append(row)
+        del step
+        release(keep, capi, torch)
+    return rows
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the reduce over P rank buffers is local); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from coconet_amd import capi
+    capi.load()
+    capi.init(0)
+    torch.cuda.set_device(0)
+    info = capi.device_info()
+    K, W = a.steps, a.warmup
+    wl = a.workload
+    own_stream = capi.Stream() if a.graph_steps > 0 else None      # the null stream cannot be recorded
+    stream = own_stream.h if own_stream else torch.cuda.current_stream().cuda_stream
+
+    step, alg_bytes, units, kernel, config, flops, P, keep = build_workload(a, wl, capi, torch, stream, a.allocator)
 
     if a.graph_steps > 0:
         if wl in ("copy",):
@@ -308,21 +401,10 @@ def main():
         eager_step, K = step, max(1, K // a.graph_steps)
         step = lambda t: graph.launch()
         config["graph_steps"] = a.graph_steps
-    for t in range(1, W + 1):
-        step(t)
-    torch.cuda.synchronize()
-    e0, e1 = capi.Event(), capi.Event()
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for t in range(W + 1, W + K + 1):
-        step(t)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    wall_ms, ev_ms = timed_steps(step, K, W, capi, torch, stream)
     if a.graph_steps > 0:
+        wall_ms, ev_ms = wall_ms / a.graph_steps, ev_ms / a.graph_steps
         K *= a.graph_steps                       # steps actually run
-    wall_ms = (t1 - t0) * 1e3 / K
-    ev_ms = e0.elapsed_ms(e1) / K
 
     # the spread of single launches, each bracketed by its own pair of events (outside the timed region)
     n_single = 0 if a.graph_steps > 0 else min(K, 50)
@@ -355,6 +437,11 @@ def main():
     if flops:
         line["mfma"] = {"achieved": round(flops / (ev_ms * 1e-3) / 1e12, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                         "unit": "TFLOP/s", "frac": round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    default_run = (wl == "adam_f32" and a.allocator == "ccn" and a.graph_steps == 0 and a.log2n is None and a.ranks is None)
+    if default_run and not a.no_others:
+        del step
+        release(keep, capi, torch)
+        line["other_workloads"] = other_workloads(a, capi, torch, stream)
     if wl != "copy" and not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl, P if wl != "mlp_outproj" else 8)
     print(json.dumps(line), flush=True)
