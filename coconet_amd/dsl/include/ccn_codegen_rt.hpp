@@ -171,6 +171,8 @@ template <class Body> struct KernelArgs {
   double* partials;      // NACC values per workgroup
   const float* norms;    // NNORM values
   size_t n;
+  size_t idx_base;       // index of element 0 in the whole tensor (a launch over one rank's slice starts at its offset):
+                         // what index-dependent expressions (the dropout mask) see is idx_base + the element's position
   typename Body::Scalars s;
 };
 
@@ -222,7 +224,7 @@ __global__ __launch_bounds__(BS) void fused_pointwise_kernel(const KernelArgs<Bo
       float in1[NINX], out1[NOUTX];
 #pragma unroll
       for (int k = 0; k < Body::NIN; k++) in1[k] = iv[k].d[e];
-      Body::apply(Body::HAS_RED ? red.d[e] : 0.0f, in1, out1, a.s, acc, nrm, (uint64_t)(e0 + e));
+      Body::apply(Body::HAS_RED ? red.d[e] : 0.0f, in1, out1, a.s, acc, nrm, (uint64_t)(a.idx_base + e0 + e));
 #pragma unroll
       for (int k = 0; k < Body::NOUT; k++) ov[k].d[e] = out1[k];
     }
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(BS) void fused_pointwise_kernel(const KernelArgs<Bo
       }
       float in1[NINX], out1[NOUTX];
       for (int k = 0; k < Body::NIN; k++) in1[k] = a.in[k][i];
-      Body::apply(red, in1, out1, a.s, acc, nrm, (uint64_t)i);
+      Body::apply(red, in1, out1, a.s, acc, nrm, (uint64_t)(a.idx_base + i));
       for (int k = 0; k < Body::NOUT; k++) {
         if ((Body::OUT_F16 >> k) & 1u) static_cast<uint16_t*>(a.out[k])[i] = f32_to_f16_bits(out1[k]);
         else static_cast<float*>(a.out[k])[i] = out1[k];
@@ -352,7 +354,8 @@ template <class Body, int VEC> unsigned launch_vec(const KernelArgs<Body>& a, hi
 
 // An upper bound on the workgroups launch() uses for n elements, whatever the shape (the partials array holds NACC
 // values per workgroup): scalar launches have 256 threads, vector launches at least 64 threads of 4 elements.
-inline unsigned blocks_for(size_t n) { return grid_for(n, 1, kBlock); }
+// (launched slice by slice, every rank's launch rounds up on its own: kMaxRanks more)
+inline unsigned blocks_for(size_t n) { return grid_for(n, 1, kBlock) + (unsigned)kMaxRanks; }
 
 // Launches the kernel and returns the number of workgroups used: that many rows of NACC partial sums are written.
 template <class Body> unsigned launch(const KernelArgs<Body>& a, void* stream) {
@@ -435,10 +438,9 @@ inline bool eqFloat(float ref, float got, float tol = 1e-5f) {
   return std::fabs(ref - got) / den <= tol;
 }
 
-inline bool compare(const char* what, const std::vector<float>& ref, const float* dev, size_t n, float tol = 1e-5f) {
-  std::vector<float> got(n);
-  CCNCHECK(ccn_memcpy_d2h(got.data(), dev, n * sizeof(float), nullptr));
-  for (size_t i = 0; i < n; i++) {
+// Host half of the comparison: reports the first element that differs by more than tol (relative).
+inline bool compare_host(const char* what, const std::vector<float>& ref, const std::vector<float>& got, float tol) {
+  for (size_t i = 0; i < ref.size(); i++) {
     if (!eqFloat(ref[i], got[i], tol)) {
       printf("Mismatch in %s at %zu : ref '%.9g', computed '%.9g'\n", what, i, ref[i], got[i]);
       return false;
@@ -447,18 +449,66 @@ inline bool compare(const char* what, const std::vector<float>& ref, const float
   return true;
 }
 
+inline bool compare(const char* what, const std::vector<float>& ref, const float* dev, size_t n, float tol = 1e-5f) {
+  std::vector<float> got(n);
+  CCNCHECK(ccn_memcpy_d2h(got.data(), dev, n * sizeof(float), nullptr));
+  return compare_host(what, ref, got, tol);
+}
+
 // fp16 outputs: widened and compared like fp32 ones
 inline bool compare(const char* what, const std::vector<float>& ref, const uint16_t* dev, size_t n, float tol = 1e-5f) {
   std::vector<uint16_t> got(n);
   CCNCHECK(ccn_memcpy_d2h(got.data(), dev, n * sizeof(uint16_t), nullptr));
-  for (size_t i = 0; i < n; i++) {
-    const float x = f16_bits_to_f32(got[i]);
-    if (!eqFloat(ref[i], x, tol)) {
-      printf("Mismatch in %s at %zu : ref '%.9g', computed '%.9g'\n", what, i, ref[i], x);
-      return false;
-    }
+  std::vector<float> wide(n);
+  for (size_t i = 0; i < n; i++) wide[i] = f16_bits_to_f32(got[i]);
+  return compare_host(what, ref, wide, tol);
+}
+
+// ---- options of the emitted main(), all from the environment ---------------------------------------------------------
+inline size_t env_size(const char* name, size_t dflt) {
+  const char* e = getenv(name);
+  if (!e || !*e) return dflt;
+  char* end = nullptr;
+  const unsigned long long x = strtoull(e, &end, 10);
+  return end && *end == 0 ? (size_t)x : dflt;
+}
+inline float env_float(const char* name, float dflt) {
+  const char* e = getenv(name);
+  if (!e || !*e) return dflt;
+  char* end = nullptr;
+  const float x = strtof(e, &end);
+  return end && *end == 0 ? x : dflt;
+}
+// Writes n elements of a device array to <prefix>.<name>.<n>.f32 (fp16 arrays widened), raw little-endian floats.
+inline void dump_host(const char* prefix, const char* name, const std::vector<float>& h) {
+  char path[1024];
+  snprintf(path, sizeof(path), "%s.%s.%zu.f32", prefix, name, h.size());
+  FILE* f = fopen(path, "wb");
+  if (!f || fwrite(h.data(), sizeof(float), h.size(), f) != h.size()) {
+    printf("Error writing %s\n", path);
+    exit(EXIT_FAILURE);
   }
-  return true;
+  fclose(f);
+}
+inline void dump(const char* prefix, const char* name, const float* dev, size_t n) {
+  std::vector<float> h(n);
+  CCNCHECK(ccn_memcpy_d2h(h.data(), dev, n * sizeof(float), nullptr));
+  dump_host(prefix, name, h);
+}
+inline void dump(const char* prefix, const char* name, const uint16_t* dev, size_t n) {
+  std::vector<uint16_t> h(n);
+  CCNCHECK(ccn_memcpy_d2h(h.data(), dev, n * sizeof(uint16_t), nullptr));
+  std::vector<float> wide(n);
+  for (size_t i = 0; i < n; i++) wide[i] = f16_bits_to_f32(h[i]);
+  dump_host(prefix, name, wide);
+}
+// Corrupts element i of a device array (adds one part in a thousand, or 1 to a zero): what the comparison must catch.
+inline void perturb(float* dev, size_t i) {
+  float x;
+  CCNCHECK(ccn_memcpy_d2h(&x, dev + i, sizeof(float), nullptr));
+  x = x != 0.0f ? x * 1.001f : 1.0f;
+  CCNCHECK(ccn_memcpy_h2d(dev + i, &x, sizeof(float), nullptr));
+  CCNCHECK(ccn_stream_sync(nullptr));
 }
 
 // ---- bf16 on the host (round-to-nearest-even), for programs that feed the MFMA GEMM ---------------------------------

@@ -181,7 +181,12 @@ def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path)
     fused = (tmp_path / "adam-fuse-rs-c-ag.hip").read_text()
     assert "HAS_RED = true" in fused and "ccn_memcpy_d2d" not in fused       # RS + compute + AG in one kernel
     unf = (tmp_path / "adam-rs-c-ag.hip").read_text()
-    assert "ccn_reduce_f32" in unf and "ccn_memcpy_d2d(w, S5" in unf         # ReduceScatter, kernel, AllGather
+    # ReduceScatter, kernel, AllGather, each on the rank's slice: every array moved on by DIVUP(N, comm_size) * rank
+    assert "ccn_reduce_f32(tbl__, comm_size, g[0] + off__, cnt__" in unf and "ccn_memcpy_d2d(w + off__, S5 + off__, cnt__" in unf
+    assert "per__ = DIVUP((size_t)((size_t)N), (size_t)comm_size), off__ = per__ * (size_t)r_" in unf
+    assert "args0.in[0] = m + off__" in unf and "args0.n = cnt__" in unf and "int comm_size, int rank" in unf
+    arc = (tmp_path / "adam-ar-c.hip").read_text()
+    assert "off__" not in arc and "ccn_reduce_f32(g, comm_size, g[0], (size_t)N" in arc     # Replicated: the whole range
     mlp = (tmp_path / "model-parallel-mm-ar-c.hip").read_text()
     assert "ccn_mlp_outproj_bf16" in mlp and "p_drop = (float)0.5;" in mlp
 
@@ -215,3 +220,37 @@ def test_emitted_programs_were_cross_compiled(dsl_build):
         subprocess.check_call(["make", "-C", DSL, "-s", "-j8", "gen"])
     for name in ("sgd-fused", "adam-fused", "adam-unfused", "lamb-fused"):
         assert os.access(os.path.join(gen, name), os.X_OK), name
+
+
+def test_the_emitted_programs_comparison_catches_a_wrong_value(tmp_path):
+    """The host half of the emitted self-check (ccn_gen::compare_host, the reference's eqFloat loop of
+    src/codegen.cpp:4421-4581 and examples/header.h:55-62): equal vectors pass, a value off by a part in a thousand is
+    reported as a mismatch, at the 1e-6 bar a value off by 3e-6 is too, and one off by 1e-7 is not.  Host code only."""
+    src = tmp_path / "cmp.cpp"
+    src.write_text(r'''
+#include "ccn_codegen_rt.hpp"
+int main() {
+  std::vector<float> ref(1000), got(1000);
+  for (size_t i = 0; i < ref.size(); i++) ref[i] = got[i] = 0.25f + (float)i;
+  if (!ccn_gen::compare_host("same", ref, got, 1e-6f)) return 10;
+  got[500] = ref[500] * 1.001f;
+  if (ccn_gen::compare_host("w", ref, got, 1e-6f)) return 11;
+  got[500] = ref[500] * (1.0f + 3e-6f);
+  if (ccn_gen::compare_host("w", ref, got, 1e-6f)) return 12;
+  if (!ccn_gen::compare_host("w", ref, got, 1e-5f)) return 13;
+  got[500] = ref[500] * (1.0f + 1.2e-7f);
+  if (!ccn_gen::compare_host("w", ref, got, 1e-6f)) return 14;
+  got[500] = ref[500];
+  got[7] = std::nanf("");
+  if (ccn_gen::compare_host("w", ref, got, 1e-6f)) return 15;
+  return 0;
+}
+''')
+    exe = tmp_path / "cmp"
+    lib = os.path.join(ROOT, "coconet_amd", "lib")
+    subprocess.check_call(["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-O1", "-std=c++17", "-I", os.path.join(ROOT, "include"),
+                           "-I", os.path.join(DSL, "include"), str(src), "-L", lib, "-lcoconet_hip", "-Wl,-rpath," + lib,
+                           "-o", str(exe)], stderr=subprocess.DEVNULL)
+    r = run(str(exe))
+    assert r.returncode == 0, (r.returncode, r.stdout)
+    assert r.stdout.count("Mismatch in w at 500") == 2 and "Mismatch in w at 7" in r.stdout

@@ -5,6 +5,7 @@ import os
 import re
 import subprocess
 
+import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
@@ -26,11 +27,17 @@ def as_the_reference_scraper_reads(line):
     return {k.strip(): v for k, v in ast.literal_eval(quoted).items()}
 
 
-def run_program(name, *args):
+def run_raw(name, *args, env=None):
     exe = os.path.join(GEN, name)
     if not os.path.exists(exe):
         pytest.skip(f"{name} was not built (make -C coconet_amd/dsl gen)")
-    r = subprocess.run([exe, *map(str, args)], capture_output=True, text=True, timeout=240)
+    full = dict(os.environ)
+    full.update({k: str(v) for k, v in (env or {}).items()})
+    return subprocess.run([exe, *map(str, args)], capture_output=True, text=True, timeout=240, env=full)
+
+
+def run_program(name, *args, env=None):
+    r = run_raw(name, *args, env=env)
     assert "do not match" not in r.stdout and "Mismatch" not in r.stdout, r.stdout[-2000:]
     assert r.returncode == 0, (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
     rows = []
@@ -70,12 +77,87 @@ def test_programs_emitted_from_the_reference_examples(name):
         assert steps == {"AllReduce", "kernel0"}
 
 
-def test_unaligned_size_takes_scalar_tail():
-    # 2^k sizes never leave a tail; an odd size comes from the explicit bounds path of another program, so run the
-    # smallest sweep point with 3 ranks instead: the kernel's n % 4 tail code is covered by N = 2^10 only when
-    # buffers are unaligned -- here we simply make sure tiny sizes work
-    rows = run_program("adam-fused", 1, 3, 1, 9, 1)
-    assert [r[0] for r in rows] == [1 << k for k in range(1, 10)]
+@pytest.mark.parametrize("name", ["adam-fused", "adam-unfused", "lamb-fused", "adamf16-fused", "ref-adam-rs-c-ag"])
+@pytest.mark.parametrize("n,misalign", [(4099, 0), (4099, 1), (1 << 12, 1), (3, 0), (1, 1)])
+def test_odd_sizes_and_unaligned_arrays(name, n, misalign):
+    """A size that leaves an n % 4 tail behind the 16-byte packs, and arrays that start 4 bytes (2 for fp16) past a
+    16-byte boundary, which take the element-wise instantiation: each program still agrees with its CPU re-execution."""
+    rows = run_program(name, 2, 3, 10, 10, 1, env={"CCN_GEN_N": n, "CCN_GEN_MISALIGN": misalign})
+    assert [r[0] for r in rows] == [n]
+
+
+def splitmix_uniform(seed, n):
+    """The emitted programs' input stream (ccn_gen::uniform01): splitmix64 of seed + golden * (i + 1), top 24 bits."""
+    with np.errstate(over="ignore"):
+        z = np.uint64(seed) + np.uint64(0x9E3779B97F4A7C15) * (np.arange(n, dtype=np.uint64) + np.uint64(1))
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> np.uint64(31))
+    return (((z >> np.uint64(40)) + np.uint64(1)).astype(np.float32) * np.float32(2.0 ** -24)).astype(np.float32)
+
+
+def emitted_inputs(ranks, n, replicated):
+    """Inputs as the emitted main() seeds them: the reduced tensor comes first in the examples' argument lists (seed
+    1234 + 100 + rank), the other tensors follow with seeds 1234 + 101, 1234 + 102, ..."""
+    g = [splitmix_uniform(1234 + 100 + p, n) for p in range(ranks)]
+    return g, [splitmix_uniform(1234 + 101 + k, n) for k in range(replicated)]
+
+
+@pytest.mark.parametrize("schedule", ["ar-c", "rs-c-ag", "fuse-rs-c-ag"])
+@pytest.mark.parametrize("n,ranks", [(1 << 16, 4), (4099, 4), (4099, 7), (10, 4), (5, 8)])
+def test_emitted_sgd_and_adam_against_the_oracle(tmp_path, schedule, n, ranks):
+    """The programs emitted from the reference's examples/sgd and examples/adam, every schedule, against the oracle's
+    restatement of the reference checkers on the same inputs, bit for bit.  The rs-c-ag schedules run rank by rank, each
+    call updating its slice [DIVUP(n, ranks) * rank, ...) only: the union must be the whole update, also when n is not a
+    multiple of the rank count or smaller than it.  lr = 1 and beta = 1/2 are the reference checker's own settings
+    (examples/test-adam.cu:84-88); with them the example's w - m_/v_ and (1 - beta2)*g*g equal the checker's
+    w - (lr*S3)/S4 and (1 - beta2)*(g*g) exactly."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    env = {"CCN_GEN_N": n, "CCN_GEN_DUMP": prefix, "CCN_GEN_lr": 1.0}
+    rows = run_program(f"ref-sgd-{schedule}", 1, ranks, 10, 10, 1, env=env)
+    assert rows[0][0] == n
+    g, (w,) = emitted_inputs(ranks, n, 1)
+    orc.sgd_f32(g, w, 1.0)
+    got = np.fromfile(f"{prefix}.w.{n}.f32", dtype=np.float32)
+    assert np.array_equal(got.view(np.uint32), w.view(np.uint32)), ("sgd", schedule)
+    run_program(f"ref-adam-{schedule}", 1, ranks, 10, 10, 1, env=env)
+    g, (w, m, v) = emitted_inputs(ranks, n, 3)
+    orc.pseudo_adam_f32(g, w, m, v, 1.0, 0.5, 0.5)
+    for name, want in (("w", w), ("m", m), ("v", v)):
+        got = np.fromfile(f"{prefix}.{name}.{n}.f32", dtype=np.float32)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), ("adam", schedule, name)
+
+
+@pytest.mark.parametrize("schedule", ["rs-c-ag", "fuse-rs-c-ag"])
+@pytest.mark.parametrize("n,ranks,rank", [(10, 4, 0), (10, 4, 3), (4099, 4, 2), (5, 8, 6)])
+def test_one_rank_updates_its_slice_only(tmp_path, schedule, n, ranks, rank):
+    """The emitted driver takes the reference's (comm_size, rank) pair and runs that rank's share: elements
+    [DIVUP(n, ranks) * rank, + DIVUP(n, ranks)) clipped at n (src/codegen.cpp:485-499 of the reference).  With n = 10 on 4
+    ranks the slices are [0,3) [3,6) [6,9) [9,10); with 5 elements on 8 ranks, ranks 5 to 7 have nothing to do."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    run_program(f"ref-sgd-{schedule}", 1, ranks, 10, 10, 1,
+                env={"CCN_GEN_N": n, "CCN_GEN_DUMP": prefix, "CCN_GEN_ONLY_RANK": rank})
+    g, (w0,) = emitted_inputs(ranks, n, 1)
+    w = w0.copy()
+    orc.sgd_f32(g, w, 0.5)
+    per = -(-n // ranks)
+    lo, hi = min(per * rank, n), min(per * rank + per, n)
+    want = w0.copy()
+    want[lo:hi] = w[lo:hi]
+    got = np.fromfile(f"{prefix}.w.{n}.f32", dtype=np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (lo, hi)
+
+
+def test_the_emitted_check_catches_a_wrong_result():
+    """One device value corrupted by a part in a thousand before the comparison: the program must say so and exit 2."""
+    for name in ("sgd-fused", "ref-adam-rs-c-ag", "lamb-fused"):
+        r = run_raw(name, 1, 4, 12, 12, 1, env={"CCN_GEN_PERTURB": 1})
+        assert r.returncode == 2, (name, r.returncode, r.stdout[-500:])
+        assert "Mismatch in" in r.stdout and "Results do not match the CPU re-execution" in r.stdout
+        ok = run_raw(name, 1, 4, 12, 12, 1)
+        assert ok.returncode == 0 and "do not match" not in ok.stdout
 
 
 @pytest.mark.parametrize("name", ["ref-model-parallel-mm-ar-c", "ref-model-parallel-mm-rs-c-ag",

@@ -357,6 +357,19 @@ def test_fused_adam_reference_variant(ccn):
         hw = torch.zeros(N, dtype=torch.int16, device=DEV)
         ccn.fused_adam_ref_f16g(ones, w, hw, m, v, N, 1.0, 0.5, 0.5)
         assert np.all(host(w) == -1.0) and np.all(host_u16(hw) == 0xBC00)
+    # beta1 != beta2, by hand: the kernel decays the first moment with beta2 (common_kernel.h:878) and divides it by
+    # beta1 (:879).  One rank, g = 1, lr = 1, beta1 = 1/2, beta2 = 1/4: m = 3/4 then 15/16; w = -(3/2)/sqrt(3), then
+    # minus (15/8)/sqrt(15/4); with beta1 in the decay m would be 1/2 then 3/4.
+    N = 777
+    one = [torch.ones(N, dtype=torch.float16, device=DEV)]
+    w, m, v = (torch.zeros(N, device=DEV) for _ in range(3))
+    hw = torch.zeros(N, dtype=torch.int16, device=DEV)
+    f = np.float32
+    ccn.fused_adam_ref_f16g(one, w, hw, m, v, N, 1.0, 0.5, 0.25)
+    w1 = f(0) - f(1.5) / np.sqrt(f(3.0))
+    assert np.all(host(m) == f(0.75)) and np.all(host(v) == f(0.75)) and np.all(host(w) == w1)
+    ccn.fused_adam_ref_f16g(one, w, hw, m, v, N, 1.0, 0.5, 0.25)
+    assert np.all(host(m) == f(15 / 16)) and np.all(host(w) == w1 - f(15 / 8) / np.sqrt(f(15 / 4)))
     P, N = 8, 100001
     g16 = [orc.f32_to_f16(x) for x in grads_f32(23, P, N, 0.5)]
     w0 = weights_f32(23, N, 0.05)
@@ -532,7 +545,8 @@ def test_lamb_reference_fixture(ccn):
 
 def test_lamb_full_size_segments(ccn):
     """benchmark configuration 4 at full size (N = 2^28 as 256 segments of 2^20, P = 8): the oracle is run on four
-    whole segments (first, two inner, last); segments are independent, so this is exact for them."""
+    whole segments (first, two inner, last); segments are independent, so this is exact for them.  The norms of all
+    256 segments are then checked against float64 norms and against the two-pass kernels' norms of the same step."""
     P, nseg, seglen = 8, 256, 1 << 20
     N = nseg * seglen
     gen = torch.Generator(device=DEV)
@@ -544,6 +558,7 @@ def test_lamb_full_size_segments(ccn):
     check = [0, 77, 200, 255]
     hg = {b: [host(x[b * seglen:(b + 1) * seglen]).copy() for x in g] for b in check}
     hw = {b: host(w[b * seglen:(b + 1) * seglen]).copy() for b in check}
+    w0 = w.clone()
     plan = ccn.LambPlan([i * seglen for i in range(nseg + 1)])
     plan.step(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, ccn.LAMB_TRUST_RATIO)
     norms = plan.norms()
@@ -554,9 +569,41 @@ def test_lamb_full_size_segments(ccn):
         sl = slice(b * seglen, (b + 1) * seglen)
         assert_f32_parity(host(m[sl]), mm, f"segment {b} m")
         assert np.max(np.abs(host(w[sl]).astype(np.float64) - ww)) <= FP32_TOL * np.max(np.abs(ww))
-    del g
     plan.close()
     assert norms.shape == (nseg, 2) and np.all(norms > 0)
+    # Every segment, not only the four above.  The one-tile kernel passes tile sums between workgroups of one launch: a
+    # tile sum that arrived late or stale would show in that segment's norms and nowhere else.  (a) against float64
+    # norms computed by torch on the device from the weights before the step and the moments after it; (b) against the
+    # two-pass kernels, which exchange nothing inside a launch, on the same inputs: their sums associate differently, so
+    # equal to rounding, not to the bit.
+    b1, b2, eps, wd = 0.9, 0.999, 1e-6, 0.01
+    ref = np.empty((nseg, 2))
+    for b in range(nseg):
+        sl = slice(b * seglen, (b + 1) * seglen)
+        mh = (m[sl].double() / (1 - b1)).float()
+        vh = (v[sl].double() / (1 - b2)).float()
+        r = mh.double() / (vh.sqrt().double() + eps) + wd * w0[sl].double()
+        ref[b] = [float(w0[sl].double().pow(2).mean().sqrt()), float(r.pow(2).mean().sqrt())]
+    assert rel_err(norms, ref) < 1e-6, rel_err(norms, ref)
+    w2, m2, v2 = w0, torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    import os
+    saved = os.environ.get("CCN_LAMB_RESIDENT")
+    os.environ["CCN_LAMB_RESIDENT"] = "0"
+    try:
+        plan2 = ccn.LambPlan([i * seglen for i in range(nseg + 1)])
+    finally:
+        if saved is None:
+            del os.environ["CCN_LAMB_RESIDENT"]
+        else:
+            os.environ["CCN_LAMB_RESIDENT"] = saved
+    plan2.step(g, w2, m2, v2, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, ccn.LAMB_TRUST_RATIO)
+    norms2 = plan2.norms()
+    plan2.close()
+    assert rel_err(norms, norms2) < 1e-12, rel_err(norms, norms2)
+    assert torch.equal(m, m2) and torch.equal(v, v2)
+    ulps = (w.view(torch.int32).long() - w2.view(torch.int32).long()).abs().max().item()
+    assert ulps <= 2, ulps
+    del g
 
 
 def test_lamb_nccl_global_variant(ccn):

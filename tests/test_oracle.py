@@ -136,6 +136,29 @@ def test_fused_adam_a3_known_answer(P):
     assert np.all(w == -1.0) and np.all(hw == 0xBC00)
 
 
+def test_fused_adam_a3_first_moment_decays_with_beta2():
+    """The kernel runs its first-moment functor through `.mixedbinOp1(beta2, mval, ...)`
+    (nccl/src/collectives/device/common_kernel.h:878): m decays with beta2, and only the division S3 = m/beta1 (:879)
+    sees beta1.  With beta1 != beta2 the two readings differ; values by hand, one rank, g = 1, w = m = v = 0, lr = 1,
+    beta1 = 1/2, beta2 = 1/4 (every intermediate is exact in binary):
+      step 1: v = 3/4, S4 = v/beta2 = 3;  m = (1 - beta2) = 3/4 (1 - beta1 would give 1/2);  S3 = m/beta1 = 3/2;
+              w = -(3/2)/sqrt(3)
+      step 2: m = 3/4 * 1/4 + 3/4 = 15/16 (beta1 would give 3/4), v = 15/16, S4 = 15/4, S3 = 15/8;
+              w -= (15/8)/sqrt(15/4)"""
+    g = [np.array([0x3C00], np.uint16)]
+    w, m, v = (np.zeros(1, np.float32) for _ in range(3))
+    hw = np.zeros(1, np.uint16)
+    f = np.float32
+    orc.fused_adam_a3(g, w, m, v, hw, 1.0, 0.5, 0.25)
+    assert m[0] == f(0.75) and v[0] == f(0.75)
+    w1 = f(0) - f(1.5) / np.sqrt(f(3.0))
+    assert w[0] == w1
+    orc.fused_adam_a3(g, w, m, v, hw, 1.0, 0.5, 0.25)
+    assert m[0] == f(15 / 16) and v[0] == f(15 / 16)
+    assert w[0] == w1 - f(15 / 8) / np.sqrt(f(15 / 4))
+    assert hw[0] == np.float16(w[0]).view(np.uint16)
+
+
 def test_fused_adam_a3_half_precision_effects():
     # the sum is carried in fp16: 2048 + 1 is not representable in half (spacing 2), so the second rank's
     # gradient is lost; an fp32 sum would give 2049.  The square is also rounded to half: 3.001^2.
