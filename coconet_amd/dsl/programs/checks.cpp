@@ -95,6 +95,54 @@ int main(int argc, char** argv) {
     pl.print(std::cout);
     return 0;
   }
+  if (c == "dims_mismatch_leading") {
+    // y has the FIRST dimension of x only: numpy-style broadcast matches trailing dimensions
+    Variable B(Int32, "B"), S(Int32, "S"), H(Int32, "H");
+    Tensor x(Float32, {B, S, H}, Replicated, "x");
+    Tensor y(Float32, B, Replicated, "y");
+    Stage s = x + y;
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "dims_mismatch_same_rank") {
+    Variable N(Int32, "N"), M(Int32, "M");
+    Tensor x(Float32, N, Replicated, "x");
+    Tensor y(Float32, M, Replicated, "y");
+    Stage s = x * y;
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "dims_mismatch_in_select") {
+    Variable N(Int32, "N"), M(Int32, "M");
+    Tensor x(Float32, N, Replicated, "x");
+    Tensor y(Float32, M, Replicated, "y");
+    Stage s = Ite(x > 0, x, y);
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "update_with_more_dims") {
+    Variable B(Int32, "B"), H(Int32, "H");
+    Tensor x(Float32, {B, H}, Replicated, "x");
+    Tensor b(Float32, H, Replicated, "b");
+    Stage s = Update(b, x + b);
+    std::cout << "not rejected" << std::endl;
+    return 0;
+  }
+  if (c == "broadcast_bias") {
+    // a bias over the last dimension added to a [B, S, H] value outside any MatMul: read modulo its element count
+    Variable B(Int32, "B"), S(Int32, "S"), H(Int32, "H");
+    Variable lr(Float32, "lr");
+    Tensor g(Float32, {B, S, H}, Local, "g");
+    Tensor x(Float32, {B, S, H}, Replicated, "x");
+    Tensor b(Float32, H, Replicated, "b");
+    Tensor sh(Float32, {S, H}, Replicated, "sh");
+    Stage g1 = AllReduce(Summation, g);
+    Stage x1 = Update(x, x - lr * ((g1 + b) * sh));
+    Pipeline pl("bc", {g, x, b, sh, lr}, {x1});
+    pl.fuse({g1, x1});
+    std::cout << generateHIP(pl, {});
+    return 0;
+  }
   if (c == "bad_file") {
     AdamParts a;
     Pipeline pl("adam", {a.g, a.w, a.m, a.v, a.lr, a.beta1, a.beta2}, {a.m1, a.v1, a.w1});

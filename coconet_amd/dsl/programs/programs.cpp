@@ -1,6 +1,6 @@
 // DSL programs for the benchmark configurations, written against the CoCoNet API.
 //   ccn-programs <program> <schedule> [output.hip]
-// program: sgd | clipsgd | reduction | adam | adamf16 | lamb     schedule: unfused | fused (adamf16: fused only)
+// program: sgd | biasadd | clipsgd | reduction | adam | adamf16 | lamb     schedule: unfused | fused (adamf16: fused only)
 #include <dsl.hpp>
 #include <pipeline.hpp>
 
@@ -17,6 +17,21 @@ static void sgd(bool fused, const std::string& out) {
   Stage gsum = AllReduce(Summation, g);
   Stage wnew = Update(w, w - lr * gsum);
   Pipeline pl("sgd", {g, w, lr}, {wnew});
+  if (fused) pl.fuse({gsum, wnew});
+  pl.codegen(out);
+}
+
+// SGD on a matrix of weights with a per-column term added to the summed gradient: b has the last dimension only and is
+// broadcast over the rows, numpy-style, as the reference's pointwise stages do (src/pipeline.cpp:14-90)
+static void biasadd(bool fused, const std::string& out) {
+  Variable B(Int32, "B"), H(Int32, "H");
+  Variable lr(Float32, "lr");
+  Tensor g(Float32, {B, H}, Local, "g");
+  Tensor w(Float32, {B, H}, Replicated, "w");
+  Tensor b(Float32, H, Replicated, "b");
+  Stage gsum = AllReduce(Summation, g);
+  Stage wnew = Update(w, w - lr * (gsum + b));
+  Pipeline pl("biasadd", {g, w, b, lr}, {wnew});
   if (fused) pl.fuse({gsum, wnew});
   pl.codegen(out);
 }
@@ -117,7 +132,7 @@ static void lamb(bool fused, const std::string& out) {
 
 int main(int argc, char** argv) {
   if (argc < 3) {
-    std::cout << "usage: " << argv[0] << " <sgd|clipsgd|reduction|adam|adamf16|lamb> <unfused|fused> [output.hip]" << std::endl;
+    std::cout << "usage: " << argv[0] << " <sgd|biasadd|clipsgd|reduction|adam|adamf16|lamb> <unfused|fused> [output.hip]" << std::endl;
     return 1;
   }
   const std::string prog = argv[1], sched = argv[2];
@@ -125,6 +140,7 @@ int main(int argc, char** argv) {
   if (!fused && sched != "unfused") { std::cout << "Invalid schedule" << std::endl; return 1; }
   const std::string out = argc > 3 ? argv[3] : prog + "-" + sched + ".hip";
   if (prog == "sgd") sgd(fused, out);
+  else if (prog == "biasadd") biasadd(fused, out);
   else if (prog == "clipsgd") clipsgd(fused, out);
   else if (prog == "reduction") reduction(fused, out);
   else if (prog == "adam") adam(fused, out);

@@ -85,10 +85,53 @@ static TensorElemType promote(TensorElemType a, TensorElemType b) {
   return rank(a) >= rank(b) ? a : b;
 }
 
+// dimensions of a tensor-valued expression: its own when it carries them, otherwise those of its operands
+static std::vector<NodePtr> dims_of(const NodePtr& n) {
+  if (!n->dims.empty()) return n->dims;
+  std::vector<NodePtr> d;
+  if (n->kind == Kind::Norm) return d;
+  for (auto& a : n->args) {
+    if (is_scalar(a)) continue;
+    auto da = dims_of(a);
+    if (da.size() > d.size()) d = da;
+  }
+  return d;
+}
+
+static std::string dims_text(const std::vector<NodePtr>& d) {
+  std::string s = "[";
+  for (size_t k = 0; k < d.size(); k++) s += (k ? ", " : "") + d[k]->name;
+  return s + "]";
+}
+
+// Dimensions of a pointwise operation over a and b.  The reference's rule (BinaryPointwiseOp::setupAndCheckDimensions,
+// src/pipeline.cpp:14-90): scalars adapt to the other operand; of two tensor-valued operands the one with fewer
+// dimensions is broadcast numpy-style, its dimensions matched against the TRAILING dimensions of the other; matching
+// means being the same dimension variable.  Anything else is rejected here, on the host, where the program is built:
+// the emitted kernels index every operand by the stage's element index and check nothing.
+static bool single_value(const NodePtr& n) {   // scalars, and norms / whole-tensor sums: one value, whatever they were taken over
+  return is_scalar(n) || n->kind == Kind::Norm || (n->kind == Kind::Stage && n->args[0]->kind == Kind::Norm);
+}
+static std::vector<NodePtr> broadcast_dims(const NodePtr& a, const NodePtr& b, const char* what) {
+  if (single_value(a)) return single_value(b) ? std::vector<NodePtr>{} : dims_of(b);
+  if (single_value(b)) return dims_of(a);
+  const auto da = dims_of(a), db = dims_of(b);
+  const auto& lng = da.size() >= db.size() ? da : db;
+  const auto& sht = da.size() >= db.size() ? db : da;
+  for (size_t k = 0; k < sht.size(); k++) {
+    const NodePtr& x = lng[lng.size() - sht.size() + k];
+    const NodePtr& y = sht[k];
+    ASSERT(x == y, what << ": operand dimensions " << dims_text(da) << " and " << dims_text(db) << " do not match ('"
+                        << x->name << "' against '" << y->name << "')");
+  }
+  return lng;
+}
+
 static NodePtr binary(BinOp op, const Expression& a, const Expression& b) {
   auto n = make(Kind::Binary);
   n->bin = op;
   n->args = {a.impl(), b.impl()};
+  n->dims = broadcast_dims(a.impl(), b.impl(), "pointwise operation");
   // a constant adapts to the other operand (1 - beta1 is a float expression)
   TensorElemType ta = a.impl()->elem, tb = b.impl()->elem;
   if (a.impl()->kind == Kind::Const) ta = tb;
@@ -110,6 +153,7 @@ Expression operator/(const Expression& a, const Expression& b) { return Expressi
 Expression operator>(const Expression& a, const Expression& b) {
   auto n = make(Kind::Compare);
   n->args = {a.impl(), b.impl()};
+  n->dims = broadcast_dims(a.impl(), b.impl(), "comparison");
   n->elem = Int32;
   n->layout = is_scalar(a.impl()) ? b.impl()->layout : a.impl()->layout;
   return Expression(n);
@@ -143,17 +187,6 @@ Tensor::Tensor(TensorElemType t, Variable n1, Variable n2, TensorLayout layout, 
 Tensor::Tensor(TensorElemType t, std::vector<Variable> dims, TensorLayout layout, std::string name)
     : Expression(tensor(t, dims, layout, std::move(name))) {}
 
-// dimensions of a tensor-valued expression = those of its first tensor-valued operand
-static std::vector<NodePtr> dims_of(const NodePtr& n) {
-  if (!n->dims.empty()) return n->dims;
-  for (auto& a : n->args) {
-    if (is_scalar(a)) continue;
-    auto d = dims_of(a);
-    if (!d.empty()) return d;
-  }
-  return {};
-}
-
 static NodePtr stage(const Expression& def) {
   ASSERT(!is_scalar(def.impl()), "a stage must be tensor valued");
   auto n = make(Kind::Stage);
@@ -178,6 +211,12 @@ static NodePtr unary_like(Kind k, const Expression& x) {
 Expression Update(const Tensor& t, const Expression& definition) {
   ASSERT(t.impl()->kind == Kind::Tensor, "Update target must be a tensor");
   auto n = make(Kind::Update);
+  if (!is_scalar(definition.impl())) {
+    // the new value has the tensor's dimensions, or fewer that broadcast into them; never more
+    const auto d = broadcast_dims(t.impl(), definition.impl(), "Update");
+    ASSERT(d.size() == t.impl()->dims.size(), "Update: the value has more dimensions " << dims_text(dims_of(definition.impl()))
+                                                  << " than tensor '" << t.impl()->name << "' " << dims_text(t.impl()->dims));
+  }
   n->args = {t.impl(), definition.impl()};
   n->elem = t.impl()->elem;
   n->layout = t.impl()->layout;
@@ -203,6 +242,12 @@ Expression Ite(const Expression& cond, const Expression& ifTrue, const Expressio
   auto n = make(Kind::Select);
   const NodePtr both = binary(BinOp::Add, ifTrue, ifFalse);
   n->args = {cond.impl(), ifTrue.impl(), ifFalse.impl()};
+  {
+    auto probe = make(Kind::Binary);   // the branches' dimensions, then the condition's against them
+    probe->dims = both->dims;
+    probe->args = {ifTrue.impl(), ifFalse.impl()};
+    n->dims = is_scalar(both) ? dims_of(cond.impl()) : broadcast_dims(probe, cond.impl(), "Ite");
+  }
   n->elem = both->elem;
   n->layout = is_scalar(both) ? cond.impl()->layout : both->layout;
   return Expression(n);

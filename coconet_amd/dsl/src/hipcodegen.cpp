@@ -120,6 +120,9 @@ struct Body {
   unsigned outHalfMask = 0;              // output array k holds fp16
   std::set<std::string> scalars;         // variable names used
   bool usesSeed = false;
+  // operands with fewer dimensions than the kernel's values (a bias over the last dimension): read at element index
+  // modulo their own element count, the reference's numpy-style broadcast (src/codegen.cpp:495-496)
+  std::vector<std::pair<std::string, std::string>> bcArrays;   // (array, element count expression)
 };
 
 struct BodyBuilder {
@@ -131,9 +134,28 @@ struct BodyBuilder {
   std::map<int, std::string> stageValue;            // stage index -> local value name
   std::map<int, int> normIndex;                     // Norm stage index -> slot
   bool phase2 = false;
+  std::vector<NodePtr> domain;                      // dimensions of the values the kernel walks
 
   BodyBuilder(Program& pr, const Pipeline::Group& g) : prog(pr), group(g) {
     for (int s : g.stages) inGroup.insert(s);
+    domain = pr.p.stages()[first_tensor_stage(pr.p, g.stages)]->dims;
+    if (domain.empty()) {   // a kernel of norms only takes the dimensions of what it sums
+      const NodePtr& x = pr.p.stages()[g.stages[0]]->args[0]->args[0];
+      domain = x->dims;
+    }
+  }
+
+  // Reads `array`, whose values have dimensions `dims`, inside this kernel: at the element index when the dimensions
+  // are the kernel's, modulo its element count when they are a trailing part of them (the front end has checked that).
+  std::string read(const std::string& array, const std::string& hint, const NodePtr& owner) {
+    if (owner->dims == domain || owner->dims.empty()) return input(array, hint);
+    ASSERT(owner->dims.size() < domain.size() &&
+               std::equal(owner->dims.begin(), owner->dims.end(), domain.end() - (long)owner->dims.size()),
+           "value '" << hint << "' does not have the dimensions of the kernel that reads it, nor trailing ones");
+    bool known = false;
+    for (auto& b : body.bcArrays) known = known || b.first == array;
+    if (!known) body.bcArrays.push_back({array, count_expr(owner)});
+    return "s.bc_" + hint + "[idx % s.bcn_" + hint + "]";
   }
 
   std::string input(const std::string& array, const std::string& hint) {
@@ -151,7 +173,7 @@ struct BodyBuilder {
         ASSERT(n->layout != Local, "tensor '" << n->name << "' is Local: it can only be read through AllReduce/ReduceScatter");
         auto it = tensorValue.find(n.get());
         if (it != tensorValue.end()) return it->second;
-        return tensorValue[n.get()] = input(n->name, n->name);
+        return tensorValue[n.get()] = read(n->name, n->name, n);
       }
       case Kind::Variable: body.scalars.insert(n->name); return "s." + n->name;
       case Kind::Const: return fconst(n);
@@ -203,7 +225,7 @@ struct BodyBuilder {
         }
         ASSERT(!inGroup.count(k) || phase2, "stage " << n->name << " used before it is computed");
         ASSERT(prog.stageBuf.count(k), "stage " << n->name << " has no buffer but is read by another kernel");
-        return stageValue[k] = input(prog.stageBuf[k], n->name);
+        return stageValue[k] = read(prog.stageBuf[k], n->name, n);
       }
       case Kind::Update:
       case Kind::Norm:
@@ -268,6 +290,10 @@ std::string body_text(const Body& b, const std::vector<NodePtr>& scalarVars) {
   o << "  static constexpr unsigned OUT_F16 = " << b.outHalfMask << "u;\n";
   o << "  struct Scalars {";
   for (auto& v : scalarVars) o << " " << elem_c_type(v->elem) << " " << v->name << ";";
+  for (auto& bc : b.bcArrays) {
+    const std::string nm = bc.first.substr(0, bc.first.find('['));
+    o << " const float* bc_" << nm << "; size_t bcn_" << nm << ";";
+  }
   o << " uint64_t seed__; };\n";
   o << "  static __host__ __device__ __forceinline__ void apply(float red, const float* in, float* out, const Scalars& s,\n"
        "                                                        double* acc, const float* nrm, uint64_t idx) {\n";
@@ -519,6 +545,10 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
     for (size_t k = 0; k < b.outArrays.size(); k++) q << "  " << var << ".out[" << k << "] = " << b.outArrays[k] << plus << ";\n";
     q << "  " << var << ".partials = partials__;\n  " << var << ".norms = norms__;\n  " << var << ".n = " << count << ";\n";
     q << "  " << var << ".idx_base = " << (off.empty() ? "0" : off) << ";\n";
+    for (auto& bc : b.bcArrays) {
+      const std::string nm = bc.first.substr(0, bc.first.find('['));
+      q << "  " << var << ".s.bc_" << nm << " = " << bc.first << ";\n  " << var << ".s.bcn_" << nm << " = " << bc.second << ";\n";
+    }
     q << scalars_init(var);
     return q.str();
   };
@@ -599,9 +629,13 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   o << ", int comm_size, uint64_t seed__) {\n  (void)seed__; (void)comm_size;\n";
   {
     // host expression emitter: arrays indexed by i0
+    std::vector<NodePtr> hostDomain;   // dimensions of the stage whose loop is being written
+    auto at = [&](const NodePtr& n) {
+      return (n->dims.empty() || n->dims == hostDomain) ? std::string("[i0]") : "[i0 % h." + n->name + ".size()]";
+    };
     std::function<std::string(const NodePtr&)> he = [&](const NodePtr& n) -> std::string {
       switch (n->kind) {
-        case Kind::Tensor: return "h." + n->name + "[i0]";
+        case Kind::Tensor: return "h." + n->name + at(n);
         case Kind::Variable: return n->name;
         case Kind::Const: return fconst(n);
         case Kind::Binary: {
@@ -631,7 +665,7 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
           return he(n->args[0]);
         case Kind::Stage: {
           if (n->args[0]->kind == Kind::Norm) return "h." + n->name + "[0]";
-          return "h." + n->name + "[i0]";
+          return "h." + n->name + at(n);
         }
         default: ASSERT(false, "unexpected node in a stage expression"); return "";
       }
@@ -644,6 +678,7 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
       if (def->kind == Kind::Norm) {
         const NodePtr& x = def->args[0];
         ASSERT(x->kind == Kind::Stage || x->kind == Kind::Tensor, "Norm takes a stage or a tensor");
+        hostDomain = x->dims;
         o << "  { double a_ = 0.0; const size_t n_ = " << count_expr(x) << ";\n";
         if (def->plain_sum) {
           o << "    for (size_t i0 = 0; i0 < n_; i0++) a_ += (double)(" << he(x) << ");\n";
@@ -655,6 +690,7 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
         continue;
       }
       const std::string cnt = count_expr(st);
+      hostDomain = st->dims;
       o << "  h." << st->name << ".resize(" << cnt << ");\n";
       o << "  for (size_t i0 = 0; i0 < " << cnt << "; i0++) {\n";
       if (def->kind == Kind::Update) {

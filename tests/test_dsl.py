@@ -48,12 +48,32 @@ def test_storage_classes_and_fusion_groups(dsl_build):
     ("allgather_of_replicated", "must be Sliced"),
     ("local_read_without_collective", "is Local"),
     ("missing_argument", "not a pipeline argument"),
+    # operands of one pointwise operation must have the same dimensions, or trailing ones (src/pipeline.cpp:14-90 of the
+    # reference): anything else would make the emitted kernel read an operand past its end
+    ("dims_mismatch_leading", "do not match"),
+    ("dims_mismatch_same_rank", "do not match"),
+    ("dims_mismatch_in_select", "do not match"),
+    ("update_with_more_dims", "more dimensions"),
 ])
 def test_invalid_programs_abort_with_a_message(dsl_build, case, needle):
     """Error convention of the reference (src/ast.hpp:33-44): message on stderr, then std::terminate()."""
     r = run(os.path.join(dsl_build, "ccn-dsl-check"), case)
     assert r.returncode != 0 and "not rejected" not in r.stdout
     assert "ASSERT failed" in r.stderr and needle in r.stderr
+
+
+def test_trailing_dimensions_broadcast(dsl_build):
+    """x[B,S,H] op b[H] and op sh[S,H]: the smaller operand is read at element index modulo its own element count, in the
+    kernel and in the emitted CPU re-execution (the reference's `%` of src/codegen.cpp:495-496); the full-size operands
+    stay plain streamed inputs."""
+    r = run(os.path.join(dsl_build, "ccn-dsl-check"), "broadcast_bias")
+    assert r.returncode == 0, r.stderr
+    text = r.stdout
+    assert "s.bc_b[idx % s.bcn_b]" in text and "s.bc_sh[idx % s.bcn_sh]" in text
+    assert "const float* bc_b; size_t bcn_b;" in text
+    assert "args0.s.bc_b = b;" in text and "args0.s.bcn_b = (size_t)H;" in text and "args0.s.bcn_sh = (size_t)S * H;" in text
+    assert "h.b[i0 % h.b.size()]" in text and "h.sh[i0 % h.sh.size()]" in text and "h.x[i0]" in text
+    assert "NIN = 1" in text            # x alone is streamed; g comes through the rank fold
 
 
 def test_unwritable_output_reports_and_returns(dsl_build):

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GEN = os.path.join(ROOT, "coconet_amd", "dsl", "build", "gen")
 LINE = re.compile(r"^\{SZ: (\d+), Epochs: (\d+)((?:, \w+: [0-9.eE+-]+)+)\}$")
 
-OWN = ["sgd-fused", "sgd-unfused", "clipsgd-fused", "clipsgd-unfused", "reduction-fused", "reduction-unfused", "adam-fused", "adam-unfused", "adamf16-fused", "lamb-fused", "lamb-unfused"]
+OWN = ["sgd-fused", "sgd-unfused", "biasadd-fused", "biasadd-unfused", "clipsgd-fused", "clipsgd-unfused", "reduction-fused", "reduction-unfused", "adam-fused", "adam-unfused", "adamf16-fused", "lamb-fused", "lamb-unfused"]
 REF = ["ref-sgd-ar-c", "ref-sgd-rs-c-ag", "ref-sgd-fuse-rs-c-ag", "ref-adam-ar-c", "ref-adam-rs-c-ag",
        "ref-adam-fuse-rs-c-ag", "ref-lamb-ar-c", "ref-lamb-rs-c-ag", "ref-lamb-fuse-rs-c-ag"]
 
@@ -54,9 +54,13 @@ def run_program(name, *args, env=None):
 @pytest.mark.parametrize("name", OWN)
 @pytest.mark.parametrize("ranks", [1, 4, 8, 11])
 def test_own_programs_check_themselves(name, ranks):
-    # sizes 2^10 .. 2^21 with the CPU re-execution switched on
-    rows = run_program(name, 2, ranks, 10, 21, 1)
-    assert [r[0] for r in rows] == [1 << k for k in range(10, 22)]
+    # sizes 2^10 .. 2^21 with the CPU re-execution switched on (biasadd walks a B x H matrix with B = H = 2^k)
+    if name.startswith("biasadd"):
+        rows = run_program(name, 2, ranks, 1, 10, 1)
+        assert [r[0] for r in rows] == [1 << (2 * k) for k in range(1, 11)]
+    else:
+        rows = run_program(name, 2, ranks, 10, 21, 1)
+        assert [r[0] for r in rows] == [1 << k for k in range(10, 22)]
     for size, epochs, f in rows:
         assert epochs == 2 and abs(sum(v for k, v in f.items() if k != "Total") - f["Total"]) < 1e-3
     steps = set(rows[0][2]) - {"Total"}
