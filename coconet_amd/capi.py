@@ -34,6 +34,7 @@ SYMBOLS = [
     "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
     "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
     "ccn_lamb_f32_scattered", "ccn_adam_bf16g", "ccn_lamb_nccl_f16g", "ccn_lamb_f32_static",
+    "ccn_mlp_outproj_bf16_ex", "ccn_bias_dropout_residual_ex", "ccn_matmul_bf16_f32",
 ]
 
 
@@ -104,6 +105,9 @@ def _declare(L):
     sig("ccn_lamb_nccl_f16g", [_vp, _pp, _i, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _vp])
     sig("ccn_mlp_outproj_bf16", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _vp])
     sig("ccn_bias_dropout_residual", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _vp])
+    sig("ccn_mlp_outproj_bf16_ex", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _i, _vp])
+    sig("ccn_bias_dropout_residual_ex", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _i, _sz, _vp])
+    sig("ccn_matmul_bf16_f32", [_vp, _vp, _vp, _i, _i, _i, _vp])
     sig("ccn_scatter_plan_create", [C.POINTER(_sz), _i, _pp])
     sig("ccn_scatter_plan_destroy", [_vp])
     sig("ccn_sgd_f32_scattered", [_vp, _pp, _i, _pp, _f, _vp])
@@ -397,13 +401,29 @@ def lamb_f32_static(g, w, m, v, n, seg_len, lr, beta1, beta2, eps, wd, step, mod
                                       mode, addr(norms), stream), "ccn_lamb_f32_static")
 
 
-def mlp_outproj_bf16(X, W, partials, bias, resid, out, M, N, K, p_drop, seed, stream=None):
-    p, _keep = ptr_table(partials)
-    _check(load().ccn_mlp_outproj_bf16(addr(X), addr(W), p, len(partials), addr(bias), addr(resid), addr(out), M, N, K,
-                                       p_drop, seed, stream), "ccn_mlp_outproj_bf16")
+DROPOUT_INVERTED, DROPOUT_REF_DSL, DROPOUT_REF_NCCL, DROPOUT_REF_NCCL_SAT = 0, 1, 2, 3
 
 
-def bias_dropout_residual(acc, partials, bias, resid, out, M, N, p_drop, seed, stream=None):
+def mlp_outproj_bf16(X, W, partials, bias, resid, out, M, N, K, p_drop, seed, stream=None, dropout_mode=None):
     p, _keep = ptr_table(partials)
-    _check(load().ccn_bias_dropout_residual(addr(acc), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
-                                            p_drop, seed, stream), "ccn_bias_dropout_residual")
+    if dropout_mode is None:
+        _check(load().ccn_mlp_outproj_bf16(addr(X), addr(W), p, len(partials), addr(bias), addr(resid), addr(out), M, N, K,
+                                           p_drop, seed, stream), "ccn_mlp_outproj_bf16")
+    else:
+        _check(load().ccn_mlp_outproj_bf16_ex(addr(X), addr(W), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
+                                              K, p_drop, seed, dropout_mode, stream), "ccn_mlp_outproj_bf16_ex")
+
+
+def bias_dropout_residual(acc, partials, bias, resid, out, M, N, p_drop, seed, stream=None, dropout_mode=None, first_row=0):
+    p, _keep = ptr_table(partials)
+    if dropout_mode is None and first_row == 0:
+        _check(load().ccn_bias_dropout_residual(addr(acc), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
+                                                p_drop, seed, stream), "ccn_bias_dropout_residual")
+    else:
+        _check(load().ccn_bias_dropout_residual_ex(addr(acc), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
+                                                   p_drop, seed, dropout_mode or 0, first_row, stream),
+               "ccn_bias_dropout_residual_ex")
+
+
+def matmul_bf16_f32(X, W, Cmat, M, N, K, stream=None):
+    _check(load().ccn_matmul_bf16_f32(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_bf16_f32")

@@ -25,6 +25,7 @@ struct EpiPrm {
   float p_drop, keep_scale;
   uint32_t seed_lo, seed_hi;
   int apply_dropout;
+  int mode;   // CCN_DROPOUT_*
 };
 
 // Epilogue for four consecutive columns n..n+3 (n % 4 == 0) of row m, in two steps so that the loads of one quad can be
@@ -42,27 +43,60 @@ __device__ __forceinline__ void epilogue_load(EpiIn<NP>& in, const SrcTable<floa
   in.rv = u32x2{0u, 0u};
   if (resid) in.rv = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(resid + idx));
 }
-template <int NP>
+// [0, 1] clamp of the reference's __hadd2_sat (NaN gives 0)
+__device__ __forceinline__ float sat01(float x) { return x > 0.0f ? (x < 1.0f ? x : 1.0f) : 0.0f; }
+
+// idx: where the quad lies in memory; mask_idx: its element index in the whole [M x N] output, which the mask is drawn
+// from (the two differ when a call covers a band of rows of a larger output).
+// REF: one of the reference's dropout forms (k.mode says which); false: standard dropout, the form the kernels are
+// tuned for, compiled without the others.
+template <int NP, bool REF>
 __device__ __forceinline__ void epilogue_finish(f32x4 acc, const EpiIn<NP>& in, const float* __restrict__ bias,
-                                                uint16_t* __restrict__ out, size_t idx, size_t n, const EpiPrm& k) {
+                                                uint16_t* __restrict__ out, size_t idx, size_t n, const EpiPrm& k,
+                                                size_t mask_idx) {
   const f32x4 bv = *reinterpret_cast<const f32x4*>(bias + n);
   f32x4 s = acc;
 #pragma unroll
   for (int q = 0; q < NP; q++) s = s + in.pv[q];
-  const f32x4 t = s + bv;
-  f32x4 d = t;
-  if (k.apply_dropout) {
-    const uint64_t blk = (uint64_t)idx >> 2;
+  const float r0 = bf16_bits_to_f32((uint16_t)(in.rv[0] & 0xffffu)), r1 = bf16_bits_to_f32((uint16_t)(in.rv[0] >> 16));
+  const float r2 = bf16_bits_to_f32((uint16_t)(in.rv[1] & 0xffffu)), r3 = bf16_bits_to_f32((uint16_t)(in.rv[1] >> 16));
+  float y0, y1, y2, y3;
+  if constexpr (!REF) {
+    // drop with probability p, survivors scaled by 1/(1-p)
+    const f32x4 t = s + bv;
+    f32x4 d = t;
+    if (k.apply_dropout) {
+      const uint64_t blk = (uint64_t)mask_idx >> 2;
+      const Philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u, k.seed_lo, k.seed_hi);
+      d[0] = keep_from_word(r.x, k.p_drop) ? t[0] * k.keep_scale : 0.0f;
+      d[1] = keep_from_word(r.y, k.p_drop) ? t[1] * k.keep_scale : 0.0f;
+      d[2] = keep_from_word(r.z, k.p_drop) ? t[2] * k.keep_scale : 0.0f;
+      d[3] = keep_from_word(r.w, k.p_drop) ? t[3] * k.keep_scale : 0.0f;
+    }
+    y0 = d[0] + r0; y1 = d[1] + r1; y2 = d[2] + r2; y3 = d[3] + r3;
+  } else {
+    const uint64_t blk = (uint64_t)mask_idx >> 2;
     const Philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u, k.seed_lo, k.seed_hi);
-    d[0] = keep_from_word(r.x, k.p_drop) ? t[0] * k.keep_scale : 0.0f;
-    d[1] = keep_from_word(r.y, k.p_drop) ? t[1] * k.keep_scale : 0.0f;
-    d[2] = keep_from_word(r.z, k.p_drop) ? t[2] * k.keep_scale : 0.0f;
-    d[3] = keep_from_word(r.w, k.p_drop) ? t[3] * k.keep_scale : 0.0f;
+    // kept where u < p: the complement of keep_from_word's u >= p
+    const bool kp[4] = {!keep_from_word(r.x, k.p_drop), !keep_from_word(r.y, k.p_drop), !keep_from_word(r.z, k.p_drop),
+                        !keep_from_word(r.w, k.p_drop)};
+    const float rs[4] = {r0, r1, r2, r3};
+    float y[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      if (k.mode == CCN_DROPOUT_REF_DSL) {
+        // the reference's emitted expression (src/codegen.cpp:634-640): (u < p ? (sum + bias) : 0) + residual
+        const float t = s[e] + bv[e];
+        y[e] = (kp[e] ? t : 0.0f) + rs[e];
+      } else {
+        // the reference's fused kernel (nccl-overlap/src/collectives/device/reduce_kernel.h:192-213):
+        // ((u < p ? sum : 0) + bias) + residual; its half specialisation adds with saturation to [0, 1]
+        const float d = kp[e] ? s[e] : 0.0f;
+        y[e] = k.mode == CCN_DROPOUT_REF_NCCL_SAT ? sat01(sat01(d + bv[e]) + rs[e]) : (d + bv[e]) + rs[e];
+      }
+    }
+    y0 = y[0]; y1 = y[1]; y2 = y[2]; y3 = y[3];
   }
-  const float y0 = d[0] + bf16_bits_to_f32((uint16_t)(in.rv[0] & 0xffffu));
-  const float y1 = d[1] + bf16_bits_to_f32((uint16_t)(in.rv[0] >> 16));
-  const float y2 = d[2] + bf16_bits_to_f32((uint16_t)(in.rv[1] & 0xffffu));
-  const float y3 = d[3] + bf16_bits_to_f32((uint16_t)(in.rv[1] >> 16));
   u32x2 o;
   o[0] = (uint32_t)f32_to_bf16_bits(y0) | ((uint32_t)f32_to_bf16_bits(y1) << 16);
   o[1] = (uint32_t)f32_to_bf16_bits(y2) | ((uint32_t)f32_to_bf16_bits(y3) << 16);
@@ -71,7 +105,9 @@ __device__ __forceinline__ void epilogue_finish(f32x4 acc, const EpiIn<NP>& in, 
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 7); }
 
-template <int NP>
+// PLAIN: the product alone, written as fp32 [M x N] through `out` (no partial buffers, bias, dropout or residual).
+// REF: the epilogue applies one of the reference's dropout forms.
+template <int NP, bool PLAIN = false, bool REF = false>
 __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
                                                              const SrcTable<float, 8> parts,
                                                              const float* __restrict__ bias,
@@ -204,45 +240,59 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
       const int q = it * kBlock + t;
       return (m0 + half * 64 + q / (BN / 4)) * (size_t)N + n0 + (q % (BN / 4)) * 4;
     };
-    EpiIn<NP> cur;
-    epilogue_load<NP>(cur, parts, resid, index_of(0));
+    if constexpr (PLAIN) {
+      float* const outc = reinterpret_cast<float*>(out);
 #pragma unroll
-    for (int it = 0; it < kIters; it++) {
-      EpiIn<NP> nxt;
-      if (it + 1 < kIters) epilogue_load<NP>(nxt, parts, resid, index_of(it + 1));
-      const int q = it * kBlock + t;
-      const int row = q / (BN / 4), colq = q % (BN / 4);
-      const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
-      epilogue_finish<NP>(a, cur, bias, out, index_of(it), n0 + colq * 4, ep);
-      if (it + 1 < kIters) cur = nxt;
+      for (int it = 0; it < kIters; it++) {
+        const int q = it * kBlock + t;
+        const int row = q / (BN / 4), colq = q % (BN / 4);
+        *reinterpret_cast<f32x4*>(outc + index_of(it)) = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
+      }
+    } else {
+      EpiIn<NP> cur;
+      epilogue_load<NP>(cur, parts, resid, index_of(0));
+#pragma unroll
+      for (int it = 0; it < kIters; it++) {
+        EpiIn<NP> nxt;
+        if (it + 1 < kIters) epilogue_load<NP>(nxt, parts, resid, index_of(it + 1));
+        const int q = it * kBlock + t;
+        const int row = q / (BN / 4), colq = q % (BN / 4);
+        const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
+        epilogue_finish<NP, REF>(a, cur, bias, out, index_of(it), n0 + colq * 4, ep, index_of(it));
+        if (it + 1 < kIters) cur = nxt;
+      }
     }
   }
 }
 
 // Standalone epilogue over an fp32 product in memory: one quad per thread, no loop, the launch shape of the other
 // streaming kernels (the y dimension of the grid only comes into play beyond 2^30 workgroups).
-template <int NP, int BS>
+template <int NP, int BS, bool REF>
 __global__ __launch_bounds__(BS) void bias_dropout_residual_kernel(const float* __restrict__ acc, const SrcTable<float, 8> parts,
                                                                    const float* __restrict__ bias,
                                                                    const uint16_t* __restrict__ resid,
                                                                    uint16_t* __restrict__ out, const size_t total,
-                                                                   const size_t N, const EpiPrm ep) {
+                                                                   const size_t N, const size_t mask_base, const EpiPrm ep) {
   const size_t q = ((size_t)blockIdx.x + (size_t)blockIdx.y * gridDim.x) * BS + threadIdx.x;
   if (q >= total) return;
   const size_t idx = q * 4;              // rows are contiguous: element index of the quad
   EpiIn<NP> in;
   const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(acc + idx));
   epilogue_load<NP>(in, parts, resid, idx);
-  epilogue_finish<NP>(a, in, bias, out, idx, idx % N, ep);
+  epilogue_finish<NP, REF>(a, in, bias, out, idx, idx % N, ep, mask_base + idx);
 }
 
-static int make_epi(float p_drop, uint64_t seed, EpiPrm* ep) {
-  if (!(p_drop >= 0.0f) || !(p_drop < 1.0f)) return CCN_EINVAL;
+static int make_epi(float p_drop, uint64_t seed, int mode, EpiPrm* ep) {
+  if (mode < CCN_DROPOUT_INVERTED || mode > CCN_DROPOUT_REF_NCCL_SAT) return CCN_EINVAL;
+  // inverted dropout rescales by 1/(1-p): p < 1.  The reference's forms keep with probability p: p = 1 keeps everything.
+  if (!(p_drop >= 0.0f) || !(mode == CCN_DROPOUT_INVERTED ? p_drop < 1.0f : p_drop <= 1.0f)) return CCN_EINVAL;
   ep->p_drop = p_drop;
-  ep->keep_scale = 1.0f / (1.0f - p_drop);
+  ep->keep_scale = mode == CCN_DROPOUT_INVERTED ? 1.0f / (1.0f - p_drop) : 1.0f;
   ep->seed_lo = (uint32_t)seed;
   ep->seed_hi = (uint32_t)(seed >> 32);
-  ep->apply_dropout = p_drop > 0.0f ? 1 : 0;
+  // p = 0 drops nothing when dropping with probability p, and everything when keeping with probability p
+  ep->apply_dropout = (mode != CCN_DROPOUT_INVERTED || p_drop > 0.0f) ? 1 : 0;
+  ep->mode = mode;
   return CCN_OK;
 }
 
@@ -250,11 +300,11 @@ static int make_epi(float p_drop, uint64_t seed, EpiPrm* ep) {
 
 using namespace ccn;
 
-extern "C" {
+namespace {
 
-int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
-                         const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
-                         uint64_t seed, void* stream) {
+int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials, const float* bias,
+                   const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop, uint64_t seed, int mode,
+                   void* stream) {
   if (!X || !W || !bias || !out || nPartials < 0 || nPartials > 8 || (nPartials > 0 && !partials)) return CCN_EINVAL;
   if (M <= 0 || N <= 0 || K <= 0) return CCN_EINVAL;
   if (M % BM || N % BN || K % BK) return CCN_ERANGE;   // whole tiles only
@@ -265,7 +315,7 @@ int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* cons
   }
   if (!aligned16(X) || !aligned16(W) || !aligned16(bias) || !aligned16(out) || (resid && !aligned16(resid))) return CCN_EINVAL;
   EpiPrm ep;
-  int rc = make_epi(p_drop, seed, &ep);
+  int rc = make_epi(p_drop, seed, mode, &ep);
   if (rc != CCN_OK) return rc;
   const DeviceInfo* di = nullptr;
   rc = current_device_info(&di);
@@ -273,8 +323,11 @@ int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* cons
   const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
   hipStream_t s = as_stream(stream);
   switch (nPartials) {
-#define CCN_CASE(Q) \
-  case Q: hipLaunchKernelGGL((mlp_outproj_kernel<Q>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); break;
+#define CCN_CASE(Q)                                                                                                          \
+  case Q:                                                                                                                    \
+    if (mode == CCN_DROPOUT_INVERTED) hipLaunchKernelGGL((mlp_outproj_kernel<Q>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
+    else hipLaunchKernelGGL((mlp_outproj_kernel<Q, false, true>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
+    break;
     CCN_CASE(0) CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
 #undef CCN_CASE
   }
@@ -282,9 +335,8 @@ int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* cons
   return CCN_OK;
 }
 
-int ccn_bias_dropout_residual(const float* acc, const float* const* partials, int nPartials, const float* bias,
-                              const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
-                              void* stream) {
+int epilogue_launch(const float* acc, const float* const* partials, int nPartials, const float* bias, const uint16_t* resid,
+                    uint16_t* out, int M, int N, float p_drop, uint64_t seed, int mode, size_t first_row, void* stream) {
   if (!acc || !bias || !out || nPartials < 0 || nPartials > 8 || (nPartials > 0 && !partials)) return CCN_EINVAL;
   if (M <= 0 || N <= 0) return CCN_EINVAL;
   if (N % 4) return CCN_ERANGE;
@@ -295,7 +347,7 @@ int ccn_bias_dropout_residual(const float* acc, const float* const* partials, in
   }
   if (!aligned16(acc) || !aligned16(bias) || !aligned16(out) || (resid && !aligned16(resid))) return CCN_EINVAL;
   EpiPrm ep;
-  int rc = make_epi(p_drop, seed, &ep);
+  int rc = make_epi(p_drop, seed, mode, &ep);
   if (rc != CCN_OK) return rc;
   const DeviceInfo* di = nullptr;
   rc = current_device_info(&di);
@@ -310,20 +362,74 @@ int ccn_bias_dropout_residual(const float* acc, const float* const* partials, in
   const size_t gx = wgs < 0x40000000ull ? wgs : 0x40000000ull;
   const dim3 grid((unsigned)gx, (unsigned)((wgs + gx - 1) / gx));
   hipStream_t s = as_stream(stream);
+  const size_t mask_base = first_row * (size_t)N;
   auto go = [&](auto qtag) {
     constexpr int Q = decltype(qtag)::value;
-    if (sh.block == kWave)
-      hipLaunchKernelGGL((bias_dropout_residual_kernel<Q, kWave>), grid, dim3(kWave), sh.lds_bytes, s, acc, tbl, bias, resid, out,
-                         total, (size_t)N, ep);
-    else
-      hipLaunchKernelGGL((bias_dropout_residual_kernel<Q, kBlock>), grid, dim3(kBlock), sh.lds_bytes, s, acc, tbl, bias, resid,
-                         out, total, (size_t)N, ep);
+    auto launch = [&](auto bstag, auto reftag) {
+      constexpr int BS = decltype(bstag)::value;
+      hipLaunchKernelGGL((bias_dropout_residual_kernel<Q, BS, decltype(reftag)::value>), grid, dim3(BS), sh.lds_bytes, s, acc, tbl, bias,
+                         resid, out, total, (size_t)N, mask_base, ep);
+    };
+    const bool ref = mode != CCN_DROPOUT_INVERTED;
+    if (sh.block == kWave) {
+      if (ref) launch(std::integral_constant<int, kWave>{}, std::true_type{});
+      else launch(std::integral_constant<int, kWave>{}, std::false_type{});
+    } else {
+      if (ref) launch(std::integral_constant<int, kBlock>{}, std::true_type{});
+      else launch(std::integral_constant<int, kBlock>{}, std::false_type{});
+    }
   };
   switch (nPartials) {
 #define CCN_CASE(Q) case Q: go(std::integral_constant<int, Q>{}); break;
     CCN_CASE(0) CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
 #undef CCN_CASE
   }
+  CCN_HIP(hipGetLastError());
+  return CCN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                         const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
+                         uint64_t seed, void* stream) {
+  return outproj_launch(X, W, partials, nPartials, bias, resid, out, M, N, K, p_drop, seed, CCN_DROPOUT_INVERTED, stream);
+}
+
+int ccn_mlp_outproj_bf16_ex(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                            const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
+                            uint64_t seed, int dropout_mode, void* stream) {
+  return outproj_launch(X, W, partials, nPartials, bias, resid, out, M, N, K, p_drop, seed, dropout_mode, stream);
+}
+
+int ccn_bias_dropout_residual(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                              const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                              void* stream) {
+  return epilogue_launch(acc, partials, nPartials, bias, resid, out, M, N, p_drop, seed, CCN_DROPOUT_INVERTED, 0, stream);
+}
+
+int ccn_bias_dropout_residual_ex(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                                 const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                                 int dropout_mode, size_t first_row, void* stream) {
+  return epilogue_launch(acc, partials, nPartials, bias, resid, out, M, N, p_drop, seed, dropout_mode, first_row, stream);
+}
+
+int ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
+  if (!X || !W || !C) return CCN_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0) return CCN_EINVAL;
+  if (M % BM || N % BN || K % BK) return CCN_ERANGE;   // whole tiles only
+  if (!aligned16(X) || !aligned16(W) || !aligned16(C)) return CCN_EINVAL;
+  const DeviceInfo* di = nullptr;
+  const int rc = current_device_info(&di);
+  if (rc != CCN_OK) return rc;
+  SrcTable<float, 8> tbl;
+  for (int q = 0; q < 8; q++) tbl.p[q] = nullptr;
+  EpiPrm ep{};
+  const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
+  hipLaunchKernelGGL((mlp_outproj_kernel<0, true>), grid, block, 0, as_stream(stream), X, W, tbl, (const float*)nullptr,
+                     (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), N, K, ep);
   CCN_HIP(hipGetLastError());
   return CCN_OK;
 }

@@ -221,6 +221,35 @@ int  ccn_bias_dropout_residual(const float* acc, const float* const* partials, i
                                const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
                                void* stream);
 
+/* ---- the same two calls with the dropout semantics as an argument.  With s = X.W + sum_q partials[q] (or acc + ...),
+ *      b = bias[col], r = resid and u the element's uniform draw (the Philox stream above: the reference draws from
+ *      cuRAND, whose stream is not reproducible here):
+ *        CCN_DROPOUT_INVERTED      out = (u >= p ? (s + b)/(1-p) : 0) + r      what the two calls above compute; p in [0,1)
+ *        CCN_DROPOUT_REF_DSL       out = (u <  p ? (s + b) : 0) + r            the reference's emitted expression for
+ *                                  Dropout(sum + b, p) + r: keeps with probability p, no rescale (src/codegen.cpp:634-640)
+ *        CCN_DROPOUT_REF_NCCL      out = ((u < p ? s : 0) + b) + r             the reference's fused kernel, FuncDropout<T>
+ *                                  (nccl-overlap/src/collectives/device/reduce_kernel.h:192-197, common_kernel.h:1037-1057)
+ *        CCN_DROPOUT_REF_NCCL_SAT  out = sat(sat((u < p ? s : 0) + b) + r), sat = clamp to [0,1], as its half
+ *                                  specialisation adds with __hadd2_sat (reduce_kernel.h:199-213)
+ *      The reference's forms take p in [0,1]: p = 0 keeps nothing, p = 1 everything.
+ *      first_row (epilogue call): row of the whole output that row 0 of this call is, for calls that cover a band of
+ *      rows each (one rank's slice): the mask of an element depends on its index in the whole output only. ---- */
+#define CCN_DROPOUT_INVERTED     0
+#define CCN_DROPOUT_REF_DSL      1
+#define CCN_DROPOUT_REF_NCCL     2
+#define CCN_DROPOUT_REF_NCCL_SAT 3
+int  ccn_mlp_outproj_bf16_ex(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                             const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K,
+                             float p_drop, uint64_t seed, int dropout_mode, void* stream);
+int  ccn_bias_dropout_residual_ex(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                                  const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                                  int dropout_mode, size_t first_row, void* stream);
+
+/* ---- the product alone: C[MxN] (fp32, row-major) = X[MxK].W[KxN], bf16 operands, fp32 accumulation on the matrix
+ *      cores.  Replaces the emitted cublasGemmEx call of the unfused schedules (matMulK, src/codegen.cpp:1058-1136);
+ *      whole 128x128x64 tiles (CCN_ERANGE otherwise). ---- */
+int  ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -452,10 +452,35 @@ void orc_dropout_mask(uint64_t seed, uint64_t first_idx, size_t n, float p_drop,
  * Dropout here is the standard one (drop with probability p, survivors scaled by 1/(1-p)); the
  * reference keeps with probability p and does not rescale (src/codegen.cpp:634-640).
  * ---------------------------------------------------------------------------------------------- */
-void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
-                     const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
-                     int M, int N, int K, float p_drop, uint64_t seed) {
-  const float scale = 1.0f / (1.0f - p_drop);
+/* One output element from its sum s (product + partial products), bias b, residual r and keep decision
+ * `kept_inverted` (u >= p), under the four dropout forms:
+ *   0  standard ("inverted") dropout:                      (u >= p ? (s + b) * 1/(1-p) : 0) + r
+ *   1  the reference's emitted expression, src/codegen.cpp:634-640 with examples/model-parallel/model-parallel.cpp:20-21:
+ *      (curand_uniform < prob ? (sum + b) : 0) + r          keeps with probability p, no rescale
+ *   2  the reference's fused kernel, FuncDropout<T>, nccl-overlap/src/collectives/device/reduce_kernel.h:192-197:
+ *      (curand_uniform < p ? val : 0) + biasVal + addTensorVal
+ *   3  its half specialisation, :199-213: __hadd2_sat(__hadd2_sat(v, biasVal), addTensorVal), sat = clamp to [0, 1] */
+static float sat01(float x) { return x > 0.0f ? (x < 1.0f ? x : 1.0f) : 0.0f; }
+float orc_epilogue_value(float s, float b, float r, int kept_inverted, float p_drop, int mode) {
+  if (mode == 0) {
+    const float scale = 1.0f / (1.0f - p_drop);
+    const float t = s + b;
+    const float d = kept_inverted ? t * scale : 0.0f;
+    return d + r;
+  }
+  const int kept = !kept_inverted;   /* u < p */
+  if (mode == 1) {
+    const float t = s + b;
+    return (kept ? t : 0.0f) + r;
+  }
+  const float v = kept ? s : 0.0f;
+  if (mode == 2) return (v + b) + r;
+  return sat01(sat01(v + b) + r);
+}
+
+void orc_mlp_outproj_mode(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                          const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                          int M, int N, int K, float p_drop, uint64_t seed, int mode) {
   for (int i = 0; i < M; i++) {
     for (int j = 0; j < N; j++) {
       double acc = 0.0;
@@ -464,11 +489,16 @@ void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* p
       float s = (float)acc;
       size_t idx = (size_t)i * N + j;
       for (int q = 0; q < nPartials; q++) s = s + partials[q][idx];
-      float t = s + bias[j];
-      float d = orc_dropout_keep(seed, idx, p_drop) ? t * scale : 0.0f;
-      float y = d + (resid ? orc_bf16_to_f32(resid[idx]) : 0.0f);
+      const int kept_inverted = orc_dropout_keep(seed, idx, p_drop);   /* u >= p; p = 0: always */
+      float y = orc_epilogue_value(s, bias[j], resid ? orc_bf16_to_f32(resid[idx]) : 0.0f, kept_inverted, p_drop, mode);
       if (out_f32) out_f32[idx] = y;
       if (out) out[idx] = orc_f32_to_bf16(y);
     }
   }
+}
+
+void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                     const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                     int M, int N, int K, float p_drop, uint64_t seed) {
+  orc_mlp_outproj_mode(X, W, partials, nPartials, bias, resid, out, out_f32, M, N, K, p_drop, seed, 0);
 }

@@ -106,6 +106,11 @@ void orc_dropout_mask(uint64_t seed, uint64_t first_idx, size_t n, float p_drop,
  *      s = acc + partial[0] + ... + partial[nPartials-1]  (fp32, ascending);
  *      t = s + bias[col]; d = keep ? t * (1/(1-p)) : 0;  y = d + resid;  out = bf16(y)
  *      out_f32 (optional) receives y before the bf16 rounding. ---- */
+/* one element of the epilogue under dropout form `mode` (0 standard, 1-3 the reference's; see ccn_oracle.c) */
+float orc_epilogue_value(float s, float b, float r, int kept_inverted, float p_drop, int mode);
+void orc_mlp_outproj_mode(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                          const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                          int M, int N, int K, float p_drop, uint64_t seed, int mode);
 void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
                      const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
                      int M, int N, int K, float p_drop, uint64_t seed);

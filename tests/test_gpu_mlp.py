@@ -172,3 +172,91 @@ def test_seeded_random_shapes(ccn, case):
     assert np.array_equal(got[~keep], (resid if with_resid else zero)[~keep])
     d = bf16_ulp_distance(got, want)
     assert d.max() <= 1 and (d > 0).mean() < 0.02, f"case {case}: M={M} N={N} K={K} nP={nP} p={p}: {d.max()} {(d > 0).mean():.4f}"
+
+
+# ---- the reference's dropout forms and the unfused pieces ---------------------------------------------------------------
+@pytest.mark.parametrize("mode", [1, 2, 3])
+@pytest.mark.parametrize("p", [0.0, 0.1, 1.0])
+def test_reference_dropout_forms(ccn, mode, p):
+    """Keep with probability p and no rescale (src/codegen.cpp:634-640), the fused kernel's placement of bias and
+    residual and its saturating adds (nccl-overlap/.../reduce_kernel.h:192-213): the standalone epilogue bit for bit
+    against the oracle, the fused GEMM within its one-ulp bar.  p = 0 keeps nothing, p = 1 everything."""
+    M, N, K, nP = 128, 256, 128, 3
+    X, W, parts, bias, resid = make_case(70 + mode, M, N, K, nP)
+    if mode == 3:       # values inside and around [0, 1] so that both clamps are exercised
+        parts = [q * np.float32(0.2) for q in parts]
+        bias = bias * np.float32(0.3)
+    pd = [torch.from_numpy(q).to(DEV) for q in parts]
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(bf16_dev(X), bf16_dev(W), pd, torch.from_numpy(bias).to(DEV), bf16_dev(resid), out, M, N, K, p, 9,
+                         dropout_mode=mode)
+    got = bf16_host(out).reshape(M, N)
+    want, want_f32 = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, p, 9, mode=mode)
+    d = bf16_ulp_distance(got, want)
+    assert d.max() <= 1 and (d > 0).mean() < 0.02
+    if mode == 1 and p == 0.0:
+        assert np.array_equal(got, resid)                   # nothing kept: the residual alone
+    # standalone epilogue on the exact product: bit for bit
+    acc = (orc.bf16_to_f32(X).astype(np.float64) @ orc.bf16_to_f32(W).astype(np.float64)).astype(np.float32)
+    out2 = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.bias_dropout_residual(torch.from_numpy(acc).to(DEV), pd, torch.from_numpy(bias).to(DEV), bf16_dev(resid), out2, M, N, p, 9,
+                              dropout_mode=mode)
+    assert np.array_equal(bf16_host(out2).reshape(M, N), want)
+    if mode == 3:
+        f = orc.bf16_to_f32(want)
+        assert f.min() >= 0.0 and f.max() <= 1.0 and (f == 0).any() and (f == 1).any()
+
+
+def test_reference_dropout_forms_reject_bad_probabilities(ccn):
+    M = N = 128
+    K = 64
+    z16 = torch.zeros(M * N, dtype=torch.int16, device=DEV)
+    zf = torch.zeros(N, device=DEV)
+    for mode, p, ok in [(0, 1.0, False), (1, 1.0, True), (1, 1.5, False), (2, -0.1, False), (4, 0.1, False)]:
+        call = lambda: ccn.mlp_outproj_bf16(z16, z16, [], zf, None, z16, M, N, K, p, 0, dropout_mode=mode)
+        if ok:
+            call()
+        else:
+            with pytest.raises(ccn.CoconetError) as e:
+                call()
+            assert e.value.code == ccn.CCN_EINVAL
+
+
+def test_epilogue_in_row_bands_draws_the_same_mask(ccn):
+    """One rank's slice of the output (a band of rows) through ccn_bias_dropout_residual_ex with first_row: the union of
+    the bands is the whole-call result, mask included."""
+    M, N, nP, p = 96, 64, 2, 0.4
+    r = rng(77)
+    acc = r.standard_normal((M, N), dtype=np.float32)
+    parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N, dtype=np.float32)
+    resid = orc.f32_to_bf16(r.standard_normal((M, N), dtype=np.float32))
+    accd, pd, bd, rd = torch.from_numpy(acc).to(DEV), [torch.from_numpy(q).to(DEV) for q in parts], torch.from_numpy(bias).to(DEV), bf16_dev(resid)
+    whole = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.bias_dropout_residual(accd, pd, bd, rd, whole, M, N, p, 5)
+    banded = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    for r0 in range(0, M, 32):
+        ccn.bias_dropout_residual(accd[r0:r0 + 32], [q[r0:r0 + 32] for q in pd], bd, rd[r0:r0 + 32], banded[r0:r0 + 32], 32, N, p, 5,
+                                  dropout_mode=0, first_row=r0)
+    assert torch.equal(whole, banded)
+
+
+def test_plain_product(ccn):
+    """ccn_matmul_bf16_f32, the unfused schedule's GEMM: exact on small integers (all-ones gives K, the reference's own
+    check at this boundary), fp32-accumulation close to float64 on random operands."""
+    M, N, K = 256, 384, 192
+    ones = lambda shape: orc.f32_to_bf16(np.ones(shape, np.float32))
+    Cd = torch.zeros(M, N, device=DEV)
+    ccn.matmul_bf16_f32(bf16_dev(ones((M, K))), bf16_dev(ones((K, N))), Cd, M, N, K)
+    torch.cuda.synchronize()
+    assert torch.all(Cd == K)
+    X, W, _, _, _ = make_case(81, M, N, K, 0)
+    ccn.matmul_bf16_f32(bf16_dev(X), bf16_dev(W), Cd, M, N, K)
+    torch.cuda.synchronize()
+    xf, wf = orc.bf16_to_f32(X).astype(np.float64), orc.bf16_to_f32(W).astype(np.float64)
+    ref = xf @ wf
+    bound = K * 2.0 ** -24 * (np.abs(xf) @ np.abs(wf))           # fp32 accumulation of K exact products
+    assert np.all(np.abs(Cd.cpu().numpy().astype(np.float64) - ref) <= bound + 1e-30)
+    with pytest.raises(ccn.CoconetError) as e:
+        ccn.matmul_bf16_f32(bf16_dev(X), bf16_dev(W), Cd, M, N, K - 1)
+    assert e.value.code == ccn.CCN_ERANGE

@@ -550,3 +550,54 @@ def test_lamb_nccl_f16g_half_chain_against_numpy_float16():
     scale = (np.sqrt(np.sum(w0.astype(np.float64) ** 2)) / np.sqrt(np.sum(r ** 2))) / np.sqrt(np.sum(r ** 2))
     assert np.max(np.abs(w - (w0 - 0.01 * scale * r))) <= 1e-6 * np.max(np.abs(w0))
     assert np.array_equal(hw, w.astype(np.float16).view(np.uint16))
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the reference's dropout forms (keep with probability p, no rescale): pinned by what the arithmetic fixes
+# ---------------------------------------------------------------------------------------------------------------------
+def test_reference_dropout_forms_closed_forms():
+    """src/codegen.cpp:634-640 emits (curand_uniform < p ? x : 0): p = 0 keeps nothing, p = 1 everything, and nothing
+    is rescaled.  FuncDropout (nccl-overlap/.../reduce_kernel.h:192-213) drops the sum only, then adds bias and
+    residual, with saturation to [0, 1] in its half form."""
+    r = rng(61)
+    M, N, K, nP = 4, 8, 16, 3
+    X = orc.f32_to_bf16(r.standard_normal((M, K), dtype=np.float32))
+    W = orc.f32_to_bf16(r.standard_normal((K, N), dtype=np.float32) * np.float32(0.1))
+    parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N, dtype=np.float32)
+    resid = orc.f32_to_bf16(r.standard_normal((M, N), dtype=np.float32))
+    rf = orc.bf16_to_f32(resid)
+    s = (orc.bf16_to_f32(X).astype(np.float64) @ orc.bf16_to_f32(W).astype(np.float64)).astype(np.float32)
+    for q in parts:
+        s = s + q
+    # p = 0: nothing survives.  DSL form: the residual alone; fused-kernel form: bias + residual
+    _, y = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, 0.0, 3, mode=1)
+    assert np.array_equal(y, rf)
+    _, y = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, 0.0, 3, mode=2)
+    assert np.array_equal(y, (np.float32(0) + bias[None, :]) + rf)
+    # p = 1: everything survives, unscaled
+    _, y = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, 1.0, 3, mode=1)
+    assert np.array_equal(y, (s + bias[None, :]) + rf)
+    _, y = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, 1.0, 3, mode=2)
+    assert np.array_equal(y, (s + bias[None, :]) + rf)
+    # in between: the survivors of "keep with probability p" are exactly the elements "drop with probability p" drops
+    p = 0.3
+    dropped_by_standard = ~orc.dropout_mask(3, 0, M * N, p).reshape(M, N).astype(bool)
+    _, y = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, p, 3, mode=1)
+    assert np.array_equal(y, np.where(dropped_by_standard, s + bias[None, :], np.float32(0)) + rf)
+    _, y0 = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, p, 3, mode=0)
+    scale = np.float32(1) / (np.float32(1) - np.float32(p))
+    assert np.array_equal(y0, np.where(dropped_by_standard, np.float32(0), (s + bias[None, :]) * scale) + rf)
+    assert 0 < dropped_by_standard.sum() < M * N
+
+
+def test_reference_saturating_dropout_form():
+    """__hadd2_sat clamps every sum to [0, 1]: all-ones inputs give 1 (not 3), a negative kept sum gives
+    sat(sat(s + b) + r) with the inner clamp at 0 applied before the residual is added."""
+    one = np.float32(1.0)
+    assert orc.epilogue_value(one, one, one, 0, 0.5, 3) == 1.0          # kept: sat(sat(1 + 1) + 1)
+    assert orc.epilogue_value(one, one, one, 1, 0.5, 3) == 1.0          # dropped: sat(sat(0 + 1) + 1)
+    assert orc.epilogue_value(-2.0, 0.5, 0.25, 0, 0.5, 3) == 0.25       # sat(-1.5) = 0, then 0 + 0.25
+    assert orc.epilogue_value(-2.0, 0.5, 0.25, 0, 0.5, 2) == -1.25      # unsaturated: (-2 + 0.5) + 0.25
+    assert orc.epilogue_value(0.25, 0.25, 0.25, 0, 0.5, 3) == 0.75 and orc.epilogue_value(0.25, 0.25, -1.0, 0, 0.5, 3) == 0.0
+    assert orc.epilogue_value(float("nan"), 0.0, 0.0, 0, 0.5, 3) == 0.0  # NaN saturates to zero
