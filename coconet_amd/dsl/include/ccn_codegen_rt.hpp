@@ -133,6 +133,28 @@ __host__ __device__ inline float dropout(float x, float p_drop, uint64_t seed, u
   return dropout_keep(seed, idx, p_drop) ? x * (1.0f / (1.0f - p_drop)) : 0.0f;
 }
 
+// The reference's form of the same stage (src/codegen.cpp:634-640): keep with probability p, no rescale.
+__host__ __device__ inline float dropout_ref(float x, float p_keep, uint64_t seed, uint64_t idx) {
+  return !dropout_keep(seed, idx, p_keep) ? x : 0.0f;   // kept where u < p
+}
+// One output element of the MLP epilogue from the sum s over the ranks' products, bias b and residual r, under dropout
+// form `mode` (CCN_DROPOUT_* of coconet_hip.h); host mirror of the library's epilogue for the emitted self-check.
+inline float epilogue_value(float s, float b, float r, float p, uint64_t seed, uint64_t idx, int mode) {
+  auto sat = [](float x) { return x > 0.0f ? (x < 1.0f ? x : 1.0f) : 0.0f; };
+  if (mode == CCN_DROPOUT_INVERTED) {
+    const float t = s + b;
+    const float d = p > 0.0f ? dropout(t, p, seed, idx) : t;
+    return d + r;
+  }
+  const bool kept = !dropout_keep(seed, idx, p);
+  if (mode == CCN_DROPOUT_REF_DSL) {
+    const float t = s + b;
+    return (kept ? t : 0.0f) + r;
+  }
+  const float d = kept ? s : 0.0f;
+  return mode == CCN_DROPOUT_REF_NCCL_SAT ? sat(sat(d + b) + r) : (d + b) + r;
+}
+
 // ---- reductions ---------------------------------------------------------------------------------------------------
 __device__ __forceinline__ double wave_sum(double x) {
 #pragma unroll
@@ -471,6 +493,11 @@ inline size_t env_size(const char* name, size_t dflt) {
   char* end = nullptr;
   const unsigned long long x = strtoull(e, &end, 10);
   return end && *end == 0 ? (size_t)x : dflt;
+}
+// The sizes a dimension variable takes: the one value of the environment variable when it is set, else the defaults.
+inline std::vector<size_t> env_sizes(const char* name, std::vector<size_t> dflt) {
+  const size_t x = env_size(name, 0);
+  return x ? std::vector<size_t>{x} : dflt;
 }
 inline float env_float(const char* name, float dflt) {
   const char* e = getenv(name);

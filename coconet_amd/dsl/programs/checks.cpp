@@ -143,6 +143,48 @@ int main(int argc, char** argv) {
     std::cout << generateHIP(pl, {});
     return 0;
   }
+  if (c.rfind("mlp_", 0) == 0) {
+    // MatMul pipelines are matched against MatMul -> AllReduce|ReduceScatter -> [+bias] -> [Dropout] -> [+residual] -> [AllGather]
+    Variable B(Int32, "B"), S(Int32, "S"), H(Int32, "H");
+    Tensor w(Float16, {H, H}, Sliced, "w");
+    Tensor b(Float16, H, Replicated, "b");
+    Tensor b2(Float16, S, Replicated, "b2");
+    Tensor in(Float16, {B, S, H}, Sliced_2, "in");
+    Tensor r(Float16, {B, S, H}, Replicated, "r");
+    Stage layer = MatMul(in, w);
+    Stage sum = AllReduce(Summation, layer);
+    std::vector<CodeGenVarBounds> bounds = {CodeGenVarBounds(B, {8}), CodeGenVarBounds(S, {1024}), CodeGenVarBounds(H, {3072})};
+    if (c == "mlp_scaled_sum") {            // a product where the chain has a sum
+      Stage out = Dropout(sum * b, 0.5) + r;
+      Pipeline pl("bad", {w, b, in, r}, {out});
+      std::cout << generateHIP(pl, bounds);
+    } else if (c == "mlp_two_dropouts") {
+      Stage out = Dropout(Dropout(sum + b, 0.5), 0.5) + r;
+      Pipeline pl("bad", {w, b, in, r}, {out});
+      std::cout << generateHIP(pl, bounds);
+    } else if (c == "mlp_residual_before_dropout") {
+      Stage out = Dropout((sum + b) + r, 0.5);
+      Pipeline pl("bad", {w, b, in, r}, {out});
+      std::cout << generateHIP(pl, bounds);
+    } else if (c == "mlp_no_collective") {
+      Stage out = Dropout(layer, 0.5) + r;
+      Pipeline pl("bad", {w, b, in, r}, {out});
+      std::cout << generateHIP(pl, bounds);
+    } else if (c == "mlp_operands_swapped") {   // b + sum, r + Dropout(.): the same chain
+      Stage out = r + Dropout(b + sum, 0.5);
+      Pipeline pl("ok", {w, b, in, r}, {out});
+      std::cout << generateHIP(pl, bounds);
+    } else if (c == "mlp_no_bias_no_dropout") {
+      Stage out = sum + r;
+      Pipeline pl("ok", {w, b, in, r}, {out});
+      pl.fuse({sum, out});
+      std::cout << generateHIP(pl, bounds);
+    } else {
+      std::cout << "unknown case" << std::endl;
+      return 64;
+    }
+    return 0;
+  }
   if (c == "bad_file") {
     AdamParts a;
     Pipeline pl("adam", {a.g, a.w, a.m, a.v, a.lr, a.beta1, a.beta2}, {a.m1, a.v1, a.w1});

@@ -1,6 +1,7 @@
 // DSL programs for the benchmark configurations, written against the CoCoNet API.
 //   ccn-programs <program> <schedule> [output.hip]
-// program: sgd | biasadd | clipsgd | reduction | adam | adamf16 | lamb     schedule: unfused | fused (adamf16: fused only)
+// program: sgd | biasadd | clipsgd | reduction | adam | adamf16 | lamb | mlp | mlpepi
+// schedule: unfused | fused (adamf16, mlpepi: fused only)
 #include <dsl.hpp>
 #include <pipeline.hpp>
 
@@ -130,9 +131,28 @@ static void lamb(bool fused, const std::string& out) {
   pl.codegen(out);
 }
 
+// The model-parallel MLP out-projection at benchmark configuration 5's shape: with 8 ranks, one rank's K-slice is
+// X [8192 x 1024] . W [1024 x 8192], the other 7 ranks' partial products are resident, then bias, dropout(0.1), residual.
+//   unfused: MatMul, AllReduce and the pointwise part as separate steps      fused: one kernel
+static void mlp(bool fused, bool epilogueOnly, const std::string& out) {
+  Variable B(Int32, "B"), S(Int32, "S"), H(Int32, "H");
+  Tensor w(Float16, {H, H}, Sliced, "w");
+  Tensor b(Float16, H, Replicated, "b");
+  Tensor in(Float16, {B, S, H}, Sliced_2, "in");
+  Tensor r(Float16, {B, S, H}, Replicated, "r");
+  Stage layer = MatMul(in, w);
+  Stage sum = AllReduce(Summation, layer);
+  Stage sum2 = sum + b;
+  Stage res = Dropout(sum2, 0.1) + r;
+  Pipeline pl("mlp", {w, b, in, r}, {res});
+  if (epilogueOnly) pl.fuse({sum, sum2, res});          // the sum over ranks joins the pointwise part; the GEMM stays alone
+  else if (fused) pl.fuse({layer, sum, sum2, res});
+  pl.codegen(out, {CodeGenVarBounds(B, {8}), CodeGenVarBounds(S, {1024}), CodeGenVarBounds(H, {8192})});
+}
+
 int main(int argc, char** argv) {
   if (argc < 3) {
-    std::cout << "usage: " << argv[0] << " <sgd|biasadd|clipsgd|reduction|adam|adamf16|lamb> <unfused|fused> [output.hip]" << std::endl;
+    std::cout << "usage: " << argv[0] << " <sgd|biasadd|clipsgd|reduction|adam|adamf16|lamb|mlp|mlpepi> <unfused|fused> [output.hip]" << std::endl;
     return 1;
   }
   const std::string prog = argv[1], sched = argv[2];
@@ -146,6 +166,8 @@ int main(int argc, char** argv) {
   else if (prog == "adam") adam(fused, out);
   else if (prog == "adamf16") adamf16(fused, out);
   else if (prog == "lamb") lamb(fused, out);
+  else if (prog == "mlp") mlp(fused, false, out);
+  else if (prog == "mlpepi") mlp(fused, true, out);
   else { std::cout << "Invalid program" << std::endl; return 1; }
   return 0;
 }

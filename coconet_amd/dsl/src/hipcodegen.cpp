@@ -20,6 +20,7 @@
 // + main() with the reference's size sweep and "{SZ: ..., Epochs: ..., <step>: ms, Total: ms}" line
 // (src/codegen.cpp:4583-4784).
 #include <algorithm>
+#include <cstdlib>
 #include <functional>
 #include <map>
 #include <set>
@@ -44,6 +45,14 @@ std::string fconst(const NodePtr& n) {
     return s + "f";
   }
   return o.str();
+}
+
+// Dropout(x, p) is lowered to standard dropout (drop with probability p, survivors scaled by 1/(1-p)) unless the
+// generator runs with CCN_DSL_DROPOUT=reference: then to the reference's emitted form, keep with probability p and no
+// rescale (src/codegen.cpp:634-640).  The mask comes from the counter-based stream either way.
+bool reference_dropout() {
+  const char* e = std::getenv("CCN_DSL_DROPOUT");
+  return e && std::string(e) == "reference";
 }
 
 // ---- program-level facts ---------------------------------------------------------------------------------------------
@@ -198,7 +207,8 @@ struct BodyBuilder {
         body.usesSeed = true;
         std::ostringstream o;
         o.precision(9);
-        o << "ccn_gen::dropout(" << emit(n->args[0]) << ", " << n->prob << "f, s.seed__, idx)";
+        o << (reference_dropout() ? "ccn_gen::dropout_ref(" : "ccn_gen::dropout(") << emit(n->args[0]) << ", " << n->prob
+          << "f, s.seed__, idx)";
         return o.str();
       }
       case Kind::Collective: {
@@ -654,7 +664,8 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
         case Kind::Dropout: {
           std::ostringstream q;
           q.precision(9);
-          q << "ccn_gen::dropout(" << he(n->args[0]) << ", " << n->prob << "f, seed__, (uint64_t)i0)";
+          q << (reference_dropout() ? "ccn_gen::dropout_ref(" : "ccn_gen::dropout(") << he(n->args[0]) << ", " << n->prob
+            << "f, seed__, (uint64_t)i0)";
           return q.str();
         }
         case Kind::Collective:

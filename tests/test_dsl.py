@@ -54,6 +54,12 @@ def test_storage_classes_and_fusion_groups(dsl_build):
     ("dims_mismatch_same_rank", "do not match"),
     ("dims_mismatch_in_select", "do not match"),
     ("update_with_more_dims", "more dimensions"),
+    # a MatMul pipeline that is not MatMul -> AllReduce|ReduceScatter -> [+bias] -> [Dropout] -> [+residual] -> [AllGather]
+    # is refused, not lowered to the nearest thing the library has
+    ("mlp_scaled_sum", "must have the shape"),
+    ("mlp_two_dropouts", "must have the shape"),
+    ("mlp_residual_before_dropout", "must have the shape"),
+    ("mlp_no_collective", "must have the shape"),
 ])
 def test_invalid_programs_abort_with_a_message(dsl_build, case, needle):
     """Error convention of the reference (src/ast.hpp:33-44): message on stderr, then std::terminate()."""
@@ -74,6 +80,38 @@ def test_trailing_dimensions_broadcast(dsl_build):
     assert "args0.s.bc_b = b;" in text and "args0.s.bcn_b = (size_t)H;" in text and "args0.s.bcn_sh = (size_t)S * H;" in text
     assert "h.b[i0 % h.b.size()]" in text and "h.sh[i0 % h.sh.size()]" in text and "h.x[i0]" in text
     assert "NIN = 1" in text            # x alone is streamed; g comes through the rank fold
+
+
+def test_matmul_chain_is_matched_by_structure_and_lowered_by_schedule(dsl_build, tmp_path):
+    """The chain may be written with its sums' operands in either order and without bias and dropout; what is emitted
+    follows the schedule: separate steps when nothing is fused (the reference emits a cuBLAS call, an all-reduce and
+    pointwise kernels, src/codegen.cpp:1058-1136, 4146-4189), one epilogue call when the collective is fused with what
+    follows it, one kernel when the MatMul is."""
+    chk = os.path.join(dsl_build, "ccn-dsl-check")
+    swapped = run(chk, "mlp_operands_swapped")
+    assert swapped.returncode == 0, swapped.stderr
+    assert "ccn_matmul_bf16_f32(X, W, C" in swapped.stdout and "ccn_reduce_f32(tbl__, comm_size, C + off__" in swapped.stdout
+    assert "ccn_bias_dropout_residual_ex(C + off__, nullptr, 0, bias, R + off__, out + off__" in swapped.stdout
+    assert "const float p_drop = (float)0.5" in swapped.stdout
+    plain = run(chk, "mlp_no_bias_no_dropout")
+    assert plain.returncode == 0, plain.stderr
+    assert "ccn_bias_dropout_residual_ex(C + off__, tbl__, nPartials" in plain.stdout and "ccn_reduce_f32" not in plain.stdout
+    assert "hB[i] = 0.0f" in plain.stdout and "CCN_DROPOUT_INVERTED ? 0.0f : 1.0f" in plain.stdout
+    prog = os.path.join(dsl_build, "ccn-programs")
+    texts = {}
+    for name, sched in (("mlp", "unfused"), ("mlp", "fused"), ("mlpepi", "fused")):
+        out = tmp_path / f"{name}-{sched}.hip"
+        assert run(prog, name, sched, str(out)).returncode == 0
+        texts[(name, sched)] = out.read_text()
+    assert "ccn_mlp_outproj_bf16_ex(" in texts[("mlp", "fused")] and "ccn_matmul_bf16_f32" not in texts[("mlp", "fused")]
+    assert "MatMul: %f, AllReduce: %f, kernel0: %f, Total" in texts[("mlp", "unfused")]
+    assert "MatMul: %f, kernel0: %f, Total" in texts[("mlpepi", "fused")]
+    # the reference's dropout form on request, at generation time
+    env = dict(os.environ, CCN_DSL_DROPOUT="reference")
+    out = tmp_path / "ref.hip"
+    assert subprocess.run([prog, "mlp", "fused", str(out)], env=env).returncode == 0
+    assert 'env_size("CCN_GEN_DROPOUT_MODE", CCN_DROPOUT_REF_DSL)' in out.read_text()
+    assert 'env_size("CCN_GEN_DROPOUT_MODE", CCN_DROPOUT_INVERTED)' in texts[("mlp", "fused")]
 
 
 def test_unwritable_output_reports_and_returns(dsl_build):
@@ -207,8 +245,14 @@ def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path)
     assert "args0.in[0] = m + off__" in unf and "args0.n = cnt__" in unf and "int comm_size, int rank" in unf
     arc = (tmp_path / "adam-ar-c.hip").read_text()
     assert "off__" not in arc and "ccn_reduce_f32(g, comm_size, g[0], (size_t)N" in arc     # Replicated: the whole range
+    # the model-parallel example: unfused schedules as separate steps, the overlapped one as the one fused kernel
     mlp = (tmp_path / "model-parallel-mm-ar-c.hip").read_text()
-    assert "ccn_mlp_outproj_bf16" in mlp and "p_drop = (float)0.5;" in mlp
+    assert "ccn_matmul_bf16_f32" in mlp and "ccn_bias_dropout_residual_ex" in mlp and "p_drop = (float)0.5" in mlp
+    assert "ccn_mlp_outproj_bf16" not in mlp and "MatMul: %f, AllReduce: %f, kernel0: %f, Total" in mlp
+    rs = (tmp_path / "model-parallel-mm-rs-c-ag.hip").read_text()
+    assert "MatMul: %f, ReduceScatter: %f, kernel0: %f, AllGather: %f, Total" in rs and "ccn_memcpy_d2d(out + off__, scOut + off__" in rs
+    ol = (tmp_path / "model-parallel-ol-mm-fuse-rs-c-ag.hip").read_text()
+    assert "ccn_mlp_outproj_bf16_ex" in ol and "MatMulFused: %f" in ol
 
 
 @pytest.mark.skipif(not os.path.exists(os.path.join(ROOT, "oracle", "_ref", "ref-adam")), reason="oracle/_ref not built")

@@ -164,15 +164,40 @@ def test_the_emitted_check_catches_a_wrong_result():
         assert ok.returncode == 0 and "do not match" not in ok.stdout
 
 
-@pytest.mark.parametrize("name", ["ref-model-parallel-mm-ar-c", "ref-model-parallel-mm-rs-c-ag",
-                                  "ref-model-parallel-ol-mm-fuse-rs-c-ag"])
+MLP_STEPS = {"ref-model-parallel-mm-ar-c": {"MatMul", "AllReduce", "kernel0"},
+             "ref-model-parallel-mm-rs-c-ag": {"MatMul", "ReduceScatter", "kernel0", "AllGather"},
+             "ref-model-parallel-ol-mm-fuse-rs-c-ag": {"MatMulFused"}}
+
+
+@pytest.mark.parametrize("name", list(MLP_STEPS))
 def test_model_parallel_programs(name):
     """Every schedule of the reference's examples/model-parallel/model-parallel.cpp (the last one has no bias and no
-    dropout in its expression): each emitted program checks its GEMM + epilogue against its own CPU re-execution."""
+    dropout in its expression): the unfused ones run the product, the sum over ranks and the pointwise part as separate
+    steps (rank by rank on bands of rows after the ReduceScatter), the overlapped one as the one fused kernel; each
+    emitted program checks its result against its own CPU re-execution."""
     rows = run_program(name, 2, 8, 1)
     # B in {8, 16}, S = 1024, H = 3072: M = B*S rows, N = 3072
     assert [r[0] for r in rows] == [8 * 1024 * 3072, 16 * 1024 * 3072]
-    assert all("MatMulFused" in r[2] for r in rows)
+    assert all(set(r[2]) - {"Total"} == MLP_STEPS[name] for r in rows)
+
+
+@pytest.mark.parametrize("name", ["mlp-unfused", "mlpepi-fused", "mlp-fused", "ref-model-parallel-mm-rs-c-ag"])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_mlp_programs_under_every_dropout_form(name, mode):
+    """Small shapes (one rank's K-slice 256 x 128 . 128 x 1024 on 8 ranks), every schedule, every dropout form of the
+    library (CCN_DROPOUT_*): the emitted self-check mirrors the form on the host."""
+    rows = run_program(name, 1, 8, 1, env={"CCN_GEN_B": 1, "CCN_GEN_S": 256, "CCN_GEN_H": 1024, "CCN_GEN_DROPOUT_MODE": mode})
+    assert [r[0] for r in rows] == [256 * 1024]
+
+
+def test_fusing_the_epilogue_into_the_gemm_pays_off_at_config5_size():
+    """Benchmark configuration 5 from the DSL (8 ranks, B*S = 8192 rows, H = 8192: one rank's K-slice is 1024 deep) in
+    three schedules: the fused kernel writes the product nowhere, the unfused ones write it to memory as fp32 and read
+    it back (once more when the sum over ranks is a step of its own)."""
+    t = {}
+    for name in ("mlp-fused", "mlpepi-fused", "mlp-unfused"):
+        t[name] = run_program(name, 5, 8, 0, 2)[0][2]["Total"]
+    assert t["mlp-fused"] < 0.9 * t["mlpepi-fused"] and t["mlpepi-fused"] < t["mlp-unfused"], t
 
 
 def test_fusion_pays_off_at_config2_size():
