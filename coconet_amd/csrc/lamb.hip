@@ -240,12 +240,26 @@ __global__ __launch_bounds__(kBlock) void lamb_pass1_f16g_kernel(const SrcTable<
 // ---- communication between workgroups of one launch ---------------------------------------------------------------------
 // Device-scope release/acquire fences write back and invalidate the XCD's whole L2; with one per tile they serialise
 // the kernel (measured: 7 to 40 ms for a 2.8 ms step).  The few words that workgroups exchange therefore go through
-// relaxed device-scope atomics only, which are performed at the point where the XCDs' L2s are coherent and cost no
-// cache maintenance, and the order "data, then the word that announces it" is kept by waiting for the data's
-// acknowledgement (vmcnt = 0) before the announcing atomic is issued.
-__device__ __forceinline__ double peek_f64(const double* p) {
-  return __longlong_as_double((long long)__hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
-                                                           __HIP_MEMORY_SCOPE_AGENT));
+// relaxed device-scope atomics only.  On gfx942/gfx950 those carry the sc1 cache policy: stores are written through to
+// where the XCDs are coherent, loads and read-modify-writes are performed there, none of them is served from an XCD's
+// own L2, so a single word written this way is seen by every later device-scope atomic load of it, from any XCD, without
+// cache maintenance.  What relaxed atomics do not give is order BETWEEN words, and the protocol is built not to need it:
+//   tile sums      every slot is set to a sentinel by the kernel that precedes the launch; a tile replaces it with its
+//                  sum (one 64-bit atomic store per sum); whoever adds a segment's sums up re-reads a slot that still
+//                  holds the sentinel, a bounded number of times, and gives the segment up if it stays: a sum that is
+//                  not there yet is waited for or left to the trailing kernel, never read as something else;
+//   arrival counts only elect the workgroup that adds a segment up (a read-modify-write: exactly one sees the last count);
+//   scale + ready  travel in ONE 64-bit word, zero until set;
+//   everything else crosses a kernel boundary (the deferred list, the stored m and v, the norms for the host).
+// The tile still waits for its stores' acknowledgement (vmcnt = 0) before it counts itself in, so that the elected
+// workgroup normally finds every sum in place; that wait is a courtesy to the reader, not what correctness rests on.
+constexpr unsigned long long kNoSumYet = ~0ull;   // a NaN pattern no arithmetic produces; real sums are canonicalised away from it
+__device__ __forceinline__ unsigned long long sum_bits(double x) {
+  const unsigned long long b = (unsigned long long)__double_as_longlong(x);
+  return b == kNoSumYet ? 0x7ff8000000000000ull : b;
+}
+__device__ __forceinline__ unsigned long long peek_u64(const double* p) {
+  return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // All vector-memory operations this wavefront has issued are acknowledged before anything after this is issued.
 __device__ __forceinline__ void drain_vector_memory() {
@@ -278,16 +292,28 @@ __device__ __forceinline__ double group_sum(double x, double* lds) {
 
 // Norms and scale of segment b from its tiles' partial sums [lo, hi).  Thread t adds tiles lo+t, lo+t+BS, ... in
 // ascending order, then the fixed shuffle/LDS tree: the result does not depend on scheduling.
-// SHARED: the partial sums were published by other workgroups of this launch.
+// SHARED: the partial sums are published by other workgroups of this launch: a slot that still holds the sentinel is
+// read again up to `patience` times; if one stays empty, nothing is written and *complete is false (thread 0).
 // Returns the scale (valid in thread 0).
 template <int BS, bool SHARED>
 __device__ __forceinline__ float lamb_finalize_segment(const double* partials, uint32_t lo, uint32_t hi, uint64_t seg_len,
-                                                      int b, double* norms, float* scale, int mode, double* lds) {
+                                                      int b, double* norms, float* scale, int mode, double* lds,
+                                                      uint32_t patience = 0, bool* complete = nullptr) {
   double aW = 0.0, aR = 0.0;
+  double missing = 0.0;   // counts slots that stayed empty (summed over the workgroup like the sums themselves)
   for (uint32_t t = lo + threadIdx.x; t < hi; t += BS) {
     if constexpr (SHARED) {
-      aW += peek_f64(partials + 2 * (size_t)t);
-      aR += peek_f64(partials + 2 * (size_t)t + 1);
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        unsigned long long bits = peek_u64(partials + 2 * (size_t)t + h);
+        for (uint32_t tries = 0; bits == kNoSumYet && tries < patience; tries++) {
+          __builtin_amdgcn_s_sleep(8);
+          bits = peek_u64(partials + 2 * (size_t)t + h);
+        }
+        if (bits == kNoSumYet) missing += 1.0;
+        else if (h == 0) aW += __longlong_as_double((long long)bits);
+        else aR += __longlong_as_double((long long)bits);
+      }
     } else {
       aW += partials[2 * (size_t)t];
       aR += partials[2 * (size_t)t + 1];
@@ -295,14 +321,20 @@ __device__ __forceinline__ float lamb_finalize_segment(const double* partials, u
   }
   const double sW = group_sum<BS>(aW, lds);
   const double sR = group_sum<BS>(aR, lds + kBlock / kWave);
+  bool ok = true;
+  if constexpr (SHARED) {
+    const double gaps = group_sum<BS>(missing, lds);
+    ok = gaps == 0.0;
+    if (complete && threadIdx.x == 0) *complete = ok;
+  }
   float sc = 0.0f;
-  if (threadIdx.x == 0 && mode == CCN_LAMB_NCCL_GLOBAL) {
+  if (threadIdx.x == 0 && ok && mode == CCN_LAMB_NCCL_GLOBAL) {
     const float wNorm = sqrtf((float)sW), rNorm = sqrtf((float)sR);
     norms[2 * b] = wNorm;
     norms[2 * b + 1] = rNorm;
     sc = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f) / rNorm;
     scale[b] = sc;
-  } else if (threadIdx.x == 0) {
+  } else if (threadIdx.x == 0 && ok) {
     const double rNorm = sqrt(sR);
     const double wNorm = sqrt(sW / (double)seg_len);
     const double ratio = ((wNorm > 0) ? (rNorm > 0 ? wNorm / rNorm : 1.0f) : 1.0f);
@@ -428,10 +460,14 @@ struct LambResident {
   uint32_t* ndeferred;              // zero at kernel start
   uint32_t ntiles;
   uint32_t spin_limit;
+  uint32_t withhold;                // test hook: scales are computed but never announced, as if their sums had not arrived
 };
 
-__global__ void lamb_reset_kernel(uint32_t* cnt, unsigned long long* ready, int nseg, uint32_t* ndeferred) {
+// Runs before every launch of the resident kernels: counters and ready words to zero, every tile-sum slot to "no sum yet".
+__global__ void lamb_reset_kernel(uint32_t* cnt, unsigned long long* ready, int nseg, uint32_t* ndeferred, double* partials,
+                                  uint32_t ntiles) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if ((uint32_t)i < 2 * ntiles) reinterpret_cast<unsigned long long*>(partials)[i] = kNoSumYet;
   if (i < nseg) {
     ready[i] = 0;
 #pragma unroll
@@ -558,10 +594,10 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       const double sW = group_sum<BS>(accW, red);
       const double sR = group_sum<BS>(accR, red + kBlock / kWave);
       if (threadIdx.x == 0) {
-        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile,
-                           (unsigned long long)__double_as_longlong(sW), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile + 1,
-                           (unsigned long long)__double_as_longlong(sR), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile, sum_bits(sW), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile + 1, sum_bits(sR), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
         drain_vector_memory();   // the sums are in place before the count says so
         const uint32_t seg_lo = rs.seg_tile_begin[t.seg];
         seg_tiles = rs.seg_tile_begin[t.seg + 1] - seg_lo;
@@ -598,9 +634,11 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       }
       __syncthreads();
       if (bc[0]) {
+        bool complete = false;
         const float sc = lamb_finalize_segment<BS, true>(partials, rs.seg_tile_begin[t.seg], rs.seg_tile_begin[t.seg + 1],
-                                                         seg_len[t.seg], (int)t.seg, norms, scale, k.mode, red);
-        if (threadIdx.x == 0)
+                                                         seg_len[t.seg], (int)t.seg, norms, scale, k.mode, red, rs.spin_limit,
+                                                         &complete);
+        if (threadIdx.x == 0 && complete && !rs.withhold)   // otherwise the trailing kernel adds the segment up
           __hip_atomic_store(&rs.ready[t.seg], (1ull << 32) | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
@@ -706,10 +744,10 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
   const double sW = group_sum<BS>(accW, red);
   const double sR = group_sum<BS>(accR, red + kBlock / kWave);
   if (threadIdx.x == 0) {
-    __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile,
-                       (unsigned long long)__double_as_longlong(sW), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile + 1,
-                       (unsigned long long)__double_as_longlong(sR), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile, sum_bits(sW), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile + 1, sum_bits(sR), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
     drain_vector_memory();   // the sums are in place before the count says so
     const uint32_t seg_lo = rs.seg_tile_begin[t.seg];
     const uint32_t seg_tiles = rs.seg_tile_begin[t.seg + 1] - seg_lo;
@@ -727,9 +765,10 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
   }
   __syncthreads();
   if (bc[0]) {
+    bool complete = false;
     const float sc = lamb_finalize_segment<BS, true>(partials, rs.seg_tile_begin[t.seg], rs.seg_tile_begin[t.seg + 1],
-                                                     seg_len[t.seg], (int)t.seg, norms, scale, k.mode, red);
-    if (threadIdx.x == 0)
+                                                     seg_len[t.seg], (int)t.seg, norms, scale, k.mode, red, rs.spin_limit, &complete);
+    if (threadIdx.x == 0 && complete && !rs.withhold)   // otherwise the trailing kernel adds the segment up
       __hip_atomic_store(&rs.ready[t.seg], (1ull << 32) | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (threadIdx.x == 0) {
@@ -780,18 +819,38 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
   }
 }
 
-// Finishes the deferred tiles: pass 2 from the stored m and v, as the two-pass path does.
+// Finishes the deferred tiles: pass 2 from the stored m and v, as the two-pass path does.  A tile is deferred because its
+// segment's scale had not been announced when its patience ran out; if it never was (the workgroup that added the segment
+// up found a sum missing), the segment is added up here, where every sum of the previous kernel is in place: every
+// workgroup that needs the scale computes the same value in the same fixed order and writes the same norms.
 template <int BS, int SUB, bool SCAT, bool HALF = false>
 __global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, uint16_t* halfw, const float* m, const float* v, const LambLayout lay,
-                                                           const float* __restrict__ scale,
+                                                           float* __restrict__ scale, const unsigned long long* __restrict__ ready,
+                                                           const double* __restrict__ partials,
+                                                           const uint32_t* __restrict__ seg_tile_begin,
+                                                           const uint64_t* __restrict__ seg_len, double* norms,
                                                            const uint32_t* __restrict__ deferred,
                                                            const uint32_t* __restrict__ ndeferred, const int vec_ok,
                                                            const LambPrm k) {
+  __shared__ double red[2 * kBlock / kWave];
+  __shared__ float late_scale;
   const uint32_t n = *ndeferred;
   for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
     const LambTile t = lamb_tile_of(lay, deferred[i]);
     float* const wt = lamb_weights_of<SCAT>(lay, w, t.seg);
-    const float step_scale = k.lr * scale[t.seg];
+    const unsigned long long word = ready[t.seg];
+    float sc;
+    if (word >> 32) {
+      sc = __uint_as_float((uint32_t)word);
+    } else {
+      const float mine = lamb_finalize_segment<BS, false>(partials, seg_tile_begin[t.seg], seg_tile_begin[t.seg + 1], seg_len[t.seg],
+                                                          (int)t.seg, norms, scale, k.mode, red);
+      if (threadIdx.x == 0) late_scale = mine;
+      __syncthreads();
+      sc = late_scale;
+      __syncthreads();
+    }
+    const float step_scale = k.lr * sc;
     for (int u = 0; u < SUB; u++) {
       const uint32_t j0 = (u * BS + threadIdx.x) * 4;
       if (j0 >= t.count) continue;
@@ -867,6 +926,7 @@ struct ccn_lamb_plan {
   uint32_t res_ntiles = 0;
   uint64_t res_uniform_seg_len = 0;
   uint32_t spin_limit = 0;
+  uint32_t withhold = 0;          // CCN_LAMB_WITHHOLD=1: test hook, see LambResident
   LambTile* rtiles = nullptr;
   uint32_t* seg_rtile_begin = nullptr;
   double* rpartials = nullptr;
@@ -1096,6 +1156,7 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   p->res_lds = res_lds;
   p->oneshot = oneshot;
   p->spin_limit = (uint32_t)env_long("CCN_LAMB_SPIN", 1 << 15);
+  p->withhold = env_long("CCN_LAMB_WITHHOLD", 0) != 0 ? 1u : 0u;
   hipError_t e = hipSuccess;
   auto alloc = [&](void** ptr, size_t bytes) { if (e == hipSuccess) e = hipMalloc(ptr, bytes ? bytes : 16); };
   auto upload = [&](void* dst, const void* src, size_t bytes) {
@@ -1243,8 +1304,12 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
     rs.deferred = plan->deferred;
     rs.ntiles = plan->res_ntiles;
     rs.spin_limit = plan->spin_limit;
-    hipLaunchKernelGGL(lamb_reset_kernel, dim3((unsigned)((plan->nseg + kBlock - 1) / kBlock)), block, 0, s, rs.cnt, rs.ready,
-                       plan->nseg, rs.ndeferred);
+    rs.withhold = plan->withhold;
+    {
+      const size_t items = 2 * (size_t)plan->res_ntiles > (size_t)plan->nseg ? 2 * (size_t)plan->res_ntiles : (size_t)plan->nseg;
+      hipLaunchKernelGGL(lamb_reset_kernel, dim3((unsigned)((items + kBlock - 1) / kBlock)), block, 0, s, rs.cnt, rs.ready, plan->nseg,
+                         rs.ndeferred, plan->rpartials, plan->res_ntiles);
+    }
     CCN_HIP(hipGetLastError());
     if (plan->oneshot) {
       with_ranks([&](auto ptag) {
@@ -1257,8 +1322,10 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
       CCN_HIP(hipGetLastError());
       const unsigned dg = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
       hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<kOneshotBlock, kOneshotSub, true> : lamb_deferred_kernel<kOneshotBlock, kOneshotSub, false>),
-                         dim3(dg), dim3(kOneshotBlock), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v, lay, (const float*)plan->scale,
-                         (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred, vec_ok, k);
+                         dim3(dg), dim3(kOneshotBlock), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v, lay, plan->scale,
+                         (const unsigned long long*)plan->ready, (const double*)plan->rpartials, (const uint32_t*)plan->seg_rtile_begin,
+                         (const uint64_t*)plan->seg_len, plan->norms, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
+                         vec_ok, k);
       CCN_HIP(hipGetLastError());
     } else {
     // The wait in the kernel is bounded either way, but it only pays when the whole grid is resident.
@@ -1288,8 +1355,9 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
       constexpr int BS = decltype(bstag)::value;
       constexpr int SUB = decltype(subtag)::value;
       hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<BS, SUB, true> : lamb_deferred_kernel<BS, SUB, false>), dim3(dgrid),
-                         dim3(BS), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v,
-                         lay, (const float*)plan->scale, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
+                         dim3(BS), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v, lay, plan->scale,
+                         (const unsigned long long*)plan->ready, (const double*)plan->rpartials, (const uint32_t*)plan->seg_rtile_begin,
+                         (const uint64_t*)plan->seg_len, plan->norms, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
                          vec_ok, k);
     });
     CCN_HIP(hipGetLastError());
@@ -1380,8 +1448,12 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
     rs.deferred = plan->deferred;
     rs.ntiles = plan->res_ntiles;
     rs.spin_limit = plan->spin_limit;
-    hipLaunchKernelGGL(lamb_reset_kernel, dim3((unsigned)((plan->nseg + kBlock - 1) / kBlock)), block, 0, s, rs.cnt, rs.ready,
-                       plan->nseg, rs.ndeferred);
+    rs.withhold = plan->withhold;
+    {
+      const size_t items = 2 * (size_t)plan->res_ntiles > (size_t)plan->nseg ? 2 * (size_t)plan->res_ntiles : (size_t)plan->nseg;
+      hipLaunchKernelGGL(lamb_reset_kernel, dim3((unsigned)((items + kBlock - 1) / kBlock)), block, 0, s, rs.cnt, rs.ready, plan->nseg,
+                         rs.ndeferred, plan->rpartials, plan->res_ntiles);
+    }
     CCN_HIP(hipGetLastError());
     with_rank_count(P, [&](auto ptag) {
       constexpr int PP = decltype(ptag)::value;
@@ -1394,8 +1466,9 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
     CCN_HIP(hipGetLastError());
     const unsigned dg = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
     hipLaunchKernelGGL((lamb_deferred_kernel<kOneshotBlock, kOneshotSub, false, true>), dim3(dg), dim3(kOneshotBlock), 0, s, w,
-                       halfw, (const float*)m, (const float*)v, lay, (const float*)plan->scale,
-                       (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred, vec_ok, k);
+                       halfw, (const float*)m, (const float*)v, lay, plan->scale, (const unsigned long long*)plan->ready,
+                       (const double*)plan->rpartials, (const uint32_t*)plan->seg_rtile_begin, (const uint64_t*)plan->seg_len,
+                       plan->norms, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred, vec_ok, k);
     CCN_HIP(hipGetLastError());
     return CCN_OK;
   }

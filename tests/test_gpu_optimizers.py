@@ -420,12 +420,16 @@ LAMB_VARIANTS = {
     "deferred": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0"},
     "deferred-wave": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0", "CCN_LAMB_RES_BLOCK": "64"},
     "two-pass": {"CCN_LAMB_RESIDENT": "0"},
+    # the workgroup that adds a segment up keeps the result to itself, as it does when a tile sum has not arrived: every
+    # tile runs out of patience and the trailing kernel adds the segments up from the sums in memory
+    "one-tile-withheld": {"CCN_LAMB_WITHHOLD": "1", "CCN_LAMB_SPIN": "8"},
+    "resident-withheld": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_WITHHOLD": "1", "CCN_LAMB_SPIN": "8"},
 }
 
 
 @pytest.fixture(params=list(LAMB_VARIANTS))
 def lamb_variant(request, monkeypatch):
-    for k in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT"):
+    for k in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT", "CCN_LAMB_WITHHOLD"):
         monkeypatch.delenv(k, raising=False)
     for k, val in LAMB_VARIANTS[request.param].items():
         monkeypatch.setenv(k, val)
@@ -576,7 +580,7 @@ def test_lamb_full_size_segments(ccn):
     # norms computed by torch on the device from the weights before the step and the moments after it; (b) against the
     # two-pass kernels, which exchange nothing inside a launch, on the same inputs: their sums associate differently, so
     # equal to rounding, not to the bit.
-    b1, b2, eps, wd = 0.9, 0.999, 1e-6, 0.01
+    b1, b2, eps, wd = (float(np.float32(x)) for x in (0.9, 0.999, 1e-6, 0.01))      # the scalars as the C ABI receives them
     ref = np.empty((nseg, 2))
     for b in range(nseg):
         sl = slice(b * seglen, (b + 1) * seglen)
