@@ -282,6 +282,86 @@ __global__ __launch_bounds__(BS) void bias_dropout_residual_kernel(const float* 
   epilogue_finish<NP, REF>(a, in, bias, out, idx, idx % N, ep, mask_base + idx);
 }
 
+// Shapes that are not whole 128 x 128 x 64 tiles (any M and K; N a multiple of 4, which keeps a quad of columns inside a
+// row and the rows of the fp32 operands 16-byte aligned): 64 x 64 output tiles, 32-deep steps staged through LDS as fp32
+// with the out-of-range part filled with zeros, 4 x 4 outputs per thread accumulated in fp32 in ascending k on the
+// vector ALUs.  Slower than the matrix-core kernel by an order of magnitude, and meant for the odd shape only; the
+// epilogue is the same code.  nP is a run-time count here: the partial sums are added to the product in buffer order
+// before the shared epilogue sees it, which is the order the fixed-count epilogue uses.
+constexpr int GT = 64, GK = 32;
+template <bool PLAIN, bool REF>
+__global__ __launch_bounds__(kBlock) void outproj_any_shape_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
+                                                                   const SrcTable<float, 8> parts, const int nP,
+                                                                   const float* __restrict__ bias,
+                                                                   const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
+                                                                   const int M, const int N, const int K, const EpiPrm ep) {
+  __shared__ float xs[GT][GK + 1];
+  __shared__ __align__(16) float ws[GK][GT];
+  const int tiles_n = (N + GT - 1) / GT;
+  const int m0 = (int)(blockIdx.x / tiles_n) * GT, n0 = (int)(blockIdx.x % tiles_n) * GT;
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += GK) {
+    // X tile: 64 rows x 32 k, 8 elements per thread (rows need not be aligned: K is arbitrary)
+#pragma unroll
+    for (int i = 0; i < (GT * GK) / kBlock; i++) {
+      const int e = i * kBlock + threadIdx.x, r = e / GK, c = e % GK;
+      const int m = m0 + r, k = k0 + c;
+      xs[r][c] = (m < M && k < K) ? bf16_bits_to_f32(X[(size_t)m * K + k]) : 0.0f;
+    }
+    // W tile: 32 k x 64 n in quads of columns (N % 4 == 0: a quad is inside the row or outside it, and 8-byte aligned)
+#pragma unroll
+    for (int i = 0; i < (GK * GT / 4) / kBlock; i++) {
+      const int e = i * kBlock + threadIdx.x, r = e / (GT / 4), c = (e % (GT / 4)) * 4;
+      const int k = k0 + r, n = n0 + c;
+      f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (k < K && n < N) {
+        const u32x2 b = *reinterpret_cast<const u32x2*>(W + (size_t)k * N + n);
+        v[0] = bf16_bits_to_f32((uint16_t)(b[0] & 0xffffu));
+        v[1] = bf16_bits_to_f32((uint16_t)(b[0] >> 16));
+        v[2] = bf16_bits_to_f32((uint16_t)(b[1] & 0xffffu));
+        v[3] = bf16_bits_to_f32((uint16_t)(b[1] >> 16));
+      }
+      *reinterpret_cast<f32x4*>(&ws[r][c]) = v;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < GK; kk++) {
+      const f32x4 b = *reinterpret_cast<const f32x4*>(&ws[kk][tx * 4]);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float a = xs[ty * 4 + i][kk];
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = acc[i][j] + a * b[j];
+      }
+    }
+    __syncthreads();
+  }
+  const int n = n0 + tx * 4;
+  if (n >= N) return;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+    const size_t idx = (size_t)m * N + n;
+    f32x4 sum = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+    if constexpr (PLAIN) {
+      *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(out) + idx) = sum;
+    } else {
+      for (int q = 0; q < nP; q++) sum = sum + __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts.p[q] + idx));
+      EpiIn<0> in;
+      epilogue_load<0>(in, parts, resid, idx);
+      epilogue_finish<0, REF>(sum, in, bias, out, idx, (size_t)n, ep, idx);
+    }
+  }
+}
+
+static inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+
 static int make_epi(float p_drop, uint64_t seed, int mode, EpiPrm* ep) {
   if (mode < CCN_DROPOUT_INVERTED || mode > CCN_DROPOUT_REF_NCCL_SAT) return CCN_EINVAL;
   // inverted dropout rescales by 1/(1-p): p < 1.  The reference's forms keep with probability p: p = 1 keeps everything.
@@ -307,7 +387,7 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
                    void* stream) {
   if (!X || !W || !bias || !out || nPartials < 0 || nPartials > 8 || (nPartials > 0 && !partials)) return CCN_EINVAL;
   if (M <= 0 || N <= 0 || K <= 0) return CCN_EINVAL;
-  if (M % BM || N % BN || K % BK) return CCN_ERANGE;   // whole tiles only
+  if (N % 4) return CCN_ERANGE;   // a quad of columns never straddles two rows
   SrcTable<float, 8> tbl;
   for (int q = 0; q < 8; q++) {
     tbl.p[q] = q < nPartials ? partials[q] : nullptr;
@@ -320,8 +400,20 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
   const DeviceInfo* di = nullptr;
   rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
-  const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
   hipStream_t s = as_stream(stream);
+  if (M % BM || N % BN || K % BK) {   // not whole tiles of the matrix-core kernel
+    const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
+    if (tiles > 0x7fffffffull) return CCN_ERANGE;
+    if (mode == CCN_DROPOUT_INVERTED)
+      hipLaunchKernelGGL((outproj_any_shape_kernel<false, false>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
+                         bias, resid, out, M, N, K, ep);
+    else
+      hipLaunchKernelGGL((outproj_any_shape_kernel<false, true>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
+                         bias, resid, out, M, N, K, ep);
+    CCN_HIP(hipGetLastError());
+    return CCN_OK;
+  }
+  const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
   switch (nPartials) {
 #define CCN_CASE(Q)                                                                                                          \
   case Q:                                                                                                                    \
@@ -345,7 +437,8 @@ int epilogue_launch(const float* acc, const float* const* partials, int nPartial
     tbl.p[q] = q < nPartials ? partials[q] : nullptr;
     if (q < nPartials && (!partials[q] || !aligned16(partials[q]))) return CCN_EINVAL;
   }
-  if (!aligned16(acc) || !aligned16(bias) || !aligned16(out) || (resid && !aligned16(resid))) return CCN_EINVAL;
+  // fp32 operands move 16 bytes at a time, the bf16 ones 8 (a band of rows of a larger output may start on any quad)
+  if (!aligned16(acc) || !aligned16(bias) || !aligned8(out) || (resid && !aligned8(resid))) return CCN_EINVAL;
   EpiPrm ep;
   int rc = make_epi(p_drop, seed, mode, &ep);
   if (rc != CCN_OK) return rc;
@@ -419,7 +512,7 @@ int ccn_bias_dropout_residual_ex(const float* acc, const float* const* partials,
 int ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
   if (!X || !W || !C) return CCN_EINVAL;
   if (M <= 0 || N <= 0 || K <= 0) return CCN_EINVAL;
-  if (M % BM || N % BN || K % BK) return CCN_ERANGE;   // whole tiles only
+  if (N % 4) return CCN_ERANGE;
   if (!aligned16(X) || !aligned16(W) || !aligned16(C)) return CCN_EINVAL;
   const DeviceInfo* di = nullptr;
   const int rc = current_device_info(&di);
@@ -427,6 +520,14 @@ int ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, i
   SrcTable<float, 8> tbl;
   for (int q = 0; q < 8; q++) tbl.p[q] = nullptr;
   EpiPrm ep{};
+  if (M % BM || N % BN || K % BK) {
+    const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
+    if (tiles > 0x7fffffffull) return CCN_ERANGE;
+    hipLaunchKernelGGL((outproj_any_shape_kernel<true, false>), dim3((unsigned)tiles), dim3(kBlock), 0, as_stream(stream), X, W, tbl,
+                       0, (const float*)nullptr, (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), M, N, K, ep);
+    CCN_HIP(hipGetLastError());
+    return CCN_OK;
+  }
   const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
   hipLaunchKernelGGL((mlp_outproj_kernel<0, true>), grid, block, 0, as_stream(stream), X, W, tbl, (const float*)nullptr,
                      (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), N, K, ep);

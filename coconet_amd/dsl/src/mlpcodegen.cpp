@@ -224,7 +224,7 @@ std::string generateMLP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   o << ind << "const size_t M = " << product(c.in->dims, 0, nd - 1) << ", Kfull = " << c.in->dims[nd - 1]->name << ", N = "
     << c.w->dims[1]->name << ";\n";
   o << ind << "const size_t K = DIVUP(Kfull, (size_t)comm_size);   // this rank's slice of the reduction dimension\n";
-  o << ind << "if (M % 128 || N % 128 || K % 64) { printf(\"skipping M=%zu N=%zu K=%zu: not whole 128x128x64 tiles\\n\", M, N, K); continue; }\n";
+  o << ind << "if (N % 4) { printf(\"skipping N=%zu: the row length must be a multiple of 4\\n\", N); continue; }\n";
   if (level < 2 && scattered)
     o << ind << "if (M % (size_t)comm_size) { printf(\"skipping M=%zu: a rank's slice must be whole rows\\n\", M); continue; }\n";
   o << ind << "const int nPartials = comm_size - 1;   // the other ranks' partial products, resident as fp32 [M,N]\n";

@@ -57,7 +57,7 @@ def test_argument_validation_happens_before_any_device_work():
     tbl[3] = None
     assert lib.ccn_reduce_f32(p, 4, 0x1000, 16, None) == capi.CCN_EINVAL
     assert lib.ccn_mlp_outproj_bf16(None, 0x1000, null, 0, 0x1000, None, 0x1000, 128, 128, 64, 0.1, 0, None) == capi.CCN_EINVAL
-    assert lib.ccn_mlp_outproj_bf16(0x1000, 0x1000, null, 0, 0x1000, None, 0x1000, 100, 128, 64, 0.1, 0, None) == capi.CCN_ERANGE
+    assert lib.ccn_mlp_outproj_bf16(0x1000, 0x1000, null, 0, 0x1000, None, 0x1000, 128, 130, 64, 0.1, 0, None) == capi.CCN_ERANGE   # N % 4
     assert lib.ccn_mlp_outproj_bf16(0x1000, 0x1000, null, 0, 0x1000, None, 0x1000, 128, 128, 64, 1.0, 0, None) == capi.CCN_EINVAL
     plan = C.c_void_p()
     offs = (C.c_size_t * 3)(0, 10, 10)

@@ -62,6 +62,37 @@ def test_outproj_against_oracle(ccn, M, N, K, nP, p):
     assert np.max(np.abs(gf - want_f32) / (np.abs(want_f32) + 1.0)) < 2.0 ** -7
 
 
+@pytest.mark.parametrize("M,N,K,nP,p,mode", [(100, 128, 64, 7, 0.1, None), (128, 132, 64, 2, 0.0, None), (128, 128, 72, 3, 0.3, None),
+                                              (1, 4, 1, 0, 0.0, None), (67, 36, 129, 7, 0.5, 1), (300, 260, 200, 8, 0.25, 3),
+                                              (130, 64, 31, 1, 0.2, 2)])
+def test_outproj_shapes_that_are_not_whole_tiles(ccn, M, N, K, nP, p, mode):
+    """Any M and K, N a multiple of 4: the vector-ALU kernel behind the same entry points (the reference's cuBLAS call
+    takes any shape), same epilogue, same bar as the matrix-core kernel."""
+    X, W, parts, bias, resid = make_case(90 + nP, M, N, K, nP)
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(bf16_dev(X), bf16_dev(W), [torch.from_numpy(q).to(DEV) for q in parts], torch.from_numpy(bias).to(DEV),
+                         bf16_dev(resid), out, M, N, K, p, 5, dropout_mode=mode)
+    got = bf16_host(out).reshape(M, N)
+    want, want_f32 = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, p, 5, mode=mode or 0)
+    d = bf16_ulp_distance(got, want)
+    assert d.max() <= 1, f"max bf16 ulp distance {d.max()}"
+    assert (d > 0).mean() < 0.03, f"{(d > 0).mean():.4f} of the outputs differ by one ulp"
+    if mode is None:
+        keep = orc.dropout_mask(5, 0, M * N, p).reshape(M, N).astype(bool)
+        assert np.array_equal(got[~keep], resid[~keep])
+
+
+@pytest.mark.parametrize("M,N,K", [(100, 132, 70), (1, 4, 1), (129, 128, 64), (64, 64, 33)])
+def test_plain_product_of_any_shape(ccn, M, N, K):
+    X, W, _, _, _ = make_case(95, M, N, K, 0)
+    Cd = torch.full((M, N), -1.0, device=DEV)
+    ccn.matmul_bf16_f32(bf16_dev(X), bf16_dev(W), Cd, M, N, K)
+    torch.cuda.synchronize()
+    xf, wf = orc.bf16_to_f32(X).astype(np.float64), orc.bf16_to_f32(W).astype(np.float64)
+    bound = K * 2.0 ** -24 * (np.abs(xf) @ np.abs(wf))
+    assert np.all(np.abs(Cd.cpu().numpy().astype(np.float64) - xf @ wf) <= bound + 1e-30)
+
+
 def test_outproj_all_ones_known_answer(ccn):
     # the reference's own check at this boundary: all-ones operands give C == K*ranks
     # (nccl-overlap/samples/matmul-allreduce-bias-dropout-layernorm.cu:520-526)
@@ -258,5 +289,5 @@ def test_plain_product(ccn):
     bound = K * 2.0 ** -24 * (np.abs(xf) @ np.abs(wf))           # fp32 accumulation of K exact products
     assert np.all(np.abs(Cd.cpu().numpy().astype(np.float64) - ref) <= bound + 1e-30)
     with pytest.raises(ccn.CoconetError) as e:
-        ccn.matmul_bf16_f32(bf16_dev(X), bf16_dev(W), Cd, M, N, K - 1)
+        ccn.matmul_bf16_f32(bf16_dev(X), bf16_dev(W), Cd, M, N - 2, K)   # a quad of columns must stay inside a row
     assert e.value.code == ccn.CCN_ERANGE
