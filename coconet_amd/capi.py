@@ -29,7 +29,7 @@ SYMBOLS = [
     "ccn_memcpy_d2d", "ccn_fill_f32", "ccn_stream_create", "ccn_stream_destroy", "ccn_stream_sync",
     "ccn_event_create", "ccn_event_destroy", "ccn_event_record", "ccn_event_elapsed_ms", "ccn_last_hip_error",
     "ccn_strerror", "ccn_reduce_f32", "ccn_sgd_f32", "ccn_sgd_axpby_f32", "ccn_pseudo_adam_f32", "ccn_adam_f32",
-    "ccn_adam_f16g", "ccn_overflow_check_f16", "ccn_fused_adam_ref_f16g", "ccn_lamb_plan_create",
+    "ccn_adam_f16g", "ccn_overflow_check_f16", "ccn_fused_adam_ref_f16g", "ccn_lamb_plan_create", "ccn_lamb_plan_create_parented",
     "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
     "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
     "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
@@ -97,6 +97,7 @@ def _declare(L):
     sig("ccn_overflow_check_f16", [_pp, _i, _sz, _vp, _vp])
     sig("ccn_fused_adam_ref_f16g", [_pp, _i, _vp, _vp, _vp, _vp, _sz, _f, _f, _f, _vp])
     sig("ccn_lamb_plan_create", [C.POINTER(_sz), _i, _pp])
+    sig("ccn_lamb_plan_create_parented", [C.POINTER(_sz), C.POINTER(_sz), _i, _pp])
     sig("ccn_lamb_plan_destroy", [_vp])
     sig("ccn_lamb_f32", [_vp, _pp, _i, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
     sig("ccn_lamb_plan_norms", [_vp, _vp, _vp])
@@ -345,12 +346,22 @@ def fused_adam_ref_f16g(g, w, halfw, m, v, n, lr, beta1, beta2, stream=None):
 class LambPlan:
     """Device-side segment tables for one segmentation of [0, N) (ccn_lamb_plan)."""
 
-    def __init__(self, seg_offsets):
-        offs = [int(x) for x in seg_offsets]
-        self.nseg = len(offs) - 1
-        arr = (_sz * len(offs))(*offs)
+    def __init__(self, seg_offsets, buf_sizes=None, buf_parent=None):
+        """seg_offsets: nseg+1 element offsets, one buffer per segment.  Or buf_sizes / buf_parent (seg_offsets None):
+        segments made of several buffers each, buffer i belonging to segment buf_parent[i]."""
         h = C.c_void_p()
-        _check(load().ccn_lamb_plan_create(arr, self.nseg, C.byref(h)), "ccn_lamb_plan_create")
+        if buf_sizes is not None:
+            sizes, parent = [int(x) for x in buf_sizes], [int(x) for x in buf_parent]
+            assert len(sizes) == len(parent)
+            self.nbuf = len(sizes)
+            self.nseg = parent[-1] + 1 if parent else 0
+            _check(load().ccn_lamb_plan_create_parented((_sz * len(sizes))(*sizes), (_sz * len(parent))(*parent), self.nbuf,
+                                                        C.byref(h)), "ccn_lamb_plan_create_parented")
+        else:
+            offs = [int(x) for x in seg_offsets]
+            self.nseg = self.nbuf = len(offs) - 1
+            arr = (_sz * len(offs))(*offs)
+            _check(load().ccn_lamb_plan_create(arr, self.nseg, C.byref(h)), "ccn_lamb_plan_create")
         self.h = h
 
     def step(self, g, w, m, v, lr, beta1, beta2, eps, wd, step, mode=LAMB_TRUST_RATIO, stream=None):
@@ -359,10 +370,10 @@ class LambPlan:
                                    stream), "ccn_lamb_f32")
 
     def step_scattered(self, g, w, m, v, lr, beta1, beta2, eps, wd, step, mode=LAMB_TRUST_RATIO, stream=None):
-        """g: P lists of nseg buffers; w: nseg buffers (one per segment of the plan); m, v: single arrays."""
-        assert len(w) == self.nseg and all(len(gp) == self.nseg for gp in g)
-        gt = (C.c_void_p * (len(g) * self.nseg))(*[addr(x) for gp in g for x in gp])
-        wt = (C.c_void_p * self.nseg)(*[addr(x) for x in w])
+        """g: P lists of nbuf buffers; w: nbuf buffers (one per buffer of the plan); m, v: single arrays."""
+        assert len(w) == self.nbuf and all(len(gp) == self.nbuf for gp in g)
+        gt = (C.c_void_p * (len(g) * self.nbuf))(*[addr(x) for gp in g for x in gp])
+        wt = (C.c_void_p * self.nbuf)(*[addr(x) for x in w])
         _check(load().ccn_lamb_f32_scattered(self.h, gt, len(g), wt, addr(m), addr(v), lr, beta1, beta2, eps, wd, step, mode,
                                              stream), "ccn_lamb_f32_scattered")
 

@@ -33,7 +33,9 @@ struct LambTile {
   uint32_t count;   // elements in the tile (<= kLambTile)
   uint32_t seg;     // segment the tile belongs to
   float nf;         // (float) element count of that segment
-  uint32_t pad[3];
+  uint32_t buf;     // buffer the tile lies in: index into the pointer tables of the scattered layout (== seg unless a
+                    // segment is made of several buffers)
+  uint32_t pad[2];
 };
 static_assert(sizeof(LambTile) == 32, "tile record is 32 bytes");
 
@@ -46,16 +48,16 @@ struct LambLayout {
   // Scattered buffers (one gradient / weight buffer per segment, moments still in single arrays): device tables of the
   // segments' pointers, each already moved back by the segment's first element index, so that "pointer + global element
   // index" addresses the segment's elements exactly as it does for flat arrays.  Null for flat arrays.
-  const float* const* gtab;   // [P][nseg], rank-major
-  float* const* wtab;         // [nseg]
-  uint32_t nseg;
+  const float* const* gtab;   // [P][nbuf], rank-major
+  float* const* wtab;         // [nbuf]
+  uint32_t nbuf;              // buffers (== segments unless a segment is made of several buffers)
 };
 
-// Gradient table and weight pointer to use for the elements of segment `seg`.
+// Gradient table and weight pointer to use for the elements of buffer `buf`.
 // SCAT is a compile-time choice so that the flat kernels carry none of this.
 template <int P, bool SCAT>
 __device__ __forceinline__ void lamb_buffers_of(const LambLayout& L, const SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g_flat,
-                                                float* w_flat, int nP, uint32_t seg,
+                                                float* w_flat, int nP, uint32_t buf,
                                                 SrcTable<float, (P ? P : CCN_MAX_RANKS)>& g, float*& w) {
   if constexpr (!SCAT) {
     g = g_flat;
@@ -64,12 +66,12 @@ __device__ __forceinline__ void lamb_buffers_of(const LambLayout& L, const SrcTa
   }
   constexpr int PX = P > 0 ? P : CCN_MAX_RANKS;
 #pragma unroll
-  for (int p = 0; p < PX; p++) g.p[p] = (P > 0 || p < nP) ? L.gtab[(size_t)p * L.nseg + seg] : nullptr;
-  w = L.wtab[seg];
+  for (int p = 0; p < PX; p++) g.p[p] = (P > 0 || p < nP) ? L.gtab[(size_t)p * L.nbuf + buf] : nullptr;
+  w = L.wtab[buf];
 }
 template <bool SCAT>
-__device__ __forceinline__ float* lamb_weights_of(const LambLayout& L, float* w_flat, uint32_t seg) {
-  if constexpr (SCAT) return L.wtab[seg];
+__device__ __forceinline__ float* lamb_weights_of(const LambLayout& L, float* w_flat, uint32_t buf) {
+  if constexpr (SCAT) return L.wtab[buf];
   return w_flat;
 }
 
@@ -79,6 +81,7 @@ __device__ __forceinline__ LambTile lamb_tile_of(const LambLayout& L, unsigned b
     t.start = (uint64_t)b * L.tile;
     t.count = L.tile;
     t.seg = (uint32_t)(t.start / L.seg_len);
+    t.buf = t.seg;
     t.nf = L.seg_len_f;
     return t;
   }
@@ -188,7 +191,7 @@ __global__ __launch_bounds__(kBlock) void lamb_pass1_kernel(const SrcTable<float
   const LambTile t = lamb_tile_of(lay, blockIdx.x);
   SrcTable<float, (P ? P : CCN_MAX_RANKS)> gt;
   float* wt;
-  lamb_buffers_of<P, SCAT>(lay, g, const_cast<float*>(w), nP, t.seg, gt, wt);
+  lamb_buffers_of<P, SCAT>(lay, g, const_cast<float*>(w), nP, t.buf, gt, wt);
   double accW = 0.0, accR = 0.0;
   const uint32_t j0 = threadIdx.x * 4;          // this thread's elements of the tile: [j0, j0+4) clipped to count
   if (j0 < t.count) {
@@ -405,7 +408,7 @@ __global__ __launch_bounds__(kBlock) void lamb_pass2_kernel(float* w, const floa
                                                             const float* __restrict__ scale, const int vec_ok,
                                                             const LambPrm k) {
   const LambTile t = lamb_tile_of(lay, blockIdx.x);
-  float* const wt = lamb_weights_of<SCAT>(lay, w, t.seg);
+  float* const wt = lamb_weights_of<SCAT>(lay, w, t.buf);
   const float step_scale = k.lr * scale[t.seg];   // stepsize * scale, then times r
   const uint32_t j0 = threadIdx.x * 4;
   if (j0 >= t.count) return;
@@ -531,7 +534,7 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
   float* wt = w;
   if (blockIdx.x < rs.ntiles) {
     next = lamb_tile_of(lay, blockIdx.x);
-    lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.seg, gt, wt);
+    lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.buf, gt, wt);
     if (is_fast(next)) lamb_pass1_load<P, 4>(pre, gt, nP, wt, m, v, next.start + threadIdx.x * 4);
   }
   for (unsigned it = 0; it < rounds + (kResDepth - 1); it++) {
@@ -588,7 +591,7 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       }
       if (it + 1 < rounds && tile + G < rs.ntiles) {
         next = lamb_tile_of(lay, tile + G);
-        lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.seg, gt, wt);
+        lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.buf, gt, wt);
         if (is_fast(next)) lamb_pass1_load<P, 4>(pre, gt, nP, wt, m, v, next.start + threadIdx.x * 4);
       }
       const double sW = group_sum<BS>(accW, red);
@@ -616,7 +619,7 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       }
       __syncthreads();
       if (bc[1]) {
-        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.seg), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
+        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.buf), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
                                   k.lr * __uint_as_float(bc[2]), vec_ok);
         retired = true;
       }
@@ -664,7 +667,7 @@ __global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float,
       }
       __syncthreads();
       if (bc[1])
-        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.seg), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
+        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.buf), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
                                   k.lr * __uint_as_float(bc[2]), vec_ok);
     }
     __syncthreads();   // bc and the retired slot are reused by the next round
@@ -696,7 +699,7 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
   SrcTable<G, (P ? P : CCN_MAX_RANKS)> gt;
   float* wt;
   if constexpr (SCAT) {
-    lamb_buffers_of<P, SCAT>(lay, g, w, nP, t.seg, gt, wt);
+    lamb_buffers_of<P, SCAT>(lay, g, w, nP, t.buf, gt, wt);
   } else {
     gt = g;
     wt = w;
@@ -837,7 +840,7 @@ __global__ __launch_bounds__(BS) void lamb_deferred_kernel(float* w, uint16_t* h
   const uint32_t n = *ndeferred;
   for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
     const LambTile t = lamb_tile_of(lay, deferred[i]);
-    float* const wt = lamb_weights_of<SCAT>(lay, w, t.seg);
+    float* const wt = lamb_weights_of<SCAT>(lay, w, t.buf);
     const unsigned long long word = ready[t.seg];
     float sc;
     if (word >> 32) {
@@ -937,7 +940,9 @@ struct ccn_lamb_plan {
   int occupancy[CCN_MAX_RANKS + 1] = {0};   // resident workgroups per CU by rank count, 0 = not asked yet
   // scattered buffers: the segments' gradient and weight pointers, moved back by the segment's first element index
   std::vector<uint64_t> seg_start;
-  const void** ptr_dev = nullptr;       // [CCN_MAX_RANKS * nseg] gradients, rank-major, then [nseg] weights; made on first use
+  int nbuf = 0;                         // buffers of the scattered layout (== nseg unless segments are made of several)
+  std::vector<uint64_t> buf_start;
+  const void** ptr_dev = nullptr;       // [CCN_MAX_RANKS * nbuf] gradients, rank-major, then [nbuf] weights; made on first use
   const void** ptr_pinned = nullptr;
   std::vector<const void*> ptr_shadow;  // what the device table holds
   int ptr_ranks = 0;
@@ -1011,14 +1016,16 @@ int oneshot_occupancy(int P, unsigned lds) {
 }
 
 // Cuts segment b into tiles of `tile` elements appended to `out`.
-void cut_segment(std::vector<LambTile>& out, const size_t* seg_offsets, int b, uint64_t tile) {
-  const uint64_t n = seg_offsets[b + 1] - seg_offsets[b];
-  for (uint64_t off = 0; off < n; off += tile) {
+// Tiles of the elements [begin, end) of buffer `buf`, which belongs to segment `seg` of seg_n elements.
+void cut_buffer(std::vector<LambTile>& out, uint64_t begin, uint64_t end, uint64_t tile, uint32_t seg, uint64_t seg_n,
+                uint32_t buf) {
+  for (uint64_t at = begin; at < end; at += tile) {
     LambTile t{};
-    t.start = seg_offsets[b] + off;
-    t.count = (uint32_t)((n - off) < tile ? (n - off) : tile);
-    t.seg = (uint32_t)b;
-    t.nf = (float)n;
+    t.start = at;
+    t.count = (uint32_t)((end - at) < tile ? (end - at) : tile);
+    t.seg = seg;
+    t.nf = (float)seg_n;
+    t.buf = buf;
     out.push_back(t);
   }
 }
@@ -1042,9 +1049,26 @@ int ccn_lamb_plan_destroy(ccn_lamb_plan* plan) {
   return rc;
 }
 
-static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_only, ccn_lamb_plan** out) {
+// buf_offsets (nbuf + 1 entries) cuts [0, N) into the buffers of the scattered layout; every segment boundary is a buffer
+// boundary.  Null: one buffer per segment.
+static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_only, ccn_lamb_plan** out,
+                            const size_t* buf_offsets = nullptr, int nbuf = 0) {
   for (int b = 0; b < nseg; b++) {
     if (seg_offsets[b + 1] <= seg_offsets[b]) return CCN_EINVAL;   // empty or descending segment
+  }
+  if (!buf_offsets) {
+    buf_offsets = seg_offsets;
+    nbuf = nseg;
+  }
+  const bool parented = nbuf != nseg;
+  {
+    if (nbuf < nseg || buf_offsets[0] != 0 || buf_offsets[nbuf] != seg_offsets[nseg]) return CCN_EINVAL;
+    int b = 0;
+    for (int q = 0; q < nbuf; q++) {
+      if (buf_offsets[q + 1] <= buf_offsets[q]) return CCN_EINVAL;        // empty buffer
+      if (buf_offsets[q] == seg_offsets[b + 1]) b++;                      // the next segment starts with this buffer
+      if (buf_offsets[q + 1] > seg_offsets[b + 1]) return CCN_EINVAL;     // a buffer may not straddle two segments
+    }
   }
   const DeviceInfo* di = nullptr;
   int rc = current_device_info(&di);
@@ -1103,24 +1127,29 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   std::vector<uint32_t> begin((size_t)nseg + 1), rbegin((size_t)nseg + 1);
   std::vector<uint64_t> len((size_t)nseg);
   bool all_two_pass = true, all_resident = true;
+  int q = 0;   // first buffer of segment b
   for (int b = 0; b < nseg; b++) {
     begin[b] = (uint32_t)tiles.size();
     rbegin[b] = (uint32_t)rtiles.size();
     const uint64_t n = seg_offsets[b + 1] - seg_offsets[b];
     len[b] = n;
-    const bool resident = resident_wanted && resident_ok && (n + res_tile - 1) / res_tile <= res_cap_tiles;
-    if (resident) {
-      cut_segment(rtiles, seg_offsets, b, res_tile);
-      all_two_pass = false;
-    } else {
-      cut_segment(tiles, seg_offsets, b, kLambTile);
-      all_resident = false;
+    int q_end = q;
+    uint64_t res_tiles = 0;   // tiles never cross a buffer boundary: every buffer rounds up on its own
+    while (q_end < nbuf && buf_offsets[q_end] < seg_offsets[b + 1]) {
+      res_tiles += (buf_offsets[q_end + 1] - buf_offsets[q_end] + res_tile - 1) / res_tile;
+      q_end++;
     }
+    const bool resident = resident_wanted && resident_ok && res_tiles <= res_cap_tiles;
+    for (; q < q_end; q++)
+      cut_buffer(resident ? rtiles : tiles, buf_offsets[q], buf_offsets[q + 1], resident ? res_tile : (uint64_t)kLambTile,
+                 (uint32_t)b, n, (uint32_t)q);
+    if (resident) all_two_pass = false;
+    else all_resident = false;
     if (tiles.size() > 0x7fffffffu || rtiles.size() > 0x7fffffffu) return CCN_ERANGE;
   }
   begin[nseg] = (uint32_t)tiles.size();
   rbegin[nseg] = (uint32_t)rtiles.size();
-  uint64_t uniform = len[0];
+  uint64_t uniform = parented ? 0 : len[0];   // tile -> segment by division only when a buffer is a segment
   for (int b = 1; b < nseg; b++) if (len[b] != uniform) uniform = 0;
 
   // groups of at most kLambFold tiles for the two-pass segments, if any of them is longer than that
@@ -1146,6 +1175,8 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   p->nseg = nseg;
   p->N = seg_offsets[nseg];
   p->seg_start.assign(seg_offsets, seg_offsets + nseg);
+  p->nbuf = nbuf;
+  p->buf_start.assign(buf_offsets, buf_offsets + nbuf);
   p->ntiles = tiles.size();
   p->uniform_seg_len = (all_two_pass && uniform % kLambTile == 0) ? uniform : 0;
   p->res_block = res_block;
@@ -1200,23 +1231,43 @@ int ccn_lamb_plan_create(const size_t* seg_offsets, int nseg, ccn_lamb_plan** ou
   return guarded([&] { return lamb_plan_create(seg_offsets, nseg, false, out); });
 }
 
+int ccn_lamb_plan_create_parented(const size_t* buf_sizes, const size_t* buf_parent, int nbuf, ccn_lamb_plan** out) {
+  if (!out) return CCN_EINVAL;
+  *out = nullptr;
+  if (!buf_sizes || !buf_parent || nbuf < 1 || buf_parent[0] != 0) return CCN_EINVAL;
+  return guarded([&] {
+    std::vector<size_t> boffs((size_t)nbuf + 1, 0), soffs(1, 0);
+    for (int q = 0; q < nbuf; q++) {
+      if (buf_sizes[q] == 0) return (int)CCN_EINVAL;
+      if (q > 0 && buf_parent[q] != buf_parent[q - 1]) {
+        if (buf_parent[q] != buf_parent[q - 1] + 1) return (int)CCN_EINVAL;   // parents in order, none skipped
+        soffs.push_back(boffs[q]);
+      }
+      boffs[q + 1] = boffs[q] + buf_sizes[q];
+    }
+    soffs.push_back(boffs[nbuf]);
+    if (soffs.size() - 1 > 0x7fffffffu) return (int)CCN_ERANGE;
+    return lamb_plan_create(soffs.data(), (int)(soffs.size() - 1), false, out, boffs.data(), nbuf);
+  });
+}
+
 }  // extern "C"
 
 namespace {
 
-// Brings the plan's device table of per-segment pointers in line with the caller's; copies (and waits for the copy, so
+// Brings the plan's device table of per-buffer pointers in line with the caller's; copies (and waits for the copy, so
 // that the staging buffer can be reused) only when they have changed since the last call.  Returns whether every
-// pointer, moved back by its segment's first element index, is 16-byte aligned.
+// pointer, moved back by its buffer's first element index, is 16-byte aligned.
 int sync_segment_pointers(ccn_lamb_plan* plan, const float* const* g, int P, float* const* w, hipStream_t s, bool* aligned) {
-  const size_t ns = (size_t)plan->nseg, words = (size_t)(CCN_MAX_RANKS + 1) * ns;
+  const size_t ns = (size_t)plan->nbuf, words = (size_t)(CCN_MAX_RANKS + 1) * ns;
   if (!plan->ptr_dev) {
     CCN_HIP(hipMalloc((void**)&plan->ptr_dev, words * sizeof(void*)));
     CCN_HIP(hipHostMalloc((void**)&plan->ptr_pinned, words * sizeof(void*), hipHostMallocDefault));
   }
   std::vector<const void*> want(words, nullptr);
   bool al = true;
-  auto moved = [&](const float* base, size_t seg) {
-    const float* q = base - plan->seg_start[seg];
+  auto moved = [&](const float* base, size_t buf) {
+    const float* q = base - plan->buf_start[buf];
     al = al && aligned16(q);
     return (const void*)q;
   };
@@ -1233,17 +1284,17 @@ int sync_segment_pointers(ccn_lamb_plan* plan, const float* const* g, int P, flo
   return CCN_OK;
 }
 
-// One step.  Flat arrays: g holds P pointers, w_flat the weights, w_seg is null.  Scattered buffers: g holds P * nseg
-// pointers (rank-major), w_seg nseg pointers, w_flat is null.
+// One step.  Flat arrays: g holds P pointers, w_flat the weights, w_seg is null.  Scattered buffers: g holds P * nbuf
+// pointers (rank-major), w_seg nbuf pointers, w_flat is null.
 int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, float* const* w_seg, float* m, float* v, float lr,
               float beta1, float beta2, float eps, float wd, int step, int mode, void* stream) {
   const bool scattered = w_seg != nullptr;
   if (!plan || !g || (!w_flat && !w_seg) || !m || !v || P < 1 || P > CCN_MAX_RANKS || step < 1) return CCN_EINVAL;
   if (mode != CCN_LAMB_TRUST_RATIO && mode != CCN_LAMB_REFERENCE && mode != CCN_LAMB_NCCL_GLOBAL) return CCN_EINVAL;
-  const size_t ng = scattered ? (size_t)P * (size_t)plan->nseg : (size_t)P;
+  const size_t ng = scattered ? (size_t)P * (size_t)plan->nbuf : (size_t)P;
   for (size_t i = 0; i < ng; i++) if (!g[i]) return CCN_EINVAL;
   if (scattered)
-    for (int b = 0; b < plan->nseg; b++) if (!w_seg[b]) return CCN_EINVAL;
+    for (int b = 0; b < plan->nbuf; b++) if (!w_seg[b]) return CCN_EINVAL;
   const DeviceInfo* di = nullptr;
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
@@ -1277,7 +1328,7 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
   const dim3 block(kBlock);
   const float* const* gtab = scattered ? reinterpret_cast<const float* const*>(plan->ptr_dev) : nullptr;
   float* const* wtab =
-      scattered ? reinterpret_cast<float* const*>(const_cast<void**>(plan->ptr_dev) + (size_t)CCN_MAX_RANKS * plan->nseg) : nullptr;
+      scattered ? reinterpret_cast<float* const*>(const_cast<void**>(plan->ptr_dev) + (size_t)CCN_MAX_RANKS * plan->nbuf) : nullptr;
 
   auto with_ranks = [&](auto body) { with_rank_count(P, body); };
   auto table = [&](auto ptag) {   // the flat arrays' gradient pointers; unused (null) for scattered buffers
@@ -1295,7 +1346,7 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
     lay.tile = (uint32_t)(plan->res_block * 4 * plan->res_sub);
     lay.gtab = gtab;
     lay.wtab = wtab;
-    lay.nseg = (uint32_t)plan->nseg;
+    lay.nbuf = (uint32_t)plan->nbuf;
     LambResident rs;
     rs.cnt = plan->sync;
     rs.ndeferred = plan->sync + (size_t)plan->nseg * kResCntStride;
@@ -1373,7 +1424,7 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
     lay.tile = kLambTile;
     lay.gtab = gtab;
     lay.wtab = wtab;
-    lay.nseg = (uint32_t)plan->nseg;
+    lay.nbuf = (uint32_t)plan->nbuf;
     // Residency caps measured for N = 2^28, P = 8: pass 1 is fastest at 4 workgroups per CU (its float64 sums and the
     // workgroup reduction need more wavefronts to hide than the plain Adam kernel), pass 2 uncapped.
     const unsigned lds1 = lds_for_residency(P >= 2 ? 4 : 0);
@@ -1439,7 +1490,7 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
     lay.tile = (uint32_t)(plan->res_block * 4 * plan->res_sub);
     lay.gtab = nullptr;
     lay.wtab = nullptr;
-    lay.nseg = (uint32_t)plan->nseg;
+    lay.nbuf = (uint32_t)plan->nbuf;
     LambResident rs;
     rs.cnt = plan->sync;
     rs.ndeferred = plan->sync + (size_t)plan->nseg * kResCntStride;
@@ -1474,9 +1525,10 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
   }
 
   if (!plan->two_pass_twin) {
-    std::vector<size_t> offs(plan->seg_start.begin(), plan->seg_start.end());
+    std::vector<size_t> offs(plan->seg_start.begin(), plan->seg_start.end()), boffs(plan->buf_start.begin(), plan->buf_start.end());
     offs.push_back(plan->N);
-    rc = lamb_plan_create(offs.data(), plan->nseg, true, &plan->two_pass_twin);
+    boffs.push_back(plan->N);
+    rc = lamb_plan_create(offs.data(), plan->nseg, true, &plan->two_pass_twin, boffs.data(), plan->nbuf);
     if (rc != CCN_OK) return rc;
   }
   ccn_lamb_plan* tp = plan->two_pass_twin;
@@ -1488,7 +1540,7 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
   lay.tile = kLambTile;
   lay.gtab = nullptr;
   lay.wtab = nullptr;
-  lay.nseg = (uint32_t)tp->nseg;
+  lay.nbuf = (uint32_t)tp->nbuf;
   with_rank_count(P, [&](auto ptag) {
     constexpr int PP = decltype(ptag)::value;
     SrcTable<uint16_t, (PP ? PP : CCN_MAX_RANKS)> tbl;
@@ -1605,7 +1657,7 @@ int ccn_lamb_f32_static(const float* const* g, int P, float* w, float* m, float*
   lay.tile = kLambTile;
   lay.gtab = nullptr;
   lay.wtab = nullptr;
-  lay.nseg = nseg;
+  lay.nbuf = nseg;
   hipStream_t s = as_stream(stream);
   const dim3 block(kBlock), grid(ntiles);
   double* const norms_dst = norms ? norms : sc->norms;

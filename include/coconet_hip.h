@@ -171,6 +171,15 @@ int  ccn_lamb_f32(ccn_lamb_plan* plan, const float* const* g, int P, float* w, f
  * buffers; moments stay in single arrays over the concatenation), as ncclAllReduceScatteredLAMB takes them
  * (nccl-overlap/src/nccl.h.in:219-221).  g: host array of P*nseg device pointers, rank-major; w: host array of nseg
  * device pointers.  The plan keeps a device copy of the pointers, refreshed (one stream synchronisation) when they change. */
+/* A plan whose norm segments are made of several buffers each: the reference cuts every parameter tensor ("parent
+ * buffer") into small buffers of at most maxBuffSize elements, passes one gradient / weight pointer per small buffer and
+ * maps them back with buffIdToParentBufferId; the norms are per parent (nccl-overlap/src/nccl.h.in:219-221, sample
+ * nccl-overlap/samples/multi-process-adam-scattered.cpp:505-517, 671-674).  buf_sizes[i]: elements of buffer i;
+ * buf_parent[i]: its parent, starting at 0 and never decreasing or skipping (the buffers of a parent are consecutive,
+ * as the sample builds them).  The plan then has buf_parent[nbuf-1]+1 segments; ccn_lamb_f32_scattered on it takes
+ * P*nbuf gradient pointers (rank-major) and nbuf weight pointers, the moments are single arrays over the concatenation
+ * of the buffers, and ccn_lamb_plan_norms returns the parents' norms.  The flat call works on such a plan as well. */
+int  ccn_lamb_plan_create_parented(const size_t* buf_sizes, const size_t* buf_parent, int nbuf, ccn_lamb_plan** plan);
 int  ccn_lamb_f32_scattered(ccn_lamb_plan* plan, const float* const* g, int P, float* const* w, float* m, float* v,
                             float lr, float beta1, float beta2, float eps, float wd, int step, int mode, void* stream);
 /* The modified NCCL's mixed-precision LAMB: fp16 gradients (their sum carried in fp16, the square taken in fp16), fp32

@@ -64,6 +64,12 @@ def test_argument_validation_happens_before_any_device_work():
     assert lib.ccn_lamb_plan_create(offs, 2, C.byref(plan)) == capi.CCN_EINVAL      # empty segment
     offs = (C.c_size_t * 3)(1, 10, 20)
     assert lib.ccn_lamb_plan_create(offs, 2, C.byref(plan)) == capi.CCN_EINVAL      # does not start at 0
+    sizes = (C.c_size_t * 3)(5, 0, 7)
+    par = (C.c_size_t * 3)(0, 0, 1)
+    assert lib.ccn_lamb_plan_create_parented(sizes, par, 3, C.byref(plan)) == capi.CCN_EINVAL   # empty buffer
+    sizes = (C.c_size_t * 3)(5, 6, 7)
+    for bad in ((1, 1, 2), (0, 2, 2), (0, 1, 0)):   # does not start at 0, skips a parent, goes back
+        assert lib.ccn_lamb_plan_create_parented(sizes, (C.c_size_t * 3)(*bad), 3, C.byref(plan)) == capi.CCN_EINVAL
     assert lib.ccn_lamb_f32(None, p, 2, 0x1000, 0x1000, 0x1000, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, 0, None) == capi.CCN_EINVAL
     assert lib.ccn_lamb_nccl_f16g(None, p, 2, 0x1000, 0x1000, 0x1000, 0x1000, 1e-3, 0.9, 0.999, 1.0, None) == capi.CCN_EINVAL
     tbl[3] = 0x1000

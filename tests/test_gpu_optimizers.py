@@ -876,6 +876,55 @@ def test_scattered_lamb(ccn, mode, lamb_variant):
         assert np.max(np.abs(got.astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("max_buf", [1000, 4096, 20000])
+def test_scattered_lamb_with_parent_buffers(ccn, mode, max_buf, lamb_variant):
+    """The reference cuts every parameter tensor into small buffers of at most maxBuffSize elements and maps them back
+    with buffIdToParentBufferId (nccl-overlap/samples/multi-process-adam-scattered.cpp:505-517); the norms are per
+    parent.  Every small buffer is an allocation of its own here; results must be the oracle's on the concatenated
+    arrays with one segment per parent, and the parents' norms those of the plan that takes the parents whole."""
+    P = 3
+    parents = [700, 4096 + 5, 1, 30000, 8192, 2 * max_buf]
+    sizes, parent_of = [], []
+    for i, n in enumerate(parents):
+        for lo in range(0, n, max_buf):
+            sizes.append(min(max_buf, n - lo))
+            parent_of.append(i)
+    segs = np.concatenate([[0], np.cumsum(parents)]).tolist()
+    offs = np.concatenate([[0], np.cumsum(sizes)]).tolist()
+    N = segs[-1]
+    g = grads_f32(197, P, N, 1e-3)
+    w0 = weights_f32(197, N, 0.05)
+    pieces = lambda flat: [dev(flat[offs[q]:offs[q + 1]]) for q in range(len(sizes))]
+    gd, wd = [pieces(x) for x in g], pieces(w0)
+    m0 = weights_f32(198, N, 0.01)
+    v0 = np.abs(weights_f32(199, N, 1e-3)) + np.float32(1e-5)
+    md, vd = dev(m0), dev(v0)
+    w, m, v = w0.copy(), m0.copy(), v0.copy()
+    plan = ccn.LambPlan(None, buf_sizes=sizes, buf_parent=parent_of)
+    assert plan.nseg == len(parents) and plan.nbuf == len(sizes)
+    for t in (1, 2):
+        plan.step_scattered(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, mode)
+        orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, mode)
+    norms = plan.norms()
+    plan.close()
+    assert_f32_parity(host(md), m, "parented lamb m")
+    assert_f32_parity(host(vd), v, "parented lamb v")
+    got = np.concatenate([host(x) for x in wd])
+    assert np.max(np.abs(got.astype(np.float64) - w)) <= FP32_TOL * np.max(np.abs(w))
+    # the same two steps with the parents whole: the norms of the second step agree to the last few bits (the tile sums
+    # are cut differently, so the float64 additions associate differently)
+    whole = ccn.LambPlan(segs)
+    wd2, md2, vd2 = dev(w0), dev(m0), dev(v0)
+    gd2 = [dev(x) for x in g]
+    for t in (1, 2):
+        whole.step(gd2, wd2, md2, vd2, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, mode)
+    want = whole.norms()
+    whole.close()
+    assert norms.shape == want.shape == (len(parents), 2)
+    assert np.max(np.abs(norms - want) / np.maximum(np.abs(want), 1e-300)) < 1e-12
+
+
 @pytest.mark.parametrize("which,ranks", [("adam", 2), ("adam", 8), ("lamb", 2), ("lamb", 3)])
 def test_cpp_harness_in_the_shape_of_the_reference_sample(which, ranks):
     """tests/harness/adam_lamb_scattered.cpp: the flow of the reference's multi-process-adam-scattered.cpp (its buffer
