@@ -6,8 +6,10 @@
 // check_epoch_results_adam / check_epoch_results_lamb (:81-153, :371-462) this runs the CPU oracle and the sample's
 // comparator (eq_float, :60-66) on every element.
 //
-//   adam_lamb_scattered <adam|lamb> [ranks=2] [scale_down=16]
+//   adam_lamb_scattered <adam|lamb> [ranks=2] [scale_down=16] [max_buff_size=0]
 // Buffer sizes: head and tail of the sample's list (:736), the large ones divided by scale_down to fit a test.
+// max_buff_size > 0 (lamb): every parent buffer is cut into small buffers of at most that many elements, each an
+// allocation of its own, with the sample's smallBufferIdToParentBufferId map (:505-517); the norms stay per parent.
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -28,7 +30,7 @@
 
 int main(int argc, char** argv) {
   if (argc < 2) {
-    printf("usage: %s <adam|lamb> [ranks=2] [scale_down=16]\n", argv[0]);
+    printf("usage: %s <adam|lamb> [ranks=2] [scale_down=16] [max_buff_size=0]\n", argv[0]);
     return 1;
   }
   const bool lamb = std::string(argv[1]) == "lamb";
@@ -36,8 +38,25 @@ int main(int argc, char** argv) {
   const size_t down = argc > 3 ? (size_t)atoi(argv[3]) : 16;
   const size_t listed[] = {31260672, 2048, 1048576, 1048576, 1048576, 1048576, 4194304, 4194304,
                            1024,     1024, 1024,    1024,    30528,   1024,    1024,    1024};
-  std::vector<size_t> sizes;
-  for (size_t s : listed) sizes.push_back(s > (1u << 20) ? s / down : s);
+  const size_t max_buff = argc > 4 ? (size_t)atoll(argv[4]) : 0;
+  std::vector<size_t> parent_sizes;
+  for (size_t s : listed) parent_sizes.push_back(s > (1u << 20) ? s / down : s);
+  const int nparents = (int)parent_sizes.size();
+  std::vector<size_t> parent_offs(nparents + 1, 0);
+  for (int i = 0; i < nparents; i++) parent_offs[i + 1] = parent_offs[i] + parent_sizes[i];
+  // the buffers the calls see: the parents themselves, or their pieces
+  std::vector<size_t> sizes, parent_of;
+  for (int i = 0; i < nparents; i++) {
+    if (lamb && max_buff > 0) {
+      for (size_t lo = 0; lo < parent_sizes[i]; lo += max_buff) {
+        sizes.push_back(parent_sizes[i] - lo < max_buff ? parent_sizes[i] - lo : max_buff);
+        parent_of.push_back((size_t)i);
+      }
+    } else {
+      sizes.push_back(parent_sizes[i]);
+      parent_of.push_back((size_t)i);
+    }
+  }
   const int nbuffs = (int)sizes.size();
   std::vector<size_t> offs(nbuffs + 1, 0);
   for (int i = 0; i < nbuffs; i++) offs[i + 1] = offs[i] + sizes[i];
@@ -46,9 +65,9 @@ int main(int argc, char** argv) {
   CCNCHECK(ccn_init(0));
   // host copies (the checker's state) and device buffers
   std::vector<float> hg(total), hw(total), hm(total, 0.f), hv(total, 0.f);
-  for (int i = 0; i < nbuffs; i++)
-    for (size_t index = 0; index < sizes[i]; index++)
-      hg[offs[i] + index] = hw[offs[i] + index] = (float)(i % 2 + 1) * (float)(index % 20 + 1);
+  for (int i = 0; i < nparents; i++)
+    for (size_t index = 0; index < parent_sizes[i]; index++)
+      hg[parent_offs[i] + index] = hw[parent_offs[i] + index] = (float)(i % 2 + 1) * (float)(index % 20 + 1);
   std::vector<const float*> g_ptrs((size_t)P * nbuffs);
   std::vector<float*> w_ptrs(nbuffs);
   for (int p = 0; p < P; p++)
@@ -72,7 +91,8 @@ int main(int argc, char** argv) {
   const float alpha = 1.0f, beta1 = 0.5f, beta2 = 0.5f, eps = 1e-6f;
   ccn_scatter_plan* sp = nullptr;
   ccn_lamb_plan* lp = nullptr;
-  if (lamb) CCNCHECK(ccn_lamb_plan_create(offs.data(), nbuffs, &lp));
+  if (lamb && max_buff > 0) CCNCHECK(ccn_lamb_plan_create_parented(sizes.data(), parent_of.data(), nbuffs, &lp));
+  else if (lamb) CCNCHECK(ccn_lamb_plan_create(offs.data(), nbuffs, &lp));
   else CCNCHECK(ccn_scatter_plan_create(sizes.data(), nbuffs, &sp));
 
   std::vector<const float*> og(P, hg.data());   // every rank holds the same gradients, as in the sample
@@ -88,8 +108,8 @@ int main(int argc, char** argv) {
     for (int i = 0; i < nbuffs; i++)
       CCNCHECK(ccn_memcpy_d2h(got.data() + offs[i], w_ptrs[i], sizes[i] * sizeof(float), nullptr));
     CCNCHECK(ccn_stream_sync(nullptr));
-    if (lamb) orc_lamb_f32(og.data(), P, hw.data(), hm.data(), hv.data(), offs.data(), nbuffs, -alpha, beta1, beta2, eps, 1.0f,
-                           iter + 1, 1, nullptr);
+    if (lamb) orc_lamb_f32(og.data(), P, hw.data(), hm.data(), hv.data(), parent_offs.data(), nparents, -alpha, beta1, beta2, eps,
+                           1.0f, iter + 1, 1, nullptr);
     else orc_adam_f32(og.data(), P, hw.data(), hm.data(), hv.data(), total, -alpha, beta1, beta2, eps, iter + 1);
     for (size_t i = 0; i < total; i++) {
       if (!orc_eq_float_1e5(hw[i], got[i])) {
@@ -98,7 +118,7 @@ int main(int argc, char** argv) {
         break;
       }
     }
-    if (ok) printf("Epoch %d: %s weights match the checker on %zu elements in %d buffers\n", iter, lamb ? "LAMB" : "Adam", total, nbuffs);
+    if (ok) printf("Epoch %d: %s weights match the checker on %zu elements in %d buffers of %d parents\n", iter, lamb ? "LAMB" : "Adam", total, nbuffs, nparents);
   }
   if (lamb) CCNCHECK(ccn_lamb_plan_destroy(lp));
   else CCNCHECK(ccn_scatter_plan_destroy(sp));

@@ -925,8 +925,9 @@ def test_scattered_lamb_with_parent_buffers(ccn, mode, max_buf, lamb_variant):
     assert np.max(np.abs(norms - want) / np.maximum(np.abs(want), 1e-300)) < 1e-12
 
 
-@pytest.mark.parametrize("which,ranks", [("adam", 2), ("adam", 8), ("lamb", 2), ("lamb", 3)])
-def test_cpp_harness_in_the_shape_of_the_reference_sample(which, ranks):
+@pytest.mark.parametrize("which,ranks,max_buff", [("adam", 2, 0), ("adam", 8, 0), ("lamb", 2, 0), ("lamb", 3, 0),
+                                                  ("lamb", 2, 65536), ("lamb", 3, 5000)])
+def test_cpp_harness_in_the_shape_of_the_reference_sample(which, ranks, max_buff):
     """tests/harness/adam_lamb_scattered.cpp: the flow of the reference's multi-process-adam-scattered.cpp (its buffer
     list, integer inputs, five checked epochs, its comparator) through the scattered entry points, from C++."""
     import os
@@ -934,7 +935,8 @@ def test_cpp_harness_in_the_shape_of_the_reference_sample(which, ranks):
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "harness", "build", "adam_lamb_scattered")
     if not os.path.exists(exe):
         pytest.skip("harness not built (make -C tests/harness)")
-    r = subprocess.run([exe, which, str(ranks)], capture_output=True, text=True, timeout=240)
+    # max_buff > 0: the parents cut into small buffers with the sample's parent map (LAMB)
+    r = subprocess.run([exe, which, str(ranks), "16", str(max_buff)], capture_output=True, text=True, timeout=240)
     assert r.returncode == 0 and "Success" in r.stdout, (r.stdout[-1500:], r.stderr[-500:])
     assert r.stdout.count("weights match the checker") == 5
 
