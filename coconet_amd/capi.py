@@ -35,6 +35,7 @@ SYMBOLS = [
     "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
     "ccn_lamb_f32_scattered", "ccn_adam_bf16g", "ccn_lamb_nccl_f16g", "ccn_lamb_f32_static",
     "ccn_mlp_outproj_bf16_ex", "ccn_bias_dropout_residual_ex", "ccn_matmul_bf16_f32",
+    "ccn_mlp_outproj_f16_ex", "ccn_bias_dropout_residual_f16_ex", "ccn_matmul_f16_f32",
 ]
 
 
@@ -109,6 +110,9 @@ def _declare(L):
     sig("ccn_mlp_outproj_bf16_ex", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _i, _vp])
     sig("ccn_bias_dropout_residual_ex", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _i, _sz, _vp])
     sig("ccn_matmul_bf16_f32", [_vp, _vp, _vp, _i, _i, _i, _vp])
+    sig("ccn_mlp_outproj_f16_ex", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _i, _vp])
+    sig("ccn_bias_dropout_residual_f16_ex", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _i, _sz, _vp])
+    sig("ccn_matmul_f16_f32", [_vp, _vp, _vp, _i, _i, _i, _vp])
     sig("ccn_scatter_plan_create", [C.POINTER(_sz), _i, _pp])
     sig("ccn_scatter_plan_destroy", [_vp])
     sig("ccn_sgd_f32_scattered", [_vp, _pp, _i, _pp, _f, _vp])
@@ -415,9 +419,13 @@ def lamb_f32_static(g, w, m, v, n, seg_len, lr, beta1, beta2, eps, wd, step, mod
 DROPOUT_INVERTED, DROPOUT_REF_DSL, DROPOUT_REF_NCCL, DROPOUT_REF_NCCL_SAT = 0, 1, 2, 3
 
 
-def mlp_outproj_bf16(X, W, partials, bias, resid, out, M, N, K, p_drop, seed, stream=None, dropout_mode=None):
+def mlp_outproj_bf16(X, W, partials, bias, resid, out, M, N, K, p_drop, seed, stream=None, dropout_mode=None, half=False):
+    """half=True: X, W, resid and out are IEEE half instead of bfloat16 (ccn_mlp_outproj_f16_ex)."""
     p, _keep = ptr_table(partials)
-    if dropout_mode is None:
+    if half:
+        _check(load().ccn_mlp_outproj_f16_ex(addr(X), addr(W), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
+                                             K, p_drop, seed, dropout_mode or 0, stream), "ccn_mlp_outproj_f16_ex")
+    elif dropout_mode is None:
         _check(load().ccn_mlp_outproj_bf16(addr(X), addr(W), p, len(partials), addr(bias), addr(resid), addr(out), M, N, K,
                                            p_drop, seed, stream), "ccn_mlp_outproj_bf16")
     else:
@@ -425,9 +433,14 @@ def mlp_outproj_bf16(X, W, partials, bias, resid, out, M, N, K, p_drop, seed, st
                                               K, p_drop, seed, dropout_mode, stream), "ccn_mlp_outproj_bf16_ex")
 
 
-def bias_dropout_residual(acc, partials, bias, resid, out, M, N, p_drop, seed, stream=None, dropout_mode=None, first_row=0):
+def bias_dropout_residual(acc, partials, bias, resid, out, M, N, p_drop, seed, stream=None, dropout_mode=None, first_row=0,
+                          half=False):
     p, _keep = ptr_table(partials)
-    if dropout_mode is None and first_row == 0:
+    if half:
+        _check(load().ccn_bias_dropout_residual_f16_ex(addr(acc), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
+                                                       p_drop, seed, dropout_mode or 0, first_row, stream),
+               "ccn_bias_dropout_residual_f16_ex")
+    elif dropout_mode is None and first_row == 0:
         _check(load().ccn_bias_dropout_residual(addr(acc), p, len(partials), addr(bias), addr(resid), addr(out), M, N,
                                                 p_drop, seed, stream), "ccn_bias_dropout_residual")
     else:
@@ -436,5 +449,8 @@ def bias_dropout_residual(acc, partials, bias, resid, out, M, N, p_drop, seed, s
                "ccn_bias_dropout_residual_ex")
 
 
-def matmul_bf16_f32(X, W, Cmat, M, N, K, stream=None):
-    _check(load().ccn_matmul_bf16_f32(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_bf16_f32")
+def matmul_bf16_f32(X, W, Cmat, M, N, K, stream=None, half=False):
+    if half:
+        _check(load().ccn_matmul_f16_f32(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_f16_f32")
+    else:
+        _check(load().ccn_matmul_bf16_f32(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_bf16_f32")

@@ -17,6 +17,7 @@
 namespace ccn {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 128, BN = 128, BK = 64;
@@ -27,6 +28,11 @@ struct EpiPrm {
   int apply_dropout;
   int mode;   // CCN_DROPOUT_*
 };
+
+// The 16-bit operands, residual and output are bfloat16 (F16 = false) or IEEE half (F16 = true: the type the reference's
+// model-parallel example declares); accumulation is fp32 either way.
+template <bool F16> __device__ __forceinline__ float half_in(uint16_t h) { return F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h); }
+template <bool F16> __device__ __forceinline__ uint16_t half_out(float f) { return F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f); }
 
 // Epilogue for four consecutive columns n..n+3 (n % 4 == 0) of row m, in two steps so that the loads of one quad can be
 // in flight while the previous one is finished.  NP, the number of partial buffers (0..8), is a compile-time constant:
@@ -50,7 +56,7 @@ __device__ __forceinline__ float sat01(float x) { return x > 0.0f ? (x < 1.0f ? 
 // from (the two differ when a call covers a band of rows of a larger output).
 // REF: one of the reference's dropout forms (k.mode says which); false: standard dropout, the form the kernels are
 // tuned for, compiled without the others.
-template <int NP, bool REF>
+template <int NP, bool REF, bool F16 = false>
 __device__ __forceinline__ void epilogue_finish(f32x4 acc, const EpiIn<NP>& in, const float* __restrict__ bias,
                                                 uint16_t* __restrict__ out, size_t idx, size_t n, const EpiPrm& k,
                                                 size_t mask_idx) {
@@ -58,8 +64,8 @@ __device__ __forceinline__ void epilogue_finish(f32x4 acc, const EpiIn<NP>& in, 
   f32x4 s = acc;
 #pragma unroll
   for (int q = 0; q < NP; q++) s = s + in.pv[q];
-  const float r0 = bf16_bits_to_f32((uint16_t)(in.rv[0] & 0xffffu)), r1 = bf16_bits_to_f32((uint16_t)(in.rv[0] >> 16));
-  const float r2 = bf16_bits_to_f32((uint16_t)(in.rv[1] & 0xffffu)), r3 = bf16_bits_to_f32((uint16_t)(in.rv[1] >> 16));
+  const float r0 = half_in<F16>((uint16_t)(in.rv[0] & 0xffffu)), r1 = half_in<F16>((uint16_t)(in.rv[0] >> 16));
+  const float r2 = half_in<F16>((uint16_t)(in.rv[1] & 0xffffu)), r3 = half_in<F16>((uint16_t)(in.rv[1] >> 16));
   float y0, y1, y2, y3;
   if constexpr (!REF) {
     // drop with probability p, survivors scaled by 1/(1-p)
@@ -98,8 +104,8 @@ __device__ __forceinline__ void epilogue_finish(f32x4 acc, const EpiIn<NP>& in, 
     y0 = y[0]; y1 = y[1]; y2 = y[2]; y3 = y[3];
   }
   u32x2 o;
-  o[0] = (uint32_t)f32_to_bf16_bits(y0) | ((uint32_t)f32_to_bf16_bits(y1) << 16);
-  o[1] = (uint32_t)f32_to_bf16_bits(y2) | ((uint32_t)f32_to_bf16_bits(y3) << 16);
+  o[0] = (uint32_t)half_out<F16>(y0) | ((uint32_t)half_out<F16>(y1) << 16);
+  o[1] = (uint32_t)half_out<F16>(y2) | ((uint32_t)half_out<F16>(y3) << 16);
   __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(out + idx));
 }
 
@@ -107,7 +113,7 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 7
 
 // PLAIN: the product alone, written as fp32 [M x N] through `out` (no partial buffers, bias, dropout or residual).
 // REF: the epilogue applies one of the reference's dropout forms.
-template <int NP, bool PLAIN = false, bool REF = false>
+template <int NP, bool PLAIN = false, bool REF = false, bool F16 = false>
 __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
                                                              const SrcTable<float, 8> parts,
                                                              const float* __restrict__ bias,
@@ -199,7 +205,11 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
       for (int bn = 0; bn < 2; bn++)
 #pragma unroll
         for (int bm = 0; bm < 2; bm++)
-          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[bn], fb[bm], acc[bn][bm], 0, 0, 0);
+          if constexpr (F16)
+            acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[bn]), __builtin_bit_cast(f16x8, fb[bm]),
+                                                                 acc[bn][bm], 0, 0, 0);
+          else
+            acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[bn], fb[bm], acc[bn][bm], 0, 0, 0);
     }
     __syncthreads();
     if (kt + 1 < nk) {
@@ -258,7 +268,7 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
         const int q = it * kBlock + t;
         const int row = q / (BN / 4), colq = q % (BN / 4);
         const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
-        epilogue_finish<NP, REF>(a, cur, bias, out, index_of(it), n0 + colq * 4, ep, index_of(it));
+        epilogue_finish<NP, REF, F16>(a, cur, bias, out, index_of(it), n0 + colq * 4, ep, index_of(it));
         if (it + 1 < kIters) cur = nxt;
       }
     }
@@ -267,7 +277,7 @@ __global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __r
 
 // Standalone epilogue over an fp32 product in memory: one quad per thread, no loop, the launch shape of the other
 // streaming kernels (the y dimension of the grid only comes into play beyond 2^30 workgroups).
-template <int NP, int BS, bool REF>
+template <int NP, int BS, bool REF, bool F16 = false>
 __global__ __launch_bounds__(BS) void bias_dropout_residual_kernel(const float* __restrict__ acc, const SrcTable<float, 8> parts,
                                                                    const float* __restrict__ bias,
                                                                    const uint16_t* __restrict__ resid,
@@ -279,7 +289,7 @@ __global__ __launch_bounds__(BS) void bias_dropout_residual_kernel(const float* 
   EpiIn<NP> in;
   const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(acc + idx));
   epilogue_load<NP>(in, parts, resid, idx);
-  epilogue_finish<NP, REF>(a, in, bias, out, idx, idx % N, ep, mask_base + idx);
+  epilogue_finish<NP, REF, F16>(a, in, bias, out, idx, idx % N, ep, mask_base + idx);
 }
 
 // Shapes that are not whole 128 x 128 x 64 tiles (any M and K; N a multiple of 4, which keeps a quad of columns inside a
@@ -289,7 +299,7 @@ __global__ __launch_bounds__(BS) void bias_dropout_residual_kernel(const float* 
 // epilogue is the same code.  nP is a run-time count here: the partial sums are added to the product in buffer order
 // before the shared epilogue sees it, which is the order the fixed-count epilogue uses.
 constexpr int GT = 64, GK = 32;
-template <bool PLAIN, bool REF>
+template <bool PLAIN, bool REF, bool F16 = false>
 __global__ __launch_bounds__(kBlock) void outproj_any_shape_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
                                                                    const SrcTable<float, 8> parts, const int nP,
                                                                    const float* __restrict__ bias,
@@ -311,7 +321,7 @@ __global__ __launch_bounds__(kBlock) void outproj_any_shape_kernel(const uint16_
     for (int i = 0; i < (GT * GK) / kBlock; i++) {
       const int e = i * kBlock + threadIdx.x, r = e / GK, c = e % GK;
       const int m = m0 + r, k = k0 + c;
-      xs[r][c] = (m < M && k < K) ? bf16_bits_to_f32(X[(size_t)m * K + k]) : 0.0f;
+      xs[r][c] = (m < M && k < K) ? half_in<F16>(X[(size_t)m * K + k]) : 0.0f;
     }
     // W tile: 32 k x 64 n in quads of columns (N % 4 == 0: a quad is inside the row or outside it, and 8-byte aligned)
 #pragma unroll
@@ -321,10 +331,10 @@ __global__ __launch_bounds__(kBlock) void outproj_any_shape_kernel(const uint16_
       f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
       if (k < K && n < N) {
         const u32x2 b = *reinterpret_cast<const u32x2*>(W + (size_t)k * N + n);
-        v[0] = bf16_bits_to_f32((uint16_t)(b[0] & 0xffffu));
-        v[1] = bf16_bits_to_f32((uint16_t)(b[0] >> 16));
-        v[2] = bf16_bits_to_f32((uint16_t)(b[1] & 0xffffu));
-        v[3] = bf16_bits_to_f32((uint16_t)(b[1] >> 16));
+        v[0] = half_in<F16>((uint16_t)(b[0] & 0xffffu));
+        v[1] = half_in<F16>((uint16_t)(b[0] >> 16));
+        v[2] = half_in<F16>((uint16_t)(b[1] & 0xffffu));
+        v[3] = half_in<F16>((uint16_t)(b[1] >> 16));
       }
       *reinterpret_cast<f32x4*>(&ws[r][c]) = v;
     }
@@ -355,7 +365,7 @@ __global__ __launch_bounds__(kBlock) void outproj_any_shape_kernel(const uint16_
       for (int q = 0; q < nP; q++) sum = sum + __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts.p[q] + idx));
       EpiIn<0> in;
       epilogue_load<0>(in, parts, resid, idx);
-      epilogue_finish<0, REF>(sum, in, bias, out, idx, (size_t)n, ep, idx);
+      epilogue_finish<0, REF, F16>(sum, in, bias, out, idx, (size_t)n, ep, idx);
     }
   }
 }
@@ -382,6 +392,7 @@ using namespace ccn;
 
 namespace {
 
+template <bool F16>
 int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials, const float* bias,
                    const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop, uint64_t seed, int mode,
                    void* stream) {
@@ -405,10 +416,10 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
     const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
     if (tiles > 0x7fffffffull) return CCN_ERANGE;
     if (mode == CCN_DROPOUT_INVERTED)
-      hipLaunchKernelGGL((outproj_any_shape_kernel<false, false>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
+      hipLaunchKernelGGL((outproj_any_shape_kernel<false, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
                          bias, resid, out, M, N, K, ep);
     else
-      hipLaunchKernelGGL((outproj_any_shape_kernel<false, true>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
+      hipLaunchKernelGGL((outproj_any_shape_kernel<false, true, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
                          bias, resid, out, M, N, K, ep);
     CCN_HIP(hipGetLastError());
     return CCN_OK;
@@ -417,8 +428,8 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
   switch (nPartials) {
 #define CCN_CASE(Q)                                                                                                          \
   case Q:                                                                                                                    \
-    if (mode == CCN_DROPOUT_INVERTED) hipLaunchKernelGGL((mlp_outproj_kernel<Q>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
-    else hipLaunchKernelGGL((mlp_outproj_kernel<Q, false, true>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
+    if (mode == CCN_DROPOUT_INVERTED) hipLaunchKernelGGL((mlp_outproj_kernel<Q, false, false, F16>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
+    else hipLaunchKernelGGL((mlp_outproj_kernel<Q, false, true, F16>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
     break;
     CCN_CASE(0) CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
 #undef CCN_CASE
@@ -427,6 +438,7 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
   return CCN_OK;
 }
 
+template <bool F16>
 int epilogue_launch(const float* acc, const float* const* partials, int nPartials, const float* bias, const uint16_t* resid,
                     uint16_t* out, int M, int N, float p_drop, uint64_t seed, int mode, size_t first_row, void* stream) {
   if (!acc || !bias || !out || nPartials < 0 || nPartials > 8 || (nPartials > 0 && !partials)) return CCN_EINVAL;
@@ -460,7 +472,7 @@ int epilogue_launch(const float* acc, const float* const* partials, int nPartial
     constexpr int Q = decltype(qtag)::value;
     auto launch = [&](auto bstag, auto reftag) {
       constexpr int BS = decltype(bstag)::value;
-      hipLaunchKernelGGL((bias_dropout_residual_kernel<Q, BS, decltype(reftag)::value>), grid, dim3(BS), sh.lds_bytes, s, acc, tbl, bias,
+      hipLaunchKernelGGL((bias_dropout_residual_kernel<Q, BS, decltype(reftag)::value, F16>), grid, dim3(BS), sh.lds_bytes, s, acc, tbl, bias,
                          resid, out, total, (size_t)N, mask_base, ep);
     };
     const bool ref = mode != CCN_DROPOUT_INVERTED;
@@ -481,35 +493,8 @@ int epilogue_launch(const float* acc, const float* const* partials, int nPartial
   return CCN_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
-                         const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
-                         uint64_t seed, void* stream) {
-  return outproj_launch(X, W, partials, nPartials, bias, resid, out, M, N, K, p_drop, seed, CCN_DROPOUT_INVERTED, stream);
-}
-
-int ccn_mlp_outproj_bf16_ex(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
-                            const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
-                            uint64_t seed, int dropout_mode, void* stream) {
-  return outproj_launch(X, W, partials, nPartials, bias, resid, out, M, N, K, p_drop, seed, dropout_mode, stream);
-}
-
-int ccn_bias_dropout_residual(const float* acc, const float* const* partials, int nPartials, const float* bias,
-                              const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
-                              void* stream) {
-  return epilogue_launch(acc, partials, nPartials, bias, resid, out, M, N, p_drop, seed, CCN_DROPOUT_INVERTED, 0, stream);
-}
-
-int ccn_bias_dropout_residual_ex(const float* acc, const float* const* partials, int nPartials, const float* bias,
-                                 const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
-                                 int dropout_mode, size_t first_row, void* stream) {
-  return epilogue_launch(acc, partials, nPartials, bias, resid, out, M, N, p_drop, seed, dropout_mode, first_row, stream);
-}
-
-int ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
+template <bool F16>
+int matmul_launch(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
   if (!X || !W || !C) return CCN_EINVAL;
   if (M <= 0 || N <= 0 || K <= 0) return CCN_EINVAL;
   if (N % 4) return CCN_ERANGE;
@@ -523,16 +508,64 @@ int ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, i
   if (M % BM || N % BN || K % BK) {
     const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
     if (tiles > 0x7fffffffull) return CCN_ERANGE;
-    hipLaunchKernelGGL((outproj_any_shape_kernel<true, false>), dim3((unsigned)tiles), dim3(kBlock), 0, as_stream(stream), X, W, tbl,
-                       0, (const float*)nullptr, (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), M, N, K, ep);
+    hipLaunchKernelGGL((outproj_any_shape_kernel<true, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, as_stream(stream), X, W,
+                       tbl, 0, (const float*)nullptr, (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), M, N, K, ep);
     CCN_HIP(hipGetLastError());
     return CCN_OK;
   }
   const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
-  hipLaunchKernelGGL((mlp_outproj_kernel<0, true>), grid, block, 0, as_stream(stream), X, W, tbl, (const float*)nullptr,
+  hipLaunchKernelGGL((mlp_outproj_kernel<0, true, false, F16>), grid, block, 0, as_stream(stream), X, W, tbl, (const float*)nullptr,
                      (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), N, K, ep);
   CCN_HIP(hipGetLastError());
   return CCN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ccn_mlp_outproj_bf16(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                         const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
+                         uint64_t seed, void* stream) {
+  return outproj_launch<false>(X, W, partials, nPartials, bias, resid, out, M, N, K, p_drop, seed, CCN_DROPOUT_INVERTED, stream);
+}
+
+int ccn_mlp_outproj_bf16_ex(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                            const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
+                            uint64_t seed, int dropout_mode, void* stream) {
+  return outproj_launch<false>(X, W, partials, nPartials, bias, resid, out, M, N, K, p_drop, seed, dropout_mode, stream);
+}
+
+int ccn_bias_dropout_residual(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                              const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                              void* stream) {
+  return epilogue_launch<false>(acc, partials, nPartials, bias, resid, out, M, N, p_drop, seed, CCN_DROPOUT_INVERTED, 0, stream);
+}
+
+int ccn_bias_dropout_residual_ex(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                                 const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                                 int dropout_mode, size_t first_row, void* stream) {
+  return epilogue_launch<false>(acc, partials, nPartials, bias, resid, out, M, N, p_drop, seed, dropout_mode, first_row, stream);
+}
+
+int ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
+  return matmul_launch<false>(X, W, C, M, N, K, stream);
+}
+
+int ccn_mlp_outproj_f16_ex(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                           const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K, float p_drop,
+                           uint64_t seed, int dropout_mode, void* stream) {
+  return outproj_launch<true>(X, W, partials, nPartials, bias, resid, out, M, N, K, p_drop, seed, dropout_mode, stream);
+}
+
+int ccn_bias_dropout_residual_f16_ex(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                                     const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                                     int dropout_mode, size_t first_row, void* stream) {
+  return epilogue_launch<true>(acc, partials, nPartials, bias, resid, out, M, N, p_drop, seed, dropout_mode, first_row, stream);
+}
+
+int ccn_matmul_f16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
+  return matmul_launch<true>(X, W, C, M, N, K, stream);
 }
 
 }  // extern "C"

@@ -26,7 +26,9 @@
 namespace ACCCDSL {
 
 // src/ast.hpp:48-102 of the reference: the same enumerators, usable with or without the enum name
-enum TensorElemType { None, Float16, Float32, Float64, Int8, Int16, Int32, Int64, UInt8, UInt16, UInt32, UInt64 };
+// BFloat16 is this build's addition (after the reference's values, which keep their numbers): the matrix-core type of
+// benchmark configuration 5; only MatMul pipelines take it.
+enum TensorElemType { None, Float16, Float32, Float64, Int8, Int16, Int32, Int64, UInt8, UInt16, UInt32, UInt64, BFloat16 };
 enum TensorLayout { Replicated, Sliced, Sliced_2, Local };
 enum ReduceOperation { Summation, Difference, Multiplication, Division, Maximum, Minimum };
 

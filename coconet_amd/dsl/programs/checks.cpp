@@ -174,6 +174,21 @@ int main(int argc, char** argv) {
       Stage out = r + Dropout(b + sum, 0.5);
       Pipeline pl("ok", {w, b, in, r}, {out});
       std::cout << generateHIP(pl, bounds);
+    } else if (c == "mlp_mixed_types") {   // a bfloat16 residual under Float16 operands
+      Tensor rb(BFloat16, {B, S, H}, Replicated, "rb");
+      Stage out = Dropout(sum + b, 0.5) + rb;
+      Pipeline pl("bad", {w, b, in, rb}, {out});
+      std::cout << generateHIP(pl, bounds);
+    } else if (c == "mlp_bfloat16") {      // the same chain declared in this build's BFloat16
+      Tensor wb(BFloat16, {H, H}, Sliced, "wb");
+      Tensor bb(BFloat16, H, Replicated, "bb");
+      Tensor inb(BFloat16, {B, S, H}, Sliced_2, "inb");
+      Tensor rb(BFloat16, {B, S, H}, Replicated, "rb");
+      Stage lb = MatMul(inb, wb);
+      Stage sb = AllReduce(Summation, lb);
+      Stage out = Dropout(sb + bb, 0.5) + rb;
+      Pipeline pl("ok", {wb, bb, inb, rb}, {out});
+      std::cout << generateHIP(pl, bounds);
     } else if (c == "mlp_no_bias_no_dropout") {
       Stage out = sum + r;
       Pipeline pl("ok", {w, b, in, r}, {out});

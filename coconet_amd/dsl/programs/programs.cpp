@@ -132,14 +132,15 @@ static void lamb(bool fused, const std::string& out) {
 }
 
 // The model-parallel MLP out-projection at benchmark configuration 5's shape: with 8 ranks, one rank's K-slice is
-// X [8192 x 1024] . W [1024 x 8192], the other 7 ranks' partial products are resident, then bias, dropout(0.1), residual.
+// X [8192 x 1024] . W [1024 x 8192] in bfloat16, the other 7 ranks' partial products are resident, then bias,
+// dropout(0.1), residual.
 //   unfused: MatMul, AllReduce and the pointwise part as separate steps      fused: one kernel
 static void mlp(bool fused, bool epilogueOnly, const std::string& out) {
   Variable B(Int32, "B"), S(Int32, "S"), H(Int32, "H");
-  Tensor w(Float16, {H, H}, Sliced, "w");
-  Tensor b(Float16, H, Replicated, "b");
-  Tensor in(Float16, {B, S, H}, Sliced_2, "in");
-  Tensor r(Float16, {B, S, H}, Replicated, "r");
+  Tensor w(BFloat16, {H, H}, Sliced, "w");
+  Tensor b(BFloat16, H, Replicated, "b");
+  Tensor in(BFloat16, {B, S, H}, Sliced_2, "in");
+  Tensor r(BFloat16, {B, S, H}, Replicated, "r");
   Stage layer = MatMul(in, w);
   Stage sum = AllReduce(Summation, layer);
   Stage sum2 = sum + b;

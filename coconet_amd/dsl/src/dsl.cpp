@@ -32,6 +32,7 @@ bool is_scalar(const NodePtr& n) {
 const char* elem_c_type(TensorElemType t) {
   switch (t) {
     case Float16: return "_Float16";
+    case BFloat16: return "__bf16";
     case Float32: return "float";
     case Float64: return "double";
     case Int8: return "int8_t";
@@ -48,7 +49,7 @@ const char* elem_c_type(TensorElemType t) {
 
 size_t elem_size(TensorElemType t) {
   switch (t) {
-    case Float16: case Int16: case UInt16: return 2;
+    case Float16: case BFloat16: case Int16: case UInt16: return 2;
     case Float32: case Int32: case UInt32: return 4;
     case Float64: case Int64: case UInt64: return 8;
     case Int8: case UInt8: return 1;
@@ -76,7 +77,7 @@ Expression::Expression(int c) : node_(constant(c, true)) {}
 static TensorElemType promote(TensorElemType a, TensorElemType b) {
   auto rank = [](TensorElemType t) {
     switch (t) {
-      case Float64: return 12; case Float32: return 11; case Float16: return 10;
+      case Float64: return 12; case Float32: return 11; case Float16: case BFloat16: return 10;
       case Int64: case UInt64: return 4; case Int32: case UInt32: return 3;
       case Int16: case UInt16: return 2; case Int8: case UInt8: return 1;
       default: return 0;
@@ -167,7 +168,7 @@ static NodePtr variable(TensorElemType t, std::string name) {
 }
 Variable::Variable(TensorElemType t, std::string name) : Expression(variable(t, std::move(name))) {}
 
-Const::Const(TensorElemType t, double v) : Expression(constant(v, t != Float16 && t != Float32 && t != Float64)) {
+Const::Const(TensorElemType t, double v) : Expression(constant(v, t != Float16 && t != BFloat16 && t != Float32 && t != Float64)) {
   node_->elem = t;
 }
 

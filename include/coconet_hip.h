@@ -262,6 +262,18 @@ int  ccn_bias_dropout_residual_ex(const float* acc, const float* const* partials
  *      any shape with N a multiple of 4, as for the fused call. ---- */
 int  ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream);
 
+/* ---- the same three calls with X, W, resid and out in IEEE half instead of bfloat16: the element type the reference's
+ *      model-parallel example declares (Float16, examples/model-parallel/model-parallel.cpp:10-15; its cublasGemmEx
+ *      multiplies CUDA_R_16F operands, src/codegen.cpp:1058-1136).  Products are accumulated in fp32 on the matrix
+ *      cores (v_mfma_f32_32x32x16_f16), where the reference accumulates in half. ---- */
+int  ccn_mlp_outproj_f16_ex(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                            const float* bias, const uint16_t* resid, uint16_t* out, int M, int N, int K,
+                            float p_drop, uint64_t seed, int dropout_mode, void* stream);
+int  ccn_bias_dropout_residual_f16_ex(const float* acc, const float* const* partials, int nPartials, const float* bias,
+                                      const uint16_t* resid, uint16_t* out, int M, int N, float p_drop, uint64_t seed,
+                                      int dropout_mode, size_t first_row, void* stream);
+int  ccn_matmul_f16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

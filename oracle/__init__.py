@@ -89,6 +89,8 @@ def _declare(L):
     L.orc_mlp_outproj.argtypes = [_vp, _vp, _pp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, C.c_uint64]
     L.orc_mlp_outproj_mode.restype = None
     L.orc_mlp_outproj_mode.argtypes = [_vp, _vp, _pp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, C.c_uint64, _i]
+    L.orc_mlp_outproj_typed.restype = None
+    L.orc_mlp_outproj_typed.argtypes = [_vp, _vp, _pp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, C.c_uint64, _i, _i]
     L.orc_epilogue_value.restype = _f
     L.orc_epilogue_value.argtypes = [_f, _f, _f, _i, _f, _i]
 
@@ -245,15 +247,16 @@ def epilogue_value(s, b, r, kept_inverted, p_drop, mode):
     return float(lib().orc_epilogue_value(s, b, r, int(kept_inverted), p_drop, mode))
 
 
-def mlp_outproj(X, W, partials, bias, resid, M, N, K, p_drop, seed, mode=0):
-    """X, W, resid: uint16 bf16 bit patterns. Returns (out_bf16_bits, out_f32).  mode: dropout form, 0 = standard."""
+def mlp_outproj(X, W, partials, bias, resid, M, N, K, p_drop, seed, mode=0, half=False):
+    """X, W, resid: uint16 bit patterns, bfloat16 or (half=True) IEEE half. Returns (out_bits, out_f32).
+    mode: dropout form, 0 = standard."""
     out = np.empty((M, N), np.uint16)
     outf = np.empty((M, N), np.float32)
     if partials:
         p, _k = _ptrs(partials, f32)
     else:
         p, _k = C.cast(None, _pp), None
-    lib().orc_mlp_outproj_mode(_ptr(X, u16), _ptr(W, u16), p, len(partials), _ptr(bias, f32),
-                               _ptr(resid, u16) if resid is not None else None, _ptr(out, u16), _ptr(outf, f32),
-                               M, N, K, p_drop, seed, mode)
+    lib().orc_mlp_outproj_typed(_ptr(X, u16), _ptr(W, u16), p, len(partials), _ptr(bias, f32),
+                                _ptr(resid, u16) if resid is not None else None, _ptr(out, u16), _ptr(outf, f32),
+                                M, N, K, p_drop, seed, mode, 1 if half else 0)
     return out, outf

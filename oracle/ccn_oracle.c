@@ -478,23 +478,34 @@ float orc_epilogue_value(float s, float b, float r, int kept_inverted, float p_d
   return sat01(sat01(v + b) + r);
 }
 
-void orc_mlp_outproj_mode(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
-                          const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
-                          int M, int N, int K, float p_drop, uint64_t seed, int mode) {
+/* half = 0: X, W, resid and out are bfloat16; half = 1: IEEE half (the type the reference's model-parallel example
+ * declares, examples/model-parallel/model-parallel.cpp:10-15).  Same arithmetic between the conversions. */
+void orc_mlp_outproj_typed(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                           const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                           int M, int N, int K, float p_drop, uint64_t seed, int mode, int half) {
   for (int i = 0; i < M; i++) {
     for (int j = 0; j < N; j++) {
       double acc = 0.0;
-      for (int k = 0; k < K; k++)
-        acc += (double)orc_bf16_to_f32(X[(size_t)i * K + k]) * (double)orc_bf16_to_f32(W[(size_t)k * N + j]);
+      for (int k = 0; k < K; k++) {
+        const uint16_t x = X[(size_t)i * K + k], w = W[(size_t)k * N + j];
+        acc += half ? (double)orc_f16_to_f32(x) * (double)orc_f16_to_f32(w) : (double)orc_bf16_to_f32(x) * (double)orc_bf16_to_f32(w);
+      }
       float s = (float)acc;
       size_t idx = (size_t)i * N + j;
       for (int q = 0; q < nPartials; q++) s = s + partials[q][idx];
       const int kept_inverted = orc_dropout_keep(seed, idx, p_drop);   /* u >= p; p = 0: always */
-      float y = orc_epilogue_value(s, bias[j], resid ? orc_bf16_to_f32(resid[idx]) : 0.0f, kept_inverted, p_drop, mode);
+      const float r = !resid ? 0.0f : (half ? orc_f16_to_f32(resid[idx]) : orc_bf16_to_f32(resid[idx]));
+      float y = orc_epilogue_value(s, bias[j], r, kept_inverted, p_drop, mode);
       if (out_f32) out_f32[idx] = y;
-      if (out) out[idx] = orc_f32_to_bf16(y);
+      if (out) out[idx] = half ? orc_f32_to_f16(y) : orc_f32_to_bf16(y);
     }
   }
+}
+
+void orc_mlp_outproj_mode(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                          const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                          int M, int N, int K, float p_drop, uint64_t seed, int mode) {
+  orc_mlp_outproj_typed(X, W, partials, nPartials, bias, resid, out, out_f32, M, N, K, p_drop, seed, mode, 0);
 }
 
 void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,

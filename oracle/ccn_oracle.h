@@ -114,6 +114,10 @@ void orc_mlp_outproj_mode(const uint16_t* X, const uint16_t* W, const float* con
 void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
                      const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
                      int M, int N, int K, float p_drop, uint64_t seed);
+/* the same with the 16-bit type as an argument: half = 0 bfloat16, 1 IEEE half */
+void orc_mlp_outproj_typed(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                           const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                           int M, int N, int K, float p_drop, uint64_t seed, int mode, int half);
 
 #ifdef __cplusplus
 }

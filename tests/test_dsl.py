@@ -60,6 +60,7 @@ def test_storage_classes_and_fusion_groups(dsl_build):
     ("mlp_two_dropouts", "must have the shape"),
     ("mlp_residual_before_dropout", "must have the shape"),
     ("mlp_no_collective", "must have the shape"),
+    ("mlp_mixed_types", "one 16-bit type"),
 ])
 def test_invalid_programs_abort_with_a_message(dsl_build, case, needle):
     """Error convention of the reference (src/ast.hpp:33-44): message on stderr, then std::terminate()."""
@@ -90,12 +91,18 @@ def test_matmul_chain_is_matched_by_structure_and_lowered_by_schedule(dsl_build,
     chk = os.path.join(dsl_build, "ccn-dsl-check")
     swapped = run(chk, "mlp_operands_swapped")
     assert swapped.returncode == 0, swapped.stderr
-    assert "ccn_matmul_bf16_f32(X, W, C" in swapped.stdout and "ccn_reduce_f32(tbl__, comm_size, C + off__" in swapped.stdout
-    assert "ccn_bias_dropout_residual_ex(C + off__, nullptr, 0, bias, R + off__, out + off__" in swapped.stdout
+    # Float16 tensors (what the reference's example declares) go to the library's IEEE-half calls
+    assert "ccn_matmul_f16_f32(X, W, C" in swapped.stdout and "ccn_reduce_f32(tbl__, comm_size, C + off__" in swapped.stdout
+    assert "ccn_bias_dropout_residual_f16_ex(C + off__, nullptr, 0, bias, R + off__, out + off__" in swapped.stdout
+    assert "ccn_gen::f32_to_f16_bits(" in swapped.stdout and "bf16" not in swapped.stdout.split("int main")[1]
     assert "const float p_drop = (float)0.5" in swapped.stdout
+    bf = run(chk, "mlp_bfloat16")        # the same chain declared in BFloat16: the bfloat16 calls
+    assert bf.returncode == 0, bf.stderr
+    assert "ccn_matmul_bf16_f32(X, W, C" in bf.stdout and "ccn_bias_dropout_residual_ex(C + off__, nullptr, 0" in bf.stdout
+    assert "ccn_gen::f32_to_bf16(" in bf.stdout and "_f16_" not in bf.stdout.split("int main")[1]
     plain = run(chk, "mlp_no_bias_no_dropout")
     assert plain.returncode == 0, plain.stderr
-    assert "ccn_bias_dropout_residual_ex(C + off__, tbl__, nPartials" in plain.stdout and "ccn_reduce_f32" not in plain.stdout
+    assert "ccn_bias_dropout_residual_f16_ex(C + off__, tbl__, nPartials" in plain.stdout and "ccn_reduce_f32" not in plain.stdout
     assert "hB[i] = 0.0f" in plain.stdout and "CCN_DROPOUT_INVERTED ? 0.0f : 1.0f" in plain.stdout
     prog = os.path.join(dsl_build, "ccn-programs")
     texts = {}
@@ -247,12 +254,13 @@ def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path)
     assert "off__" not in arc and "ccn_reduce_f32(g, comm_size, g[0], (size_t)N" in arc     # Replicated: the whole range
     # the model-parallel example: unfused schedules as separate steps, the overlapped one as the one fused kernel
     mlp = (tmp_path / "model-parallel-mm-ar-c.hip").read_text()
-    assert "ccn_matmul_bf16_f32" in mlp and "ccn_bias_dropout_residual_ex" in mlp and "p_drop = (float)0.5" in mlp
-    assert "ccn_mlp_outproj_bf16" not in mlp and "MatMul: %f, AllReduce: %f, kernel0: %f, Total" in mlp
+    # (the example declares Float16: the library's IEEE-half calls)
+    assert "ccn_matmul_f16_f32" in mlp and "ccn_bias_dropout_residual_f16_ex" in mlp and "p_drop = (float)0.5" in mlp
+    assert "ccn_mlp_outproj_" not in mlp and "MatMul: %f, AllReduce: %f, kernel0: %f, Total" in mlp
     rs = (tmp_path / "model-parallel-mm-rs-c-ag.hip").read_text()
     assert "MatMul: %f, ReduceScatter: %f, kernel0: %f, AllGather: %f, Total" in rs and "ccn_memcpy_d2d(out + off__, scOut + off__" in rs
     ol = (tmp_path / "model-parallel-ol-mm-fuse-rs-c-ag.hip").read_text()
-    assert "ccn_mlp_outproj_bf16_ex" in ol and "MatMulFused: %f" in ol
+    assert "ccn_mlp_outproj_f16_ex" in ol and "MatMulFused: %f" in ol
 
 
 @pytest.mark.skipif(not os.path.exists(os.path.join(ROOT, "oracle", "_ref", "ref-adam")), reason="oracle/_ref not built")

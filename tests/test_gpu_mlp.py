@@ -93,6 +93,89 @@ def test_plain_product_of_any_shape(ccn, M, N, K):
     assert np.all(np.abs(Cd.cpu().numpy().astype(np.float64) - xf @ wf) <= bound + 1e-30)
 
 
+def u16_dev(bits):
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(DEV)
+
+
+def f16_ulp_distance(a, b):
+    def key(x):
+        x = x.astype(np.int32)
+        return np.where(x & 0x8000, -(x & 0x7fff), x)
+    return np.abs(key(a) - key(b))
+
+
+@pytest.mark.parametrize("M,N,K,nP,p,mode", [(128, 128, 64, 7, 0.1, 0), (256, 384, 192, 3, 0.3, 0), (128, 256, 1024, 7, 0.5, 1),
+                                              (256, 128, 128, 2, 0.25, 2), (128, 128, 64, 1, 0.5, 3), (100, 36, 70, 7, 0.1, 0),
+                                              (1, 4, 1, 0, 0.0, 0)])
+def test_outproj_in_ieee_half(ccn, M, N, K, nP, p, mode):
+    """X, W, resid and out in IEEE half (ccn_mlp_outproj_f16_ex): the element type the reference's model-parallel example
+    declares.  Same bar as for bfloat16, with the unit in the last place of a half: the fp32 accumulation order differs
+    from the oracle's float64 sum, so an output may land on the neighbouring half where the error straddles a
+    rounding boundary."""
+    r = rng(130 + nP)
+    X = r.standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    W = (r.standard_normal((K, N)) * 0.02).astype(np.float16).view(np.uint16)
+    parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N, dtype=np.float32)
+    resid = r.standard_normal((M, N)).astype(np.float16).view(np.uint16)
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(u16_dev(X), u16_dev(W), [torch.from_numpy(q).to(DEV) for q in parts], torch.from_numpy(bias).to(DEV),
+                         u16_dev(resid), out, M, N, K, p, 9, dropout_mode=mode, half=True)
+    got = bf16_host(out).reshape(M, N)
+    want, want_f32 = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, p, 9, mode=mode, half=True)
+    d = f16_ulp_distance(got, want)
+    # A half has 3 more mantissa bits than a bfloat16, so the same fp32 error crosses a rounding boundary 8 times as
+    # often; and where the dropped-and-scaled sum cancels against the residual the result is small while the error of the
+    # fp32 sum is not (a half resolves 6e-8 near zero), so "one ulp" is the bar only away from cancellation.  Everywhere:
+    # the error is within what an fp32 sum of K products and nP + 3 terms of these magnitudes may have, plus the rounding
+    # to half.
+    assert (d > 0).mean() < 0.08, f"{(d > 0).mean():.4f} of the outputs differ"
+    assert (d > 1).mean() < 0.002, f"{(d > 1).mean():.5f} of the outputs differ by more than one ulp"
+    xf, wf = X.view(np.float16).astype(np.float64), W.view(np.float16).astype(np.float64)
+    scale = 1.0 / (1.0 - p) if mode == 0 else 1.0
+    mag = (np.abs(xf) @ np.abs(wf) + sum(np.abs(q).astype(np.float64) for q in parts) + np.abs(bias)) * scale \
+        + np.abs(resid.view(np.float16).astype(np.float64))
+    gf = got.view(np.float16).astype(np.float64)
+    ulp = np.spacing(np.abs(want_f32).astype(np.float16)).astype(np.float64)
+    assert np.all(np.abs(gf - want_f32) <= (K + nP + 4) * 2.0 ** -24 * mag + ulp)
+    if mode == 0:
+        keep = orc.dropout_mask(9, 0, M * N, p).reshape(M, N).astype(bool)
+        assert np.array_equal(got[~keep], resid[~keep])
+
+
+def test_half_product_and_standalone_epilogue(ccn):
+    """ccn_matmul_f16_f32 against float64 within the fp32 accumulation bound, all-ones C == K, and the standalone epilogue
+    in half bit for bit against the oracle's per-element routine."""
+    M, N, K = 256, 128, 192
+    r = rng(140)
+    Xh = r.standard_normal((M, K)).astype(np.float16)
+    Wh = (r.standard_normal((K, N)) * 0.02).astype(np.float16)
+    Cd = torch.full((M, N), -1.0, device=DEV)
+    ccn.matmul_bf16_f32(u16_dev(Xh.view(np.uint16)), u16_dev(Wh.view(np.uint16)), Cd, M, N, K, half=True)
+    torch.cuda.synchronize()
+    xf, wf = Xh.astype(np.float64), Wh.astype(np.float64)
+    bound = K * 2.0 ** -24 * (np.abs(xf) @ np.abs(wf))
+    assert np.all(np.abs(Cd.cpu().numpy().astype(np.float64) - xf @ wf) <= bound + 1e-30)
+    ones = lambda shape: u16_dev(np.ones(shape, np.float16).view(np.uint16))
+    ccn.matmul_bf16_f32(ones((M, K)), ones((K, N)), Cd, M, N, K, half=True)
+    torch.cuda.synchronize()
+    assert torch.all(Cd == K)
+    acc = r.standard_normal((M, N), dtype=np.float32)
+    parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(2)]
+    bias = r.standard_normal(N, dtype=np.float32)
+    resid = r.standard_normal((M, N)).astype(np.float16)
+    for mode in (0, 1, 2, 3):
+        out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+        ccn.bias_dropout_residual(torch.from_numpy(acc).to(DEV), [torch.from_numpy(q).to(DEV) for q in parts],
+                                  torch.from_numpy(bias).to(DEV), u16_dev(resid.view(np.uint16)), out, M, N, 0.3, 7,
+                                  dropout_mode=mode, half=True)
+        s = (acc + parts[0]) + parts[1]
+        kept = orc.dropout_mask(7, 0, M * N, 0.3).reshape(M, N)
+        y = np.array([[orc.epilogue_value(s[i, j], bias[j], np.float32(resid[i, j]), int(kept[i, j]), 0.3, mode)
+                       for j in range(N)] for i in range(M)], np.float32)
+        assert np.array_equal(bf16_host(out).reshape(M, N), y.astype(np.float16).view(np.uint16)), mode
+
+
 def test_outproj_all_ones_known_answer(ccn):
     # the reference's own check at this boundary: all-ones operands give C == K*ranks
     # (nccl-overlap/samples/matmul-allreduce-bias-dropout-layernorm.cu:520-526)

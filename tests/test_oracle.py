@@ -420,6 +420,33 @@ def test_mlp_outproj_float64_brute_force_and_all_ones():
     assert np.all(outf == K * 8)
 
 
+def test_mlp_outproj_in_ieee_half():
+    """The same routine with X, W, resid and out in IEEE half (the type of the reference's model-parallel example):
+    float64 brute force over numpy's own float16 values, the output rounded by numpy's float16 cast, and the
+    reference's all-ones check."""
+    M, N, K, nP = 8, 12, 16, 3
+    r = rng(11)
+    Xh = r.standard_normal((M, K)).astype(np.float16)
+    Wh = (r.standard_normal((K, N)) * 0.02).astype(np.float16)
+    Rh = r.standard_normal((M, N)).astype(np.float16)
+    parts = [r.standard_normal((M, N)).astype(np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N).astype(np.float32)
+    out, outf = orc.mlp_outproj(Xh.view(np.uint16), Wh.view(np.uint16), parts, bias, Rh.view(np.uint16), M, N, K, 0.1, 0,
+                                half=True)
+    s = Xh.astype(np.float64) @ Wh.astype(np.float64) + np.sum(np.stack(parts).astype(np.float64), axis=0) + bias
+    keep = orc.dropout_mask(0, 0, M * N, 0.1).reshape(M, N).astype(bool)
+    y = np.where(keep, s / 0.9, 0.0) + Rh.astype(np.float64)
+    assert np.max(np.abs(outf - y)) < 1e-5
+    assert np.array_equal(out, outf.astype(np.float16).view(np.uint16))
+    # the two 16-bit types give different answers on the same bits: the argument is not ignored
+    out_b, _ = orc.mlp_outproj(Xh.view(np.uint16), Wh.view(np.uint16), parts, bias, Rh.view(np.uint16), M, N, K, 0.1, 0)
+    assert not np.array_equal(out, out_b)
+    ones = lambda shape: np.ones(shape, np.float16).view(np.uint16)
+    parts1 = [np.full((M, N), K, np.float32) for _ in range(7)]
+    o, outf = orc.mlp_outproj(ones((M, K)), ones((K, N)), parts1, np.zeros(N, np.float32), None, M, N, K, 0.0, 0, half=True)
+    assert np.all(outf == K * 8) and np.all(o.view(np.float16) == K * 8)
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # the modified NCCL's global-norm LAMB arithmetic (mode 2)
 # ---------------------------------------------------------------------------------------------------------------------
