@@ -224,6 +224,45 @@ def test_standalone_epilogue_bit_exact(ccn, M, N, nP, p):
     assert np.array_equal(bf16_host(out).reshape(M, N), orc.f32_to_bf16(y.astype(np.float32)))
 
 
+def test_outproj_config5_shape_in_ieee_half(ccn):
+    """The shape of benchmark configuration 5 with the operands, residual and output in IEEE half: mask exact on sampled
+    rows, drop rate over all 2^26 outputs, values within the fp32-sum bound plus the rounding to half."""
+    M = N = 8192
+    K = 1024
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(6)
+    X = torch.randn(M, K, device=DEV, generator=gen).to(torch.float16)
+    W = (torch.randn(K, N, device=DEV, generator=gen) * 0.02).to(torch.float16)
+    parts = [torch.randn(M, N, device=DEV, generator=gen) for _ in range(7)]
+    bias = torch.randn(N, device=DEV, generator=gen)
+    resid = torch.randn(M, N, device=DEV, generator=gen).to(torch.float16)
+    out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    ccn.mlp_outproj_bf16(X, W, parts, bias, resid, out, M, N, K, 0.1, 0, dropout_mode=0, half=True)
+    torch.cuda.synchronize()
+    rows = [0, 1, 127, 128, 4095, 4096, 8191]
+    keep_rows = np.stack([orc.dropout_mask(0, r * N, N, 0.1) for r in rows]).astype(bool)
+    xf = X[rows].cpu().numpy().astype(np.float64)
+    wf = W.cpu().numpy().astype(np.float64)
+    ph = [q[rows].cpu().numpy() for q in parts]
+    rh = resid[rows].cpu().numpy()
+    got = out[rows].cpu().numpy()
+    s = (xf @ wf).astype(np.float32)
+    for q in ph:
+        s = s + q
+    t = s + bias.cpu().numpy()[None, :]
+    scale = np.float32(1.0) / (np.float32(1.0) - np.float32(0.1))
+    y = np.where(keep_rows, t * scale, np.float32(0)) + rh.astype(np.float32)
+    assert np.array_equal(got[~keep_rows].view(np.uint16), rh[~keep_rows].view(np.uint16))
+    mag = (np.abs(xf) @ np.abs(wf) + sum(np.abs(q).astype(np.float64) for q in ph) + np.abs(bias.cpu().numpy())) * float(scale) \
+        + np.abs(rh.astype(np.float64))
+    ulp = np.spacing(np.abs(y).astype(np.float16)).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - y) <= (K + 11) * 2.0 ** -24 * mag + ulp)
+    d = f16_ulp_distance(got.view(np.uint16), y.astype(np.float16).view(np.uint16))
+    assert (d > 1).mean() < 0.002 and (d > 0).mean() < 0.08
+    dropped = float((out == resid).float().mean())
+    assert abs(dropped - 0.1) < 2e-3
+
+
 def test_outproj_config5_full_size(ccn):
     """benchmark configuration 5 at full size (8192 x 1024 x 8192, 7 partials, p = 0.1, seed 0).  Checked by:
     the exact dropout mask over all 2^26 outputs (torch recomputes nothing: dropped outputs equal the
