@@ -420,6 +420,9 @@ LAMB_VARIANTS = {
     "deferred": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0"},
     "deferred-wave": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0", "CCN_LAMB_RES_BLOCK": "64"},
     "two-pass": {"CCN_LAMB_RESIDENT": "0"},
+    # a patience of a poll or two: some tiles see their segment's scale in time, the others go to the trailing kernel
+    "one-tile-short-patience": {"CCN_LAMB_SPIN": "6"},
+    "resident-short-patience": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "3"},
     # the workgroup that adds a segment up keeps the result to itself, as it does when a tile sum has not arrived: every
     # tile runs out of patience and the trailing kernel adds the segments up from the sums in memory
     "one-tile-withheld": {"CCN_LAMB_WITHHOLD": "1", "CCN_LAMB_SPIN": "8"},
