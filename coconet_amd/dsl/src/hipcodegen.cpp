@@ -566,9 +566,22 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   const std::string rank_loop =
       "  for (int r_ = rank < 0 ? 0 : rank; r_ < (rank < 0 ? comm_size : rank + 1); r_++) {\n";
   auto slice_of = [&](const std::string& count) {
-    return "  const size_t per__ = DIVUP((size_t)(" + count + "), (size_t)comm_size), off__ = per__ * (size_t)r_;\n"
-           "  if (off__ >= (size_t)(" + count + ")) continue;\n"
-           "  const size_t cnt__ = off__ + per__ <= (size_t)(" + count + ") ? per__ : (size_t)(" + count + ") - off__;\n";
+    return "  const size_t n__ = " + count + ", per__ = DIVUP(n__, (size_t)comm_size), off__ = per__ * (size_t)r_;\n"
+           "  if (off__ >= n__) continue;\n"
+           "  const size_t cnt__ = off__ + per__ <= n__ ? per__ : n__ - off__;\n";
+  };
+  // the body of a rank loop, one level deeper
+  auto deeper = [](const std::string& text) {
+    std::string out;
+    size_t at = 0;
+    while (at < text.size()) {
+      const size_t nl = text.find('\n', at);
+      const std::string line = text.substr(at, nl == std::string::npos ? std::string::npos : nl - at + 1);
+      out += (line == "\n" ? "" : "  ") + line;
+      if (nl == std::string::npos) break;
+      at = nl + 1;
+    }
+    return out;
   };
 
   o << "void " << fn << "(" << sig(true) << ") {\n";
@@ -580,42 +593,52 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
     if (st.type == Step::Reduce && !st.sliced) {
       o << "  CCNCHECK(ccn_reduce_f32(" << st.src << ", comm_size, " << st.dst << ", " << st.count << ", stream));\n";
     } else if (st.type == Step::Reduce) {
-      o << rank_loop << slice_of(st.count);
-      o << "  const float* tbl__[ccn_gen::kMaxRanks];\n";
-      o << "  for (int p_ = 0; p_ < comm_size; p_++) tbl__[p_] = " << st.src << "[p_] + off__;\n";
-      o << "  CCNCHECK(ccn_reduce_f32(tbl__, comm_size, " << st.dst << " + off__, cnt__, stream));\n  }\n";
+      o << rank_loop
+        << deeper(slice_of(st.count) + "  const float* tbl__[ccn_gen::kMaxRanks];\n" +
+                  "  for (int p_ = 0; p_ < comm_size; p_++) tbl__[p_] = " + st.src + "[p_] + off__;\n" +
+                  "  CCNCHECK(ccn_reduce_f32(tbl__, comm_size, " + st.dst + " + off__, cnt__, stream));\n")
+        << "  }\n";
     } else if (st.type == Step::Copy && !st.sliced) {
       o << "  CCNCHECK(ccn_memcpy_d2d(" << st.dst << ", " << st.src << ", (" << st.count << ") * sizeof(float), stream));\n";
     } else if (st.type == Step::Copy) {
-      o << rank_loop << slice_of(st.count);
-      o << "  CCNCHECK(ccn_memcpy_d2d(" << st.dst << " + off__, " << st.src << " + off__, cnt__ * sizeof(float), stream));\n  }\n";
+      o << rank_loop
+        << deeper(slice_of(st.count) + "  CCNCHECK(ccn_memcpy_d2d(" + st.dst + " + off__, " + st.src +
+                  " + off__, cnt__ * sizeof(float), stream));\n")
+        << "  }\n";
     } else if (st.type == Step::Kernel) {
       const std::string a = "args" + std::to_string(argNo++);
       if (!st.sliced) {
-        o << "  {\n" << fill_args(st.body, a, st.count, "") << "  ccn_gen::launch(" << a << ", stream);\n  }\n";
+        o << "  {\n" << deeper(fill_args(st.body, a, st.count, "") + "  ccn_gen::launch(" + a + ", stream);\n") << "  }\n";
       } else {
-        o << rank_loop << slice_of(st.count) << fill_args(st.body, a, "cnt__", "off__") << "  ccn_gen::launch(" << a
-          << ", stream);\n  }\n";
+        o << rank_loop << deeper(slice_of(st.count) + fill_args(st.body, a, "cnt__", "off__") + "  ccn_gen::launch(" + a + ", stream);\n")
+          << "  }\n";
       }
     } else if (!st.sliced) {
       const std::string a = "args" + std::to_string(argNo++), b = "args" + std::to_string(argNo++);
-      o << "  {\n" << fill_args(st.body, a, st.count, "") << "  const unsigned blocks__ = ccn_gen::launch(" << a << ", stream);\n";
-      o << "  ccn_gen::finalize_norms(partials__, partials__ + (size_t)ccn_gen::blocks_for(" << st.count << ") * 8, blocks__, "
+      std::ostringstream q;
+      q << fill_args(st.body, a, st.count, "") << "  const unsigned blocks__ = ccn_gen::launch(" << a << ", stream);\n";
+      q << "  ccn_gen::finalize_norms(partials__, partials__ + (size_t)ccn_gen::blocks_for(" << st.count << ") * 8, blocks__, "
         << st.body.nacc << ", " << st.body.sqrtMask << "u, norms__, stream);\n";
-      o << fill_args(st.body2, b, st.count, "") << "  ccn_gen::launch(" << b << ", stream);\n  }\n";
+      q << fill_args(st.body2, b, st.count, "") << "  ccn_gen::launch(" << b << ", stream);\n";
+      o << "  {\n" << deeper(q.str()) << "  }\n";
     } else {
       // Norms over Sliced values span every rank's slice (the reference all-reduces them): pass 1 on every slice, each
       // launch's partial sums behind the previous one's, one finalize over all of them, then pass 2 on every slice.
       const std::string a = "args" + std::to_string(argNo++), b = "args" + std::to_string(argNo++);
       o << "  if (rank >= 0 && comm_size > 1) { printf(\"this pipeline's norms span all slices: call with rank = -1\\n\"); exit(EXIT_FAILURE); }\n";
-      o << "  {\n  unsigned rows__ = 0;\n";
-      o << rank_loop << slice_of(st.count) << fill_args(st.body, a, "cnt__", "off__");
-      o << "  " << a << ".partials = partials__ + (size_t)rows__ * " << st.body.nacc << ";\n";
-      o << "  rows__ += ccn_gen::launch(" << a << ", stream);\n  }\n";
-      o << "  ccn_gen::finalize_norms(partials__, partials__ + (size_t)ccn_gen::blocks_for(" << st.count << ") * 8, rows__, "
+      std::ostringstream q;
+      q << "  unsigned rows__ = 0;\n";
+      q << rank_loop
+        << deeper(slice_of(st.count) + fill_args(st.body, a, "cnt__", "off__") + "  " + a +
+                  ".partials = partials__ + (size_t)rows__ * " + std::to_string(st.body.nacc) + ";   // behind the previous slice's\n" +
+                  "  rows__ += ccn_gen::launch(" + a + ", stream);\n")
+        << "  }\n";
+      q << "  ccn_gen::finalize_norms(partials__, partials__ + (size_t)ccn_gen::blocks_for(" << st.count << ") * 8, rows__, "
         << st.body.nacc << ", " << st.body.sqrtMask << "u, norms__, stream);\n";
-      o << rank_loop << slice_of(st.count) << fill_args(st.body2, b, "cnt__", "off__") << "  ccn_gen::launch(" << b
-        << ", stream);\n  }\n  }\n";
+      q << rank_loop
+        << deeper(slice_of(st.count) + fill_args(st.body2, b, "cnt__", "off__") + "  ccn_gen::launch(" + b + ", stream);\n")
+        << "  }\n";
+      o << "  {\n" << deeper(q.str()) << "  }\n";
     }
     o << "  CCNCHECK(ccn_event_record(stop__, stream));\n";
     o << "  CCNCHECK(ccn_event_elapsed_ms(start__, stop__, &elapsedTime));\n";

@@ -248,7 +248,7 @@ def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path)
     unf = (tmp_path / "adam-rs-c-ag.hip").read_text()
     # ReduceScatter, kernel, AllGather, each on the rank's slice: every array moved on by DIVUP(N, comm_size) * rank
     assert "ccn_reduce_f32(tbl__, comm_size, g[0] + off__, cnt__" in unf and "ccn_memcpy_d2d(w + off__, S5 + off__, cnt__" in unf
-    assert "per__ = DIVUP((size_t)((size_t)N), (size_t)comm_size), off__ = per__ * (size_t)r_" in unf
+    assert "n__ = (size_t)N, per__ = DIVUP(n__, (size_t)comm_size), off__ = per__ * (size_t)r_" in unf
     assert "args0.in[0] = m + off__" in unf and "args0.n = cnt__" in unf and "int comm_size, int rank" in unf
     arc = (tmp_path / "adam-ar-c.hip").read_text()
     assert "off__" not in arc and "ccn_reduce_f32(g, comm_size, g[0], (size_t)N" in arc     # Replicated: the whole range
