@@ -18,7 +18,8 @@
  *   orc_sgd_f32           examples/test-sgd.cu:17-18; numpy axpy identity       pinned
  *   orc_sgd_axpby_f32     nccl-overlap/samples/single-process-wX.cu:141        pinned (numpy identity)
  *   orc_pseudo_adam_f32   examples/test-adam.cu:14-38; known answer w=-1/P      pinned
- *   orc_fused_adam_a3     nccl/.../reduce_kernel.h:36-68 functors; known answer w=-1, half 0xBC00   pinned
+ *   orc_fused_adam_a3     nccl/.../reduce_kernel.h:36-68 functors; known answer w=-1, half 0xBC00; two steps by hand at
+ *                         beta1 != beta2 (the first moment decays with beta2, common_kernel.h:878)          pinned
  *   orc_adam_f32          nccl-overlap/samples/multi-process-adam-scattered.cpp:112-136;
  *                         reference integer fixture, torch.optim.Adam (CPU) cross-check, step-1 closed form   pinned
  *   orc_lamb_f32          same file :402-449; single-segment/w==0 special cases, float64 brute force  pinned
@@ -33,6 +34,11 @@
  *   orc_mlp_outproj       no reference test beyond the all-ones C == K check
  *                         (nccl-overlap/samples/matmul-allreduce-bias-dropout-layernorm.cu:520-526);
  *                         float64 brute force; dropout mask build-defined ("parity unpinned" vs cuRAND)
+ *   orc_epilogue_value,   the four dropout forms (src/codegen.cpp:634-640; nccl-overlap/.../reduce_kernel.h:192-213):
+ *   orc_mlp_outproj_mode  closed forms at p = 0 and p = 1, complementary survivors at p = 0.3, saturating cases by hand   pinned
+ *                         (the uniform draws themselves: "parity unpinned" vs cuRAND)
+ *   orc_mlp_outproj_typed the same routine on IEEE-half operands: float64 brute force over numpy's float16 values, numpy's
+ *                         float16 cast of the result, the reference's all-ones check                          pinned
  */
 #ifndef CCN_ORACLE_H
 #define CCN_ORACLE_H
