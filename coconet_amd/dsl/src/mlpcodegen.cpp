@@ -1,4 +1,6 @@
-// Lowering of the model-parallel MLP pipeline (examples/model-parallel/model-parallel.cpp of the reference):
+// Lowering of the model-parallel MLP pipeline (examples/model-parallel/model-parallel.cpp of the reference; the
+// programs of examples/pipeline-parallel/pipeline-parallel.cpp are the same chain without bias and dropout, and what
+// they hand to the next pipeline stage is the output this rank computes):
 //
 //   layer = MatMul(in, w);  sum = AllReduce | ReduceScatter (layer);  [sum2 = sum + b;]  [Dropout(., p)]  [+ r | + Scatter(r)]
 //   [out = AllGather(.)]
@@ -196,7 +198,8 @@ std::string generateMLP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
                    : (level == 1 ? "the product, then one kernel for the sum over ranks and what follows it"
                                  : "the product, the sum over ranks and the pointwise part as separate steps"))
     << ".\n";
-  o << "// 16-bit tensors of the program are held as bfloat16; the product accumulates in fp32.\n";
+  o << "// 16-bit tensors keep the program's type (" << (c.in->elem == Float16 ? "Float16: IEEE half" : "BFloat16")
+    << "); the product accumulates in fp32.\n";
   o << "// Run:   ./a.out <epochs> [ranks=8] [check=1] [untimed_warmup_epochs=0]\n";
   o << "// Environment: CCN_GEN_<dimension>=<n> replaces the sizes of a dimension variable; CCN_GEN_DROPOUT_MODE=0..3 the\n"
        "//        dropout form (CCN_DROPOUT_* of coconet_hip.h).\n";

@@ -235,14 +235,15 @@ def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path)
     schedule produces a program."""
     for ex, schedules in [("sgd", ["AR_C", "RS_C_AG", "fuse_RS_C_AG"]), ("adam", ["AR_C", "RS_C_AG", "fuse_RS_C_AG"]),
                           ("lamb", ["AR_C", "RS_C_AG", "fuse_RS_C_AG"]),
-                          ("model-parallel", ["MM_AR_C", "MM_RS_C_AG", "ol_MM_fuse_RS_C_AG"])]:
+                          ("model-parallel", ["MM_AR_C", "MM_RS_C_AG", "ol_MM_fuse_RS_C_AG"]),
+                          ("pipeline-parallel", ["AR_P2P_C", "RS_P2P_C_AG", "ol_RS_fuse_P2P_C_AG"])]:
         exe = os.path.join(dsl_build, "ex-" + ex)
         assert os.path.exists(exe), exe
         for s in schedules:
             r = run(exe, s, cwd=tmp_path)
             assert r.returncode == 0, r.stderr
     made = sorted(f for f in os.listdir(tmp_path) if f.endswith(".hip"))
-    assert len(made) == 12 and "adam-fuse-rs-c-ag.hip" in made
+    assert len(made) == 15 and "adam-fuse-rs-c-ag.hip" in made
     fused = (tmp_path / "adam-fuse-rs-c-ag.hip").read_text()
     assert "HAS_RED = true" in fused and "ccn_memcpy_d2d" not in fused       # RS + compute + AG in one kernel
     unf = (tmp_path / "adam-rs-c-ag.hip").read_text()
@@ -261,6 +262,14 @@ def test_reference_examples_compile_unmodified_and_generate(dsl_build, tmp_path)
     assert "MatMul: %f, ReduceScatter: %f, kernel0: %f, AllGather: %f, Total" in rs and "ccn_memcpy_d2d(out + off__, scOut + off__" in rs
     ol = (tmp_path / "model-parallel-ol-mm-fuse-rs-c-ag.hip").read_text()
     assert "ccn_mlp_outproj_f16_ex" in ol and "MatMulFused: %f" in ol
+    # the pipeline-parallel example: the same chain with neither bias nor dropout (every element kept), residual added
+    pp = (tmp_path / "pipeline-parallel-ar-p2p-c.hip").read_text()
+    assert "MatMul: %f, AllReduce: %f, kernel0: %f, Total" in pp and "ccn_matmul_f16_f32" in pp
+    assert "no Dropout in the pipeline" in pp and "hB[i] = 0.0f" in pp and "bias, R + off__" in pp
+    pprs = (tmp_path / "pipeline-parallel-rs-p2p-c-ag.hip").read_text()
+    assert "MatMul: %f, ReduceScatter: %f, kernel0: %f, AllGather: %f, Total" in pprs
+    ppol = (tmp_path / "pipeline-parallel-ol-rs-fuse-p2p-c-ag.hip").read_text()
+    assert "ccn_mlp_outproj_f16_ex(X, W, partials.data(), nPartials, bias, R, out" in ppol
 
 
 @pytest.mark.skipif(not os.path.exists(os.path.join(ROOT, "oracle", "_ref", "ref-adam")), reason="oracle/_ref not built")

@@ -166,13 +166,17 @@ def test_the_emitted_check_catches_a_wrong_result():
 
 MLP_STEPS = {"ref-model-parallel-mm-ar-c": {"MatMul", "AllReduce", "kernel0"},
              "ref-model-parallel-mm-rs-c-ag": {"MatMul", "ReduceScatter", "kernel0", "AllGather"},
-             "ref-model-parallel-ol-mm-fuse-rs-c-ag": {"MatMulFused"}}
+             "ref-model-parallel-ol-mm-fuse-rs-c-ag": {"MatMulFused"},
+             "ref-pipeline-parallel-ar-p2p-c": {"MatMul", "AllReduce", "kernel0"},
+             "ref-pipeline-parallel-rs-p2p-c-ag": {"MatMul", "ReduceScatter", "kernel0", "AllGather"},
+             "ref-pipeline-parallel-ol-rs-fuse-p2p-c-ag": {"MatMulFused"}}
 
 
 @pytest.mark.parametrize("name", list(MLP_STEPS))
 def test_model_parallel_programs(name):
     """Every schedule of the reference's examples/model-parallel/model-parallel.cpp (the last one has no bias and no
-    dropout in its expression): the unfused ones run the product, the sum over ranks and the pointwise part as separate
+    dropout in its expression) and of examples/pipeline-parallel/pipeline-parallel.cpp (product, sum over ranks and
+    residual; what that example sends on to the next pipeline stage is this output): the unfused ones run the product, the sum over ranks and the pointwise part as separate
     steps (rank by rank on bands of rows after the ReduceScatter), the overlapped one as the one fused kernel; each
     emitted program checks its result against its own CPU re-execution."""
     rows = run_program(name, 2, 8, 1)
