@@ -145,12 +145,14 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {   // round-to-nea
   return __builtin_bit_cast(uint16_t, x);
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {  // round-to-nearest-even, quiet nan
-  uint32_t x = __float_as_uint(f);
-  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
-  x += 0x7fffu + ((x >> 16) & 1u);
-  return (uint16_t)(x >> 16);
+// round-to-nearest-even, quiet nan; the rounded word with the bfloat16 in its upper half (selects, no branch: the
+// epilogues convert four values per quad and stay one basic block)
+__device__ __forceinline__ uint32_t f32_to_bf16_hi(float f) {
+  const uint32_t x = __float_as_uint(f);
+  const uint32_t r = x + 0x7fffu + ((x >> 16) & 1u);
+  return f != f ? (x | 0x00400000u) : r;
 }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return (uint16_t)(f32_to_bf16_hi(f) >> 16); }
 
 // ---- Philox-4x32-10, and the dropout keep decision built on it -----------------------------------------------------
 struct Philox4 { uint32_t x, y, z, w; };
@@ -173,6 +175,14 @@ __host__ __device__ __forceinline__ bool keep_from_word(uint32_t word, float p_d
   const float u = (float)(word >> 8) * 5.9604644775390625e-08f;
   return u >= p_drop;
 }
+// The same decision on integers: u = k * 2^-24 with k = word >> 8 is exact, so u >= p  <=>  k >= ceil(p * 2^24)
+// (p * 2^24 is exact in double).  The host computes the threshold once per launch; 2^24 (p = 1) means "never".
+inline uint32_t keep_threshold(float p_drop) {
+  const double t = (double)p_drop * 16777216.0;
+  const double c = (double)(uint64_t)t;
+  return (uint32_t)(c < t ? c + 1.0 : c);
+}
+__device__ __forceinline__ bool keep_from_threshold(uint32_t word, uint32_t thr) { return (word >> 8) >= thr; }
 
 // ---- launch geometry for streaming kernels ----------------------------------------------------------------------------
 // Number of workgroups for a grid-stride kernel whose workgroup consumes `tile` units per iteration

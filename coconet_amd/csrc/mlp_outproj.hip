@@ -2,14 +2,13 @@
 // dropout and residual fused into the tile write-back, plus the same epilogue as a standalone kernel.
 //
 // GEMM tiling: a 256-thread workgroup owns a 128(m) x 128(n) tile of C and walks K in steps of 64.
-// The four wavefronts form a 2x2 grid; each owns 64x64 as 2x2 v_mfma_f32_32x32x16_bf16 blocks.
-// The MFMA computes C^T blocks (rows = n from W, columns = m from X) so that every lane ends up with
-// four CONSECUTIVE n of one row m in its accumulator quads: the epilogue then moves 16-byte pieces of
-// the fp32 partial buffers and 8-byte pieces of the bf16 residual/output.
+// Wavefront w owns the 32 tile rows 8j + 2w, 8j + 2w + 1 (j = 0..15) over all 128 columns, as four
+// v_mfma_f32_32x32x16_bf16 blocks.  The MFMA computes C^T blocks (rows = n from W, columns = m from X)
+// so that every lane ends up with four CONSECUTIVE n of one row m in its accumulator quads.
 // W is [K x N] row-major (n contiguous) while the MFMA wants k contiguous per lane, so the W tile is
 // transposed in registers on its way into LDS.  LDS rows are 128 bytes (64 k) with the eight 16-byte
 // chunks XOR-swizzled by (row%8)^((row/8)%8): conflict-free for the 8-byte transposed writes and the
-// 16-byte fragment reads.
+// 16-byte fragment reads (also with the rows a wavefront owns: they differ in row/8).
 #include "ccn_common.hpp"
 
 #include <type_traits>
@@ -24,6 +23,7 @@ constexpr int BM = 128, BN = 128, BK = 64;
 
 struct EpiPrm {
   float p_drop, keep_scale;
+  uint32_t thr;   // keep_threshold(p_drop): an element survives standard dropout when (word >> 8) >= thr
   uint32_t seed_lo, seed_hi;
   int apply_dropout;
   int mode;   // CCN_DROPOUT_*
@@ -52,226 +52,252 @@ __device__ __forceinline__ void epilogue_load(EpiIn<NP>& in, const SrcTable<floa
 // [0, 1] clamp of the reference's __hadd2_sat (NaN gives 0)
 __device__ __forceinline__ float sat01(float x) { return x > 0.0f ? (x < 1.0f ? x : 1.0f) : 0.0f; }
 
-// idx: where the quad lies in memory; mask_idx: its element index in the whole [M x N] output, which the mask is drawn
-// from (the two differ when a call covers a band of rows of a larger output).
+// Two 16-bit halves into one word: the upper halves of lo and hi (lo in bits 0-15)
+__device__ __forceinline__ uint32_t pack_upper_halves(uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); }
+
+// The four finished 16-bit outputs of a quad.  mask_idx: the quad's element index in the whole [M x N] output, which
+// the mask is drawn from; bv: the bias of the quad's four columns.
 // REF: one of the reference's dropout forms (k.mode says which); false: standard dropout, the form the kernels are
 // tuned for, compiled without the others.
+// The quad's four draws as a mask: bit e is set where u >= p for element e (the element survives standard dropout; the
+// reference's forms keep the complement).  Without dropout every bit is set and nothing is drawn.
+template <bool REF>
+__device__ __forceinline__ uint32_t draw_quad(const EpiPrm& k, size_t mask_idx) {
+  if (!REF && !k.apply_dropout) return 0xfu;
+  const uint64_t blk = (uint64_t)mask_idx >> 2;   // the Philox counter: one block of four words per quad
+  const Philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u, k.seed_lo, k.seed_hi);
+  return (keep_from_threshold(r.x, k.thr) ? 1u : 0u) | (keep_from_threshold(r.y, k.thr) ? 2u : 0u) |
+         (keep_from_threshold(r.z, k.thr) ? 4u : 0u) | (keep_from_threshold(r.w, k.thr) ? 8u : 0u);
+}
+// ge: draw_quad's mask for this quad.
+template <int NP, bool REF, bool F16 = false>
+__device__ __forceinline__ u32x2 epilogue_quad(f32x4 acc, const EpiIn<NP>& in, const f32x4 bv, const EpiPrm& k, uint32_t ge) {
+  f32x4 s = acc;
+#pragma unroll
+  for (int q = 0; q < NP; q++) s = s + in.pv[q];
+  const float rs[4] = {half_in<F16>((uint16_t)(in.rv[0] & 0xffffu)), half_in<F16>((uint16_t)(in.rv[0] >> 16)),
+                       half_in<F16>((uint16_t)(in.rv[1] & 0xffffu)), half_in<F16>((uint16_t)(in.rv[1] >> 16))};
+  float y[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const bool g = (ge >> e) & 1u;
+    if constexpr (!REF) {
+      // drop with probability p, survivors scaled by 1/(1-p) (keep_scale is 1 without dropout)
+      const float t = s[e] + bv[e];
+      y[e] = (g ? t * k.keep_scale : 0.0f) + rs[e];
+    } else if (k.mode == CCN_DROPOUT_REF_DSL) {
+      // the reference's emitted expression (src/codegen.cpp:634-640): (u < p ? (sum + bias) : 0) + residual
+      const float t = s[e] + bv[e];
+      y[e] = (!g ? t : 0.0f) + rs[e];
+    } else {
+      // the reference's fused kernel (nccl-overlap/src/collectives/device/reduce_kernel.h:192-213):
+      // ((u < p ? sum : 0) + bias) + residual; its half specialisation adds with saturation to [0, 1]
+      const float d = !g ? s[e] : 0.0f;
+      y[e] = k.mode == CCN_DROPOUT_REF_NCCL_SAT ? sat01(sat01(d + bv[e]) + rs[e]) : (d + bv[e]) + rs[e];
+    }
+  }
+  u32x2 o;
+  if constexpr (F16) {
+    o[0] = (uint32_t)half_out<F16>(y[0]) | ((uint32_t)half_out<F16>(y[1]) << 16);
+    o[1] = (uint32_t)half_out<F16>(y[2]) | ((uint32_t)half_out<F16>(y[3]) << 16);
+  } else {
+    o[0] = pack_upper_halves(f32_to_bf16_hi(y[0]), f32_to_bf16_hi(y[1]));
+    o[1] = pack_upper_halves(f32_to_bf16_hi(y[2]), f32_to_bf16_hi(y[3]));
+  }
+  return o;
+}
+// The same with the quad addressed by its element index idx in `out` and its first column n.
 template <int NP, bool REF, bool F16 = false>
 __device__ __forceinline__ void epilogue_finish(f32x4 acc, const EpiIn<NP>& in, const float* __restrict__ bias,
                                                 uint16_t* __restrict__ out, size_t idx, size_t n, const EpiPrm& k,
                                                 size_t mask_idx) {
-  const f32x4 bv = *reinterpret_cast<const f32x4*>(bias + n);
-  f32x4 s = acc;
-#pragma unroll
-  for (int q = 0; q < NP; q++) s = s + in.pv[q];
-  const float r0 = half_in<F16>((uint16_t)(in.rv[0] & 0xffffu)), r1 = half_in<F16>((uint16_t)(in.rv[0] >> 16));
-  const float r2 = half_in<F16>((uint16_t)(in.rv[1] & 0xffffu)), r3 = half_in<F16>((uint16_t)(in.rv[1] >> 16));
-  float y0, y1, y2, y3;
-  if constexpr (!REF) {
-    // drop with probability p, survivors scaled by 1/(1-p)
-    const f32x4 t = s + bv;
-    f32x4 d = t;
-    if (k.apply_dropout) {
-      const uint64_t blk = (uint64_t)mask_idx >> 2;
-      const Philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u, k.seed_lo, k.seed_hi);
-      d[0] = keep_from_word(r.x, k.p_drop) ? t[0] * k.keep_scale : 0.0f;
-      d[1] = keep_from_word(r.y, k.p_drop) ? t[1] * k.keep_scale : 0.0f;
-      d[2] = keep_from_word(r.z, k.p_drop) ? t[2] * k.keep_scale : 0.0f;
-      d[3] = keep_from_word(r.w, k.p_drop) ? t[3] * k.keep_scale : 0.0f;
-    }
-    y0 = d[0] + r0; y1 = d[1] + r1; y2 = d[2] + r2; y3 = d[3] + r3;
-  } else {
-    const uint64_t blk = (uint64_t)mask_idx >> 2;
-    const Philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, 0u, k.seed_lo, k.seed_hi);
-    // kept where u < p: the complement of keep_from_word's u >= p
-    const bool kp[4] = {!keep_from_word(r.x, k.p_drop), !keep_from_word(r.y, k.p_drop), !keep_from_word(r.z, k.p_drop),
-                        !keep_from_word(r.w, k.p_drop)};
-    const float rs[4] = {r0, r1, r2, r3};
-    float y[4];
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      if (k.mode == CCN_DROPOUT_REF_DSL) {
-        // the reference's emitted expression (src/codegen.cpp:634-640): (u < p ? (sum + bias) : 0) + residual
-        const float t = s[e] + bv[e];
-        y[e] = (kp[e] ? t : 0.0f) + rs[e];
-      } else {
-        // the reference's fused kernel (nccl-overlap/src/collectives/device/reduce_kernel.h:192-213):
-        // ((u < p ? sum : 0) + bias) + residual; its half specialisation adds with saturation to [0, 1]
-        const float d = kp[e] ? s[e] : 0.0f;
-        y[e] = k.mode == CCN_DROPOUT_REF_NCCL_SAT ? sat01(sat01(d + bv[e]) + rs[e]) : (d + bv[e]) + rs[e];
-      }
-    }
-    y0 = y[0]; y1 = y[1]; y2 = y[2]; y3 = y[3];
-  }
-  u32x2 o;
-  o[0] = (uint32_t)half_out<F16>(y0) | ((uint32_t)half_out<F16>(y1) << 16);
-  o[1] = (uint32_t)half_out<F16>(y2) | ((uint32_t)half_out<F16>(y3) << 16);
+  const u32x2 o = epilogue_quad<NP, REF, F16>(acc, in, *reinterpret_cast<const f32x4*>(bias + n), k, draw_quad<REF>(k, mask_idx));
   __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(out + idx));
 }
+
+// Buffer addressing: a workgroup-uniform base (a resource descriptor in scalar registers, no bounds: the host checks the
+// offsets), a uniform scalar offset and one 32-bit offset per lane.  The addresses of a tile walk then cost scalar
+// adds where 64-bit flat addresses cost a vector register pair and a 64-bit vector add per access.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t buffer_at(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7ffffffc, 0x00020000);
+}
+constexpr int kAuxNt = 2;   // the nontemporal bit of a gfx950 buffer instruction's cache policy
+// The matrix-core kernel reaches 128 rows of N fp32 and 128 rows of K 16-bit elements from one descriptor: both must stay
+// inside the 2 GiB a descriptor spans.  Larger row lengths take the any-shape kernel.
+constexpr int kMaxRowLen = 1 << 21;
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 7); }
 
 // PLAIN: the product alone, written as fp32 [M x N] through `out` (no partial buffers, bias, dropout or residual).
 // REF: the epilogue applies one of the reference's dropout forms.
+// The rows are dealt to the wavefronts (see the top of the file) so that the epilogue needs no workgroup barrier: after
+// the main loop a wavefront turns its own accumulators into rows through a private piece of LDS (16 rows at a time) and
+// walks its 16 row pairs.  At step j the four wavefronts of the workgroup together touch 8 adjacent rows x 512 bytes of
+// every partial buffer; the operands of step j+1 are requested before step j is finished, step 0's under the last MFMA
+// step.  Three workgroups share a CU (168 registers, 33 KiB of LDS).
 template <int NP, bool PLAIN = false, bool REF = false, bool F16 = false>
-__global__ __launch_bounds__(kBlock) void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
-                                                             const SrcTable<float, 8> parts,
-                                                             const float* __restrict__ bias,
-                                                             const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
-                                                             const int N, const int K, const EpiPrm ep) {
-  // main loop: X tile [m][k] and transposed W tile [n][k], 16 KiB each, chunk-swizzled.
-  // epilogue: half of the fp32 C tile, 64 rows x (128 + 4 pad) floats, to turn the MFMA register layout
-  // into whole 512-byte row segments per wavefront.
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 3)))
+void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
+                                                                  const SrcTable<float, 8> parts,
+                                                                  const float* __restrict__ bias,
+                                                                  const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
+                                                                  const int N, const int K, const EpiPrm ep) {
   constexpr int kCStride = BN + 4;
-  constexpr int kLdsBytes = (BM / 2) * kCStride * 4 > 2 * BM * BK * 2 ? (BM / 2) * kCStride * 4 : 2 * BM * BK * 2;
+  constexpr int kWaveRows = 16;   // rows of C a wavefront has in LDS at a time
+  constexpr int kCBytes = (kBlock / kWave) * kWaveRows * kCStride * 4;
+  constexpr int kTileBytes = 2 * BM * BK * 2;                 // one K-step of X and W^T
+  constexpr int kLdsBytes = kCBytes > kTileBytes ? kCBytes : kTileBytes;
   __shared__ __attribute__((aligned(16))) uint8_t lds_all[kLdsBytes];
   uint8_t* const lds_x = lds_all;
   uint8_t* const lds_w = lds_all + BM * BK * 2;
-  float* const lds_c = reinterpret_cast<float*>(lds_all);
 
-  // ---- workgroup -> tile: along a tile row first.  Workgroups that run at the same time then cover whole rows of
-  //      the partial buffers between them (measured: the epilogue streams reach 75-79 % of HBM peak this way, 62-66 %
-  //      when neighbours in time are neighbours in a tile column), and since workgroups are dealt round-robin to the
-  //      8 XCDs, an XCD only ever touches the W panels of every 8th tile column: with N/BN a multiple of 8 they stay
-  //      in its L2 (8 panels of 2*K*BN bytes), while an X panel is shared by the XCD's 8 tiles of a row.
   const int tilesN = N / BN;
   const int tm = blockIdx.x / tilesN, tn = blockIdx.x % tilesN;
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int li = lane & 31, lh = lane >> 5;
+  const int rho = 8 * (li >> 1) + 2 * wave + (li & 1);   // tile row behind this lane's accumulator column
 
-  // global -> register staging assignments
+  // Addresses are a workgroup-uniform 64-bit base, kept in scalar registers and advanced by scalar adds, plus a 32-bit
+  // byte offset per lane that never changes (the host checks that the offsets fit): no vector address arithmetic.
   const int xr = t >> 3, xc = t & 7;          // X: rows xr + 32*j, 16-byte chunk xc
   const int wg = t & 15, wq = t >> 4;         // W: k rows wq*4 + j, columns wg*8..+7
-  u32x4 xreg[4], wreg[4];
+  struct Staged { u32x4 x[4], w[4]; };
+  uint32_t xoff[4], woff[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    xoff[j] = (uint32_t)(((xr + 32 * j) * K + xc * 8) * 2);
+    woff[j] = (uint32_t)(((wq * 4 + j) * N + wg * 8) * 2);
+  }
+  const rsrc_t x_rs = buffer_at(X + m0 * (size_t)K);   // the tile's 128 rows of X
+  const uint16_t* const wbase = W + n0;
 
-  auto load_tile = [&](int k0) {
+  auto load_tile = [&](Staged& r, int k0) {
+    const rsrc_t w_rs = buffer_at(wbase + (size_t)k0 * N);   // the 64 rows of W of this K-step
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      xreg[j] = *reinterpret_cast<const u32x4*>(X + (m0 + xr + 32 * j) * (size_t)K + k0 + xc * 8);
-      wreg[j] = *reinterpret_cast<const u32x4*>(W + (size_t)(k0 + wq * 4 + j) * N + n0 + wg * 8);
+      r.x[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rs, xoff[j], (uint32_t)k0 * 2u, 0));
+      r.w[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w_rs, woff[j], 0, 0));
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](const Staged& r) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int row = xr + 32 * j;
-      *reinterpret_cast<u32x4*>(lds_x + row * 128 + ((xc ^ swz(row)) << 4)) = xreg[j];
+      *reinterpret_cast<u32x4*>(lds_x + row * 128 + ((xc ^ swz(row)) << 4)) = r.x[j];
     }
-    // transpose 4(k) x 8(n) -> 8 rows of 4 k
+    // transpose 4(k) x 8(n) -> 8 rows of 4 k, one byte permute per word
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-      const uint32_t a0 = wreg[0][q], a1 = wreg[1][q], a2 = wreg[2][q], a3 = wreg[3][q];
+      const uint32_t a0 = r.w[0][q], a1 = r.w[1][q], a2 = r.w[2][q], a3 = r.w[3][q];
       u32x2 lo, hi;   // lo: column 2q, hi: column 2q+1; each k0..k3
-      lo[0] = (a0 & 0xffffu) | (a1 << 16);
-      lo[1] = (a2 & 0xffffu) | (a3 << 16);
-      hi[0] = (a0 >> 16) | (a1 & 0xffff0000u);
-      hi[1] = (a2 >> 16) | (a3 & 0xffff0000u);
+      lo[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100u);
+      lo[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100u);
+      hi[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302u);
+      hi[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
       const int r0 = wg * 8 + 2 * q, r1 = r0 + 1;
       *reinterpret_cast<u32x2*>(lds_w + r0 * 128 + (((wq >> 1) ^ swz(r0)) << 4) + ((wq & 1) << 3)) = lo;
       *reinterpret_cast<u32x2*>(lds_w + r1 * 128 + (((wq >> 1) ^ swz(r1)) << 4) + ((wq & 1) << 3)) = hi;
     }
   };
 
-  f32x16 acc[2][2];   // [bn][bm]
+  f32x16 acc[4];   // [bn]: register 4*i4+e is C[rho][bn*32 + i4*8 + lh*4 + e]
 #pragma unroll
-  for (int a = 0; a < 2; a++)
+  for (int a = 0; a < 4; a++)
 #pragma unroll
-    for (int b = 0; b < 2; b++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
+    for (int i = 0; i < 16; i++) acc[a][i] = 0.0f;
 
-  const int nk = K / BK;
-  load_tile(0);
-  store_tile();
-  __syncthreads();
-  for (int kt = 0; kt < nk; kt++) {
-    if (kt + 1 < nk) load_tile((kt + 1) * BK);
+  auto mfma_step = [&]() {
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ks++) {
-      const int c = ks * 2 + (lane >> 5);
-      bf16x8 fa[2], fb[2];
+      const int c = ks * 2 + lh;
+      const bf16x8 fb = *reinterpret_cast<const bf16x8*>(lds_x + rho * 128 + ((c ^ swz(rho)) << 4));
 #pragma unroll
-      for (int bn = 0; bn < 2; bn++) {
-        const int row = wn * 64 + bn * 32 + (lane & 31);
-        fa[bn] = *reinterpret_cast<const bf16x8*>(lds_w + row * 128 + ((c ^ swz(row)) << 4));
+      for (int bn = 0; bn < 4; bn++) {
+        const int row = bn * 32 + li;
+        const bf16x8 fa = *reinterpret_cast<const bf16x8*>(lds_w + row * 128 + ((c ^ swz(row)) << 4));
+        if constexpr (F16)
+          acc[bn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa), __builtin_bit_cast(f16x8, fb), acc[bn], 0, 0, 0);
+        else
+          acc[bn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[bn], 0, 0, 0);
       }
-#pragma unroll
-      for (int bm = 0; bm < 2; bm++) {
-        const int row = wm * 64 + bm * 32 + (lane & 31);
-        fb[bm] = *reinterpret_cast<const bf16x8*>(lds_x + row * 128 + ((c ^ swz(row)) << 4));
-      }
-#pragma unroll
-      for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-        for (int bm = 0; bm < 2; bm++)
-          if constexpr (F16)
-            acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[bn]), __builtin_bit_cast(f16x8, fb[bm]),
-                                                                 acc[bn][bm], 0, 0, 0);
-          else
-            acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[bn], fb[bm], acc[bn][bm], 0, 0, 0);
     }
-    __syncthreads();
-    if (kt + 1 < nk) {
-      store_tile();
-      __syncthreads();
-    }
-  }
+  };
 
-  // ---- epilogue.  Accumulator register 4*i4+e of block (bn,bm) is C[m][n+e] with
-  //      n = wn*64 + bn*32 + i4*8 + (lane/32)*4,  m = wm*64 + bm*32 + lane%32  (tile-local).
-  //      Read straight from HBM in that layout, a wavefront instruction would touch 32 rows x 32 bytes of every
-  //      partial buffer; going through LDS makes it 2 rows x 512 contiguous bytes.
-  for (int half = 0; half < 2; half++) {
-    __syncthreads();   // main-loop tiles (half 0) or the previous half's C rows are no longer needed
-    if (wm == half) {
+  // the walk of the epilogue: at step j this lane has row 8j + 2*wave + lane/32, columns 4*(lane%32)..+3
+  const int sc = li * 4;
+  const size_t tile0 = m0 * (size_t)N + n0;                                  // first element of the tile (uniform)
+  const uint32_t eoff = (uint32_t)((2 * wave + lh) * N + sc);                // this lane's element within a step
+  const uint32_t estep = 8u * (uint32_t)N;                                   // elements from one step to the next
+  rsrc_t p_rs[NP > 0 ? NP : 1];
 #pragma unroll
-      for (int bm = 0; bm < 2; bm++) {
-        const int row = bm * 32 + (lane & 31);
+  for (int q = 0; q < (PLAIN ? 0 : NP); q++) p_rs[q] = buffer_at(parts.p[q] + tile0);
+  const rsrc_t r_rs = buffer_at(resid ? resid + tile0 : nullptr);
+  const rsrc_t o_rs = buffer_at(PLAIN ? static_cast<void*>(reinterpret_cast<float*>(out) + tile0) : static_cast<void*>(out + tile0));
+  auto load_step = [&](EpiIn<PLAIN ? 0 : NP>& in, int j) {
 #pragma unroll
-        for (int bn = 0; bn < 2; bn++) {
-#pragma unroll
-          for (int i4 = 0; i4 < 4; i4++) {
-            const int col = wn * 64 + bn * 32 + i4 * 8 + (lane >> 5) * 4;
-            f32x4 a;
-            a[0] = acc[bn][bm][i4 * 4 + 0];
-            a[1] = acc[bn][bm][i4 * 4 + 1];
-            a[2] = acc[bn][bm][i4 * 4 + 2];
-            a[3] = acc[bn][bm][i4 * 4 + 3];
-            *reinterpret_cast<f32x4*>(lds_c + row * kCStride + col) = a;
-          }
-        }
-      }
-    }
+    for (int q = 0; q < (PLAIN ? 0 : NP); q++)
+      in.pv[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(p_rs[q], eoff * 4u, (uint32_t)j * estep * 4u, kAuxNt));
+    in.rv = u32x2{0u, 0u};
+    if (resid) in.rv = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r_rs, eoff * 2u, (uint32_t)j * estep * 2u, kAuxNt));
+  };
+  EpiIn<PLAIN ? 0 : NP> cur;
+
+  // main loop: the tile of step kt+1 travels from memory to registers while step kt is multiplied
+  const int nk = K / BK;
+  Staged st;
+  load_tile(st, 0);
+  store_tile(st);
+  __syncthreads();
+  for (int kt = 0; kt + 1 < nk; kt++) {
+    load_tile(st, (kt + 1) * BK);
+    __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the MFMA step (the scheduler would sink them to their use)
+    mfma_step();
     __syncthreads();
-    constexpr int kIters = (BM / 2) * (BN / 4) / kBlock;
-    // the loads of quad it+1 are issued before quad it is finished
-    auto index_of = [&](int it) {
-      const int q = it * kBlock + t;
-      return (m0 + half * 64 + q / (BN / 4)) * (size_t)N + n0 + (q % (BN / 4)) * 4;
-    };
-    if constexpr (PLAIN) {
-      float* const outc = reinterpret_cast<float*>(out);
+    store_tile(st);
+    __syncthreads();
+  }
+  if constexpr (!PLAIN) load_step(cur, 0);
+  mfma_step();
+  __syncthreads();   // every wavefront is done with the operand tiles: LDS becomes four private C pieces
+
+  float* const cw = reinterpret_cast<float*>(lds_all) + wave * (kWaveRows * kCStride);
+  f32x4 bv = {0.0f, 0.0f, 0.0f, 0.0f};
+  if constexpr (!PLAIN) bv = *reinterpret_cast<const f32x4*>(bias + n0 + sc);
 #pragma unroll
-      for (int it = 0; it < kIters; it++) {
-        const int q = it * kBlock + t;
-        const int row = q / (BN / 4), colq = q % (BN / 4);
-        *reinterpret_cast<f32x4*>(outc + index_of(it)) = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
-      }
-    } else {
-      EpiIn<NP> cur;
-      epilogue_load<NP>(cur, parts, resid, index_of(0));
+  for (int half = 0; half < 2; half++) {
+    if ((li >> 4) == half) {
+      const int r16 = li & 15;
 #pragma unroll
-      for (int it = 0; it < kIters; it++) {
+      for (int bn = 0; bn < 4; bn++)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          f32x4 v;
+          v[0] = acc[bn][i4 * 4 + 0];
+          v[1] = acc[bn][i4 * 4 + 1];
+          v[2] = acc[bn][i4 * 4 + 2];
+          v[3] = acc[bn][i4 * 4 + 3];
+          *reinterpret_cast<f32x4*>(cw + r16 * kCStride + bn * 32 + i4 * 8 + lh * 4) = v;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();   // a wavefront's LDS operations complete in order: no wait between its writes and reads
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) {
+      const int j = half * 8 + jj;
+      const f32x4 v = *reinterpret_cast<const f32x4*>(cw + (2 * jj + lh) * kCStride + sc);
+      if constexpr (PLAIN) {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), o_rs, eoff * 4u, (uint32_t)j * estep * 4u, 0);
+      } else {
+        const uint32_t ge = draw_quad<REF>(ep, tile0 + (size_t)j * estep + eoff);
         EpiIn<NP> nxt;
-        if (it + 1 < kIters) epilogue_load<NP>(nxt, parts, resid, index_of(it + 1));
-        const int q = it * kBlock + t;
-        const int row = q / (BN / 4), colq = q % (BN / 4);
-        const f32x4 a = *reinterpret_cast<const f32x4*>(lds_c + row * kCStride + colq * 4);
-        epilogue_finish<NP, REF, F16>(a, cur, bias, out, index_of(it), n0 + colq * 4, ep, index_of(it));
-        if (it + 1 < kIters) cur = nxt;
+        if (j + 1 < 16) load_step(nxt, j + 1);
+        const u32x2 o = epilogue_quad<NP, REF, F16>(v, cur, bv, ep, ge);
+        __builtin_amdgcn_raw_buffer_store_b64(o, o_rs, eoff * 2u, (uint32_t)j * estep * 2u, kAuxNt);
+        if (j + 1 < 16) cur = nxt;
       }
     }
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -377,6 +403,7 @@ static int make_epi(float p_drop, uint64_t seed, int mode, EpiPrm* ep) {
   // inverted dropout rescales by 1/(1-p): p < 1.  The reference's forms keep with probability p: p = 1 keeps everything.
   if (!(p_drop >= 0.0f) || !(mode == CCN_DROPOUT_INVERTED ? p_drop < 1.0f : p_drop <= 1.0f)) return CCN_EINVAL;
   ep->p_drop = p_drop;
+  ep->thr = keep_threshold(p_drop);
   ep->keep_scale = mode == CCN_DROPOUT_INVERTED ? 1.0f / (1.0f - p_drop) : 1.0f;
   ep->seed_lo = (uint32_t)seed;
   ep->seed_hi = (uint32_t)(seed >> 32);
@@ -412,7 +439,7 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
   rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
   hipStream_t s = as_stream(stream);
-  if (M % BM || N % BN || K % BK) {   // not whole tiles of the matrix-core kernel
+  if (M % BM || N % BN || K % BK || N > kMaxRowLen || K > kMaxRowLen) {   // not whole tiles of the matrix-core kernel
     const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
     if (tiles > 0x7fffffffull) return CCN_ERANGE;
     if (mode == CCN_DROPOUT_INVERTED)
@@ -505,7 +532,7 @@ int matmul_launch(const uint16_t* X, const uint16_t* W, float* C, int M, int N, 
   SrcTable<float, 8> tbl;
   for (int q = 0; q < 8; q++) tbl.p[q] = nullptr;
   EpiPrm ep{};
-  if (M % BM || N % BN || K % BK) {
+  if (M % BM || N % BN || K % BK || N > kMaxRowLen || K > kMaxRowLen) {
     const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
     if (tiles > 0x7fffffffull) return CCN_ERANGE;
     hipLaunchKernelGGL((outproj_any_shape_kernel<true, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, as_stream(stream), X, W,
