@@ -208,20 +208,37 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[a][i] = 0.0f;
 
+  // One K-step: four rounds of 16 k, each one X fragment against four W fragments: 16 MFMAs.  The W fragment of MFMA
+  // i+2 (and the X fragment of the next round) is read from LDS before MFMA i is issued, so that an MFMA does not wait
+  // for the read just before it; two fragments ahead is what the register budget of three workgroups per CU allows.
+  auto read_w = [&](int i) {
+    const int c = (i >> 2) * 2 + lh, row = (i & 3) * 32 + li;
+    return *reinterpret_cast<const bf16x8*>(lds_w + row * 128 + ((c ^ swz(row)) << 4));
+  };
+  auto read_x = [&](int ks) {
+    const int c = ks * 2 + lh;
+    return *reinterpret_cast<const bf16x8*>(lds_x + rho * 128 + ((c ^ swz(rho)) << 4));
+  };
   auto mfma_step = [&]() {
+    constexpr int kAhead = 2;
+    bf16x8 fa[kAhead + 1], fb[2];
+    fb[0] = read_x(0);
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      const int c = ks * 2 + lh;
-      const bf16x8 fb = *reinterpret_cast<const bf16x8*>(lds_x + rho * 128 + ((c ^ swz(rho)) << 4));
+    for (int i = 0; i < kAhead; i++) fa[i] = read_w(i);
+    __builtin_amdgcn_sched_group_barrier(0x100, 1 + kAhead, 0);
 #pragma unroll
-      for (int bn = 0; bn < 4; bn++) {
-        const int row = bn * 32 + li;
-        const bf16x8 fa = *reinterpret_cast<const bf16x8*>(lds_w + row * 128 + ((c ^ swz(row)) << 4));
-        if constexpr (F16)
-          acc[bn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa), __builtin_bit_cast(f16x8, fb), acc[bn], 0, 0, 0);
-        else
-          acc[bn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[bn], 0, 0, 0);
-      }
+    for (int i = 0; i < 16; i++) {
+      int reads = 0;
+      if (i + kAhead < 16) { fa[(i + kAhead) % (kAhead + 1)] = read_w(i + kAhead); reads++; }
+      if ((i & 3) == 4 - kAhead && (i >> 2) + 1 < 4) { fb[((i >> 2) + 1) & 1] = read_x((i >> 2) + 1); reads++; }
+      if (reads == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      if (reads == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      const bf16x8 a = fa[i % (kAhead + 1)], b = fb[(i >> 2) & 1];
+      if constexpr (F16)
+        acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc[i & 3], 0, 0, 0);
+      else
+        acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i & 3], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
   };
 
@@ -249,13 +266,16 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
   Staged st;
   load_tile(st, 0);
   store_tile(st);
+  if (nk > 1) load_tile(st, BK);
   __syncthreads();
   for (int kt = 0; kt + 1 < nk; kt++) {
-    load_tile(st, (kt + 1) * BK);
-    __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the MFMA step (the scheduler would sink them to their use)
     mfma_step();
     __syncthreads();
     store_tile(st);
+    // the next tile's loads go out as soon as the staging registers are free, ahead of the barrier and the MFMA step
+    // (the sched_barrier keeps the scheduler from sinking them to their use)
+    if (kt + 2 < nk) load_tile(st, (kt + 2) * BK);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
   }
   if constexpr (!PLAIN) load_step(cur, 0);
