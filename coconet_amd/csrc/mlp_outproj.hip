@@ -55,12 +55,9 @@ __device__ __forceinline__ float sat01(float x) { return x > 0.0f ? (x < 1.0f ? 
 // Two 16-bit halves into one word: the upper halves of lo and hi (lo in bits 0-15)
 __device__ __forceinline__ uint32_t pack_upper_halves(uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); }
 
-// The four finished 16-bit outputs of a quad.  mask_idx: the quad's element index in the whole [M x N] output, which
-// the mask is drawn from; bv: the bias of the quad's four columns.
-// REF: one of the reference's dropout forms (k.mode says which); false: standard dropout, the form the kernels are
-// tuned for, compiled without the others.
 // The quad's four draws as a mask: bit e is set where u >= p for element e (the element survives standard dropout; the
 // reference's forms keep the complement).  Without dropout every bit is set and nothing is drawn.
+// mask_idx: the quad's element index in the whole [M x N] output, which the mask is drawn from.
 template <bool REF>
 __device__ __forceinline__ uint32_t draw_quad(const EpiPrm& k, size_t mask_idx) {
   if (!REF && !k.apply_dropout) return 0xfu;
@@ -69,7 +66,9 @@ __device__ __forceinline__ uint32_t draw_quad(const EpiPrm& k, size_t mask_idx) 
   return (keep_from_threshold(r.x, k.thr) ? 1u : 0u) | (keep_from_threshold(r.y, k.thr) ? 2u : 0u) |
          (keep_from_threshold(r.z, k.thr) ? 4u : 0u) | (keep_from_threshold(r.w, k.thr) ? 8u : 0u);
 }
-// ge: draw_quad's mask for this quad.
+// The four finished 16-bit outputs of a quad.  ge: draw_quad's mask for this quad; bv: the bias of its four columns.
+// REF: one of the reference's dropout forms (k.mode says which); false: standard dropout, the form the kernels are
+// tuned for, compiled without the others.
 template <int NP, bool REF, bool F16 = false>
 __device__ __forceinline__ u32x2 epilogue_quad(f32x4 acc, const EpiIn<NP>& in, const f32x4 bv, const EpiPrm& k, uint32_t ge) {
   f32x4 s = acc;
@@ -138,11 +137,9 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 7
 // step.  Three workgroups share a CU (168 registers, 33 KiB of LDS).
 template <int NP, bool PLAIN = false, bool REF = false, bool F16 = false>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 3)))
-void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
-                                                                  const SrcTable<float, 8> parts,
-                                                                  const float* __restrict__ bias,
-                                                                  const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
-                                                                  const int N, const int K, const EpiPrm ep) {
+void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, const SrcTable<float, 8> parts,
+                        const float* __restrict__ bias, const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
+                        const int N, const int K, const EpiPrm ep) {
   constexpr int kCStride = BN + 4;
   constexpr int kWaveRows = 16;   // rows of C a wavefront has in LDS at a time
   constexpr int kCBytes = (kBlock / kWave) * kWaveRows * kCStride * 4;
