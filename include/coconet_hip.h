@@ -216,9 +216,9 @@ int  ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream);
  *      fp32 [MxN]; bias fp32 [N]; resid may be NULL.  Dropout: element idx=row*N+col is dropped when
  *      u(seed, idx) < p_drop, survivors are scaled by 1/(1-p_drop); u comes from Philox-4x32-10 with
  *      counter (idx/4, 0) and key seed, word idx%4, u = (word>>8)*2^-24.
- *      Shapes: any M and K; N a multiple of 4 (CCN_ERANGE otherwise).  Whole 128x128x64 tiles run on the matrix cores;
- *      any other shape takes a vector-ALU kernel that is an order of magnitude slower (the reference's cuBLAS call
- *      takes any shape too).  fp32 arrays 16-byte aligned, bf16 arrays 8-byte aligned (X, W: 16).
+ *      Shapes: any M and K; N a multiple of 4 (CCN_ERANGE otherwise).  Whole 128x128x64 tiles with N and K up to 2^21
+ *      run on the matrix cores; any other shape takes a vector-ALU kernel that is an order of magnitude slower (the
+ *      reference's cuBLAS call takes any shape too).  fp32 arrays 16-byte aligned, bf16 arrays 8-byte aligned (X, W: 16).
  *      Replaces MatMul + AllReduce + (sum+b) + Dropout + r of examples/model-parallel/model-parallel.cpp:18-21
  *      (emitted cublasGemmEx src/codegen.cpp:1058-1136; fused epilogue
  *      nccl-overlap/src/collectives/device/common_kernel.h:1037-1057, reduce_kernel.h:192-213). ---- */
