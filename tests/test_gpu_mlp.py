@@ -203,6 +203,37 @@ def test_outproj_tile_order_and_indexing(ccn):
     assert np.array_equal(orc.bf16_to_f32(bf16_host(out)).reshape(M, N), Wf[sel])
 
 
+def _awkward_probabilities():
+    """Drop probabilities around the places where the kernels' integer form of the keep decision (draw >= ceil(p * 2^24))
+    could part from the oracle's float comparison u >= p: multiples of 2^-24 and their float neighbours, the smallest and
+    the largest probabilities, and a few arbitrary ones."""
+    f = np.float32
+    ps = [f(2.0 ** -24), np.nextafter(f(2.0 ** -24), f(1)), np.nextafter(f(2.0 ** -24), f(0)), f(2.0 ** -30),
+          f(0.25), np.nextafter(f(0.25), f(1)), np.nextafter(f(0.25), f(0)), f(1.0) - f(2.0 ** -24),
+          np.nextafter(f(1.0), f(0)), f(3 * 2.0 ** -24), f(0.1), f(1.0 / 3.0), f(0.999)]
+    return [float(x) for x in ps]
+
+
+@pytest.mark.parametrize("p", _awkward_probabilities())
+def test_dropout_decision_matches_the_oracle_for_awkward_probabilities(ccn, p):
+    """The mask, element by element: with a zero product, zero bias and a residual of zero, an output element is zero
+    exactly where the element was dropped (the inputs are bounded away from zero).  2^20 draws per probability, through
+    the stand-alone epilogue and through the fused kernel."""
+    M, N, K = 1024, 1024, 64
+    acc = np.full((M, N), 1.0, dtype=np.float32)
+    zero_bias = np.zeros(N, dtype=np.float32)
+    keep = orc.dropout_mask(5, 0, M * N, p).reshape(M, N).astype(bool)
+    out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.bias_dropout_residual(torch.from_numpy(acc).to(DEV), [], torch.from_numpy(zero_bias).to(DEV), None, out, M, N, p, 5)
+    assert np.array_equal(bf16_host(out).reshape(M, N) != 0, keep)
+    # fused kernel: X = 0, so the product is zero and the partial buffer carries the ones
+    X = torch.zeros(M, K, dtype=torch.int16, device=DEV)
+    W = torch.zeros(K, N, dtype=torch.int16, device=DEV)
+    out2 = torch.zeros(M, N, dtype=torch.int16, device=DEV)
+    ccn.mlp_outproj_bf16(X, W, [torch.from_numpy(acc).to(DEV)], torch.from_numpy(zero_bias).to(DEV), None, out2, M, N, K, p, 5)
+    assert np.array_equal(bf16_host(out2).reshape(M, N) != 0, keep)
+
+
 @pytest.mark.parametrize("M,N,nP,p", [(64, 128, 7, 0.1), (3, 20, 2, 0.3), (1000, 36, 0, 0.0), (17, 4, 7, 0.9)])
 def test_standalone_epilogue_bit_exact(ccn, M, N, nP, p):
     r = rng(50 + nP)
