@@ -27,10 +27,10 @@ LAMB_NCCL_GLOBAL = 2
 SYMBOLS = [
     "ccn_version", "ccn_init", "ccn_device_info", "ccn_malloc", "ccn_free", "ccn_memcpy_h2d", "ccn_memcpy_d2h",
     "ccn_memcpy_d2d", "ccn_fill_f32", "ccn_stream_create", "ccn_stream_destroy", "ccn_stream_sync",
-    "ccn_event_create", "ccn_event_destroy", "ccn_event_record", "ccn_event_elapsed_ms", "ccn_last_hip_error",
+    "ccn_event_create", "ccn_event_destroy", "ccn_event_record", "ccn_stream_wait_event", "ccn_event_elapsed_ms", "ccn_last_hip_error",
     "ccn_strerror", "ccn_reduce_f32", "ccn_sgd_f32", "ccn_sgd_axpby_f32", "ccn_pseudo_adam_f32", "ccn_adam_f32",
     "ccn_adam_f16g", "ccn_overflow_check_f16", "ccn_fused_adam_ref_f16g", "ccn_lamb_plan_create", "ccn_lamb_plan_create_parented",
-    "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_mlp_outproj_bf16",
+    "ccn_lamb_plan_destroy", "ccn_lamb_f32", "ccn_lamb_plan_norms", "ccn_lamb_plan_tune", "ccn_mlp_outproj_bf16",
     "ccn_bias_dropout_residual", "ccn_graph_begin", "ccn_graph_end", "ccn_graph_launch", "ccn_graph_destroy",
     "ccn_scatter_plan_create", "ccn_scatter_plan_destroy", "ccn_sgd_f32_scattered", "ccn_adam_f32_scattered",
     "ccn_lamb_f32_scattered", "ccn_adam_bf16g", "ccn_lamb_nccl_f16g", "ccn_lamb_f32_static",
@@ -85,6 +85,7 @@ def _declare(L):
     sig("ccn_event_create", [_pp])
     sig("ccn_event_destroy", [_vp])
     sig("ccn_event_record", [_vp, _vp])
+    sig("ccn_stream_wait_event", [_vp, _vp])
     sig("ccn_event_elapsed_ms", [_vp, _vp, C.POINTER(_f)])
     sig("ccn_last_hip_error", [])
     sig("ccn_strerror", [_i], C.c_char_p)
@@ -102,6 +103,7 @@ def _declare(L):
     sig("ccn_lamb_plan_destroy", [_vp])
     sig("ccn_lamb_f32", [_vp, _pp, _i, _vp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
     sig("ccn_lamb_plan_norms", [_vp, _vp, _vp])
+    sig("ccn_lamb_plan_tune", [_vp, _i, C.c_long])
     sig("ccn_lamb_f32_static", [_pp, _i, _vp, _vp, _vp, _sz, _sz, _f, _f, _f, _f, _f, _i, _i, _vp, _vp])
     sig("ccn_lamb_f32_scattered", [_vp, _pp, _i, _pp, _vp, _vp, _f, _f, _f, _f, _f, _i, _i, _vp])
     sig("ccn_lamb_nccl_f16g", [_vp, _pp, _i, _vp, _vp, _vp, _vp, _f, _f, _f, _f, _vp])
@@ -204,7 +206,12 @@ class Event:
         self.h = h
 
     def record(self, stream=None):
-        _check(load().ccn_event_record(self.h, stream), "ccn_event_record")
+        _check(load().ccn_event_record(self.h, stream.h if isinstance(stream, Stream) else stream), "ccn_event_record")
+
+    def close(self):
+        if self.h:
+            _check(load().ccn_event_destroy(self.h), "ccn_event_destroy")
+            self.h = None
 
     def elapsed_ms(self, stop):
         ms = _f(0)
@@ -262,6 +269,9 @@ class Stream:
 
     def sync(self):
         _check(load().ccn_stream_sync(self.h), "ccn_stream_sync")
+
+    def wait_event(self, event):
+        _check(load().ccn_stream_wait_event(self.h, event.h), "ccn_stream_wait_event")
 
     def close(self):
         if self.h:
@@ -347,12 +357,18 @@ def fused_adam_ref_f16g(g, w, halfw, m, v, n, lr, beta1, beta2, stream=None):
                                           stream), "ccn_fused_adam_ref_f16g")
 
 
+LAMB_KNOB_SPIN_LIMIT, LAMB_KNOB_TWO_PASS, LAMB_KNOB_WITHHOLD = 0, 1, 2
+# knobs every new LambPlan is tuned with ({knob: value}): how the tests run whole files under another kernel path
+LAMB_DEFAULT_KNOBS = {}
+
+
 class LambPlan:
     """Device-side segment tables for one segmentation of [0, N) (ccn_lamb_plan)."""
 
-    def __init__(self, seg_offsets, buf_sizes=None, buf_parent=None):
+    def __init__(self, seg_offsets, buf_sizes=None, buf_parent=None, knobs=None):
         """seg_offsets: nseg+1 element offsets, one buffer per segment.  Or buf_sizes / buf_parent (seg_offsets None):
-        segments made of several buffers each, buffer i belonging to segment buf_parent[i]."""
+        segments made of several buffers each, buffer i belonging to segment buf_parent[i].
+        knobs: {LAMB_KNOB_*: value} passed to ccn_lamb_plan_tune (default: LAMB_DEFAULT_KNOBS)."""
         h = C.c_void_p()
         if buf_sizes is not None:
             sizes, parent = [int(x) for x in buf_sizes], [int(x) for x in buf_parent]
@@ -367,6 +383,11 @@ class LambPlan:
             arr = (_sz * len(offs))(*offs)
             _check(load().ccn_lamb_plan_create(arr, self.nseg, C.byref(h)), "ccn_lamb_plan_create")
         self.h = h
+        for knob, value in (LAMB_DEFAULT_KNOBS if knobs is None else knobs).items():
+            self.tune(knob, value)
+
+    def tune(self, knob, value):
+        _check(load().ccn_lamb_plan_tune(self.h, knob, value), "ccn_lamb_plan_tune")
 
     def step(self, g, w, m, v, lr, beta1, beta2, eps, wd, step, mode=LAMB_TRUST_RATIO, stream=None):
         p, _keep = ptr_table(g)

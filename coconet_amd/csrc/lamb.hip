@@ -5,10 +5,8 @@
 //   elements at the default shape) go through lamb_oneshot_kernel, one tile per workgroup.  A workgroup runs pass 1
 //   on its tile (P-way gradient reduce, m/v update, r, the tile's float64 sums of w^2 and r^2), keeps r in registers
 //   and the old w in LDS, waits until the workgroup that finished the segment's last tile has published the scale,
-//   and writes w from what it kept: 56 bytes per element instead of 68.  (lamb_resident_kernel, a persistent grid that
-//   parks tiles in LDS and retires them a round later, is the older form of the same thing; CCN_LAMB_ONESHOT=0 selects
-//   it.)  No sum is an atomic accumulation: tile sums are stored one by one and added in a fixed order, so results do
-//   not depend on scheduling.
+//   and writes w from what it kept: 56 bytes per element instead of 68.  No sum is an atomic accumulation: tile sums
+//   are stored one by one and added in a fixed order, so results do not depend on scheduling.
 // the other segments take two streaming passes with a finalize kernel between them:
 //   pass 1   one workgroup per tile of kLambTile elements, one 4-element pack per thread
 //   finalize one workgroup per segment: fixed-order sum of the segment's tile pairs, norms, scale
@@ -435,19 +433,9 @@ __global__ __launch_bounds__(kBlock) void lamb_pass2_f16w_kernel(float* w, uint1
   }
 }
 
-// ---- segment-resident variant, persistent form ----------------------------------------------------------------------
-// A persistent grid that is resident as a whole walks the tiles of the "resident" segments round-robin.  A workgroup
-// runs pass 1 on a tile, parks the tile's r and old w in LDS, and retires the tile one round later, when the
-// segment's scale is known: pass 2 then reads nothing from memory.  The workgroup that finishes a segment's last tile
-// computes its norms and scale and publishes them through a flag.  Every wait is bounded: a tile whose segment is not
-// ready within the spin limit goes onto a deferred list, and a trailing kernel finishes it from the stored m and v
-// (w is still the old one), so the result is the same whatever the scheduling and every workgroup exits.
-// A segment may hold at most kResDepth * gridDim.x tiles: with more, a workgroup's parking slots would fill up
-// with tiles of a segment whose other tiles it has yet to start.
-constexpr int kResDepth = 2;   // parking slots per workgroup
-constexpr int kResSub = 4;     // packs per thread per tile
-constexpr int kOneshotSub = 8;
-constexpr int kOneshotBlock = 256; // the same for the one-tile-per-workgroup kernel
+// ---- segments that stay on chip: shared state of the one-tile kernel ------------------------------------------------------
+constexpr int kOneshotSub = 8;       // packs per thread per tile
+constexpr int kOneshotBlock = 256;   // threads per workgroup: a tile is 256 * 4 * 8 = 8192 elements
 // Arrival counters.  Device-scope atomics on one address are served one after the other (some 15 ns each, measured),
 // so a segment's tiles count into kResFan counters, each on a cache line of its own, and the tile that completes one
 // of them counts into the segment's top counter.
@@ -463,10 +451,10 @@ struct LambResident {
   uint32_t* ndeferred;              // zero at kernel start
   uint32_t ntiles;
   uint32_t spin_limit;
-  uint32_t withhold;                // test hook: scales are computed but never announced, as if their sums had not arrived
+  uint32_t withhold;                // diagnostic: scales are computed but never announced, as if their sums had not arrived
 };
 
-// Runs before every launch of the resident kernels: counters and ready words to zero, every tile-sum slot to "no sum yet".
+// Runs before every launch of the one-tile kernel: counters and ready words to zero, every tile-sum slot to "no sum yet".
 __global__ void lamb_reset_kernel(uint32_t* cnt, unsigned long long* ready, int nseg, uint32_t* ndeferred, double* partials,
                                   uint32_t ntiles) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -479,208 +467,13 @@ __global__ void lamb_reset_kernel(uint32_t* cnt, unsigned long long* ready, int 
   if (i == 0) *ndeferred = 0;
 }
 
-template <int BS, int SUB>
-__device__ __forceinline__ void lamb_retire_tile(float* w, const LambTile& t, const Pack<float, 4>* park, float step_scale,
-                                                 int vec_ok) {
-#pragma unroll
-  for (int u = 0; u < SUB; u++) {
-    const uint32_t j0 = (u * BS + threadIdx.x) * 4;
-    if (j0 >= t.count) continue;
-    const Pack<float, 4> rv = park[(u * 2) * BS + threadIdx.x];
-    Pack<float, 4> wv = park[(u * 2 + 1) * BS + threadIdx.x];
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      const float x = step_scale * rv.d[e];
-      wv.d[e] = wv.d[e] - x;
-    }
-    if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-      store_stream<float, 4>(w + t.start + j0, wv);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        if (j0 + e < t.count) w[t.start + j0 + e] = wv.d[e];
-      }
-    }
-  }
-}
-
-// BS threads per workgroup, SUB packs per thread per tile: a tile is BS * 4 * SUB elements.
-template <int P, int BS, int SUB, bool SCAT>
-__global__ __launch_bounds__(BS) void lamb_resident_kernel(const SrcTable<float, (P ? P : CCN_MAX_RANKS)> g, const int nP,
-                                                           float* w, float* m, float* v, const LambLayout lay,
-                                                           double* partials, const uint64_t* __restrict__ seg_len,
-                                                           double* norms, float* scale, const LambResident rs,
-                                                           const int vec_ok, const LambPrm k) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  constexpr int kSlotPacks = SUB * 2 * BS;
-  Pack<float, 4>* park = reinterpret_cast<Pack<float, 4>*>(smem);
-  double* red = reinterpret_cast<double*>(smem + (size_t)kResDepth * kSlotPacks * sizeof(Pack<float, 4>));
-  uint32_t* bc = reinterpret_cast<uint32_t*>(red + 2 * kBlock / kWave);   // [0] last tile of its segment, [1] ready, [2] scale
-  const unsigned G = gridDim.x;
-  const unsigned rounds = (rs.ntiles + G - 1) / G;
-  bool degraded = false;   // thread 0: a wait ran out before; later waits poll once
-  LambTile prev{};         // the tile parked in the previous round
-  bool have_prev = false;
-  // A whole, aligned tile takes the pipelined path: the loads of a pack are issued before the pack before it is
-  // worked on, and those of the next tile's first pack before this tile's sums and counters are dealt with, so that
-  // the workgroup has memory traffic in flight while it synchronises.
-  // (Not for 9..CCN_MAX_RANKS ranks: two packs of up to 19 loads each do not fit the registers of two wavefronts per SIMD.)
-  auto is_fast = [&](const LambTile& x) {
-    return P > 0 && vec_ok && (x.start & 3u) == 0 && x.count == (uint32_t)(BS * 4 * SUB);
-  };
-  LambTile next{};
-  LambIn<P, 4> pre;
-  SrcTable<float, (P ? P : CCN_MAX_RANKS)> gt = g;   // buffers of the tile in `next`
-  float* wt = w;
-  if (blockIdx.x < rs.ntiles) {
-    next = lamb_tile_of(lay, blockIdx.x);
-    lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.buf, gt, wt);
-    if (is_fast(next)) lamb_pass1_load<P, 4>(pre, gt, nP, wt, m, v, next.start + threadIdx.x * 4);
-  }
-  for (unsigned it = 0; it < rounds + (kResDepth - 1); it++) {
-    const unsigned tile = blockIdx.x + it * G;
-    const bool have_tile = it < rounds && tile < rs.ntiles;
-    // Thread 0 asks for the previous tile's scale now; the answer is looked at after this round's pass 1.
-    unsigned long long early = 0;
-    if (threadIdx.x == 0 && have_prev)
-      early = __hip_atomic_load(&rs.ready[prev.seg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    LambTile t{};
-    uint32_t arrived = 0, fan_target = 0, seg_tiles = 0;
-    if (have_tile) {
-      t = next;
-      const SrcTable<float, (P ? P : CCN_MAX_RANKS)> gc = gt;   // this tile's buffers
-      float* const wc = wt;
-      Pack<float, 4>* slot = park + (size_t)(it % kResDepth) * kSlotPacks;
-      double accW = 0.0, accR = 0.0;
-      if (is_fast(t)) {
-        LambIn<P, 4> cur = pre;
-#pragma unroll
-        for (int u = 0; u < SUB; u++) {
-          const size_t e0 = t.start + (size_t)(u * BS + threadIdx.x) * 4;
-          LambIn<P, 4> nxt;
-          if (u + 1 < SUB) lamb_pass1_load<P, 4>(nxt, gc, nP, wc, m, v, e0 + BS * 4);
-          Pack<float, 4> r4, w4;
-          lamb_pass1_math<P, 4>(cur, nP, m, v, e0, t.nf, k, accW, accR, r4, w4);
-          slot[(u * 2) * BS + threadIdx.x] = r4;
-          slot[(u * 2 + 1) * BS + threadIdx.x] = w4;
-          if (u + 1 < SUB) cur = nxt;
-        }
-      } else {
-#pragma unroll
-        for (int u = 0; u < SUB; u++) {
-          const uint32_t j0 = (u * BS + threadIdx.x) * 4;
-          Pack<float, 4> r4 = {}, w4 = {};
-          if (j0 < t.count) {
-            if (vec_ok && (t.start & 3u) == 0 && j0 + 4 <= t.count) {
-              lamb_pass1_pack<P, 4>(gc, nP, wc, m, v, t.start + j0, t.nf, k, accW, accR, r4, w4);
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; e++) {
-                if (j0 + e < t.count) {
-                  Pack<float, 1> r1, w1;
-                  lamb_pass1_pack<P, 1>(gc, nP, wc, m, v, t.start + j0 + e, t.nf, k, accW, accR, r1, w1);
-                  r4.d[e] = r1.d[0];
-                  w4.d[e] = w1.d[0];
-                }
-              }
-            }
-          }
-          slot[(u * 2) * BS + threadIdx.x] = r4;
-          slot[(u * 2 + 1) * BS + threadIdx.x] = w4;
-        }
-      }
-      if (it + 1 < rounds && tile + G < rs.ntiles) {
-        next = lamb_tile_of(lay, tile + G);
-        lamb_buffers_of<P, SCAT>(lay, g, w, nP, next.buf, gt, wt);
-        if (is_fast(next)) lamb_pass1_load<P, 4>(pre, gt, nP, wt, m, v, next.start + threadIdx.x * 4);
-      }
-      const double sW = group_sum<BS>(accW, red);
-      const double sR = group_sum<BS>(accR, red + kBlock / kWave);
-      if (threadIdx.x == 0) {
-        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile, sum_bits(sW), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(reinterpret_cast<unsigned long long*>(partials) + 2 * (size_t)tile + 1, sum_bits(sR), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-        drain_vector_memory();   // the sums are in place before the count says so
-        const uint32_t seg_lo = rs.seg_tile_begin[t.seg];
-        seg_tiles = rs.seg_tile_begin[t.seg + 1] - seg_lo;
-        const uint32_t f = (tile - seg_lo) % kResFan;
-        fan_target = (seg_tiles - f + kResFan - 1) / kResFan;   // tiles of the segment that count into counter f
-        arrived = __hip_atomic_fetch_add(&rs.cnt[(size_t)t.seg * kResCntStride + (1 + f) * kResCntLine], 1u, __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT) + 1;
-      }
-    }
-    // Previous tile, if its scale was already known at the top of the round: retire it while the count comes back.
-    bool retired = !have_prev;
-    if (have_prev) {
-      if (threadIdx.x == 0) {
-        bc[1] = (uint32_t)(early >> 32);
-        bc[2] = (uint32_t)early;
-      }
-      __syncthreads();
-      if (bc[1]) {
-        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.buf), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
-                                  k.lr * __uint_as_float(bc[2]), vec_ok);
-        retired = true;
-      }
-    }
-    // The workgroup that finishes a segment's last tile computes the segment's norms and scale.
-    if (have_tile) {
-      if (threadIdx.x == 0) {
-        uint32_t last = 0;
-        if (arrived == fan_target) {   // this tile completed its fan counter
-          const uint32_t fans = seg_tiles < (uint32_t)kResFan ? seg_tiles : (uint32_t)kResFan;
-          last = __hip_atomic_fetch_add(&rs.cnt[(size_t)t.seg * kResCntStride], 1u, __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_AGENT) + 1 == fans;
-        }
-        bc[0] = last;
-      }
-      __syncthreads();
-      if (bc[0]) {
-        bool complete = false;
-        const float sc = lamb_finalize_segment<BS, true>(partials, rs.seg_tile_begin[t.seg], rs.seg_tile_begin[t.seg + 1],
-                                                         seg_len[t.seg], (int)t.seg, norms, scale, k.mode, red, rs.spin_limit,
-                                                         &complete);
-        if (threadIdx.x == 0 && complete && !rs.withhold)   // otherwise the trailing kernel adds the segment up
-          __hip_atomic_store(&rs.ready[t.seg], (1ull << 32) | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    // Previous tile, otherwise: wait for its scale, within the spin limit.  This comes after the finalize step above
-    // because the segment waited for may be the one this workgroup has just finished.
-    if (!retired) {
-      __syncthreads();   // bc[1], bc[2] were read above
-      if (threadIdx.x == 0) {
-        uint32_t budget = degraded ? 0u : rs.spin_limit;
-        unsigned long long word;
-        while (((word = __hip_atomic_load(&rs.ready[prev.seg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
-          if (budget == 0) break;
-          budget--;
-          __builtin_amdgcn_s_sleep(4);
-        }
-        if ((word >> 32) == 0) {
-          degraded = true;
-          const uint32_t at = __hip_atomic_fetch_add(rs.ndeferred, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          rs.deferred[at] = blockIdx.x + (it - 1) * G;
-        }
-        bc[1] = (uint32_t)(word >> 32);
-        bc[2] = (uint32_t)word;
-      }
-      __syncthreads();
-      if (bc[1])
-        lamb_retire_tile<BS, SUB>(lamb_weights_of<SCAT>(lay, w, prev.buf), prev, park + (size_t)((it - 1) % kResDepth) * kSlotPacks,
-                                  k.lr * __uint_as_float(bc[2]), vec_ok);
-    }
-    __syncthreads();   // bc and the retired slot are reused by the next round
-    prev = t;
-    have_prev = have_tile;
-  }
-}
-
-// ---- one tile per workgroup, no persistent loop ----------------------------------------------------------------------
-// The same protocol with the hardware's dispatcher in place of the round-robin walk: workgroup b runs pass 1 on tile b
-// (SUB packs per thread), keeps the tile's r in registers and its old w in LDS, counts itself in, waits (within the spin
-// limit) for the segment's scale and writes w.  Workgroups are dispatched in tile order, so the tiles a waiting
-// workgroup depends on are already running; a tile that runs out of patience goes onto the deferred list as above.
+// ---- one tile per workgroup ----------------------------------------------------------------------------------------------
+// Workgroup b runs pass 1 on tile b (SUB packs per thread), keeps the tile's r in registers and its old w in LDS, counts
+// itself in, waits (within the spin limit) for the segment's scale and writes w.  The workgroup that finishes a segment's
+// last tile adds the segment's tile sums up and publishes the scale.  Workgroups are dispatched in tile order, so the
+// tiles a waiting workgroup depends on are already running.  Every wait is bounded: a tile whose segment is not ready
+// within the spin limit goes onto a deferred list, and a trailing kernel finishes it from the stored m and v (w is still
+// the old one), so the result is the same whatever the scheduling and every workgroup exits.
 // G = uint16_t: fp16 gradients and an fp16 copy of the new weights in halfw (flat arrays only).
 template <int P, int BS, int SUB, bool SCAT, class G = float>
 __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void lamb_oneshot_kernel(const SrcTable<G, (P ? P : CCN_MAX_RANKS)> g, const int nP,
@@ -775,7 +568,7 @@ __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(3, 3))) void
       __hip_atomic_store(&rs.ready[t.seg], (1ull << 32) | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (threadIdx.x == 0) {
-    uint32_t budget = rs.spin_limit / 4;   // polls are four times as far apart as in the persistent kernel
+    uint32_t budget = rs.spin_limit / 4;
     unsigned long long word;
     while (((word = __hip_atomic_load(&rs.ready[t.seg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) == 0) {
       if (budget == 0) break;
@@ -923,21 +716,19 @@ struct ccn_lamb_plan {
   uint32_t* group_begin = nullptr;      // [ngroups+1] tile index where each group starts
   uint32_t* seg_group_begin = nullptr;  // [nseg+1]
   double* folded = nullptr;             // [2*ngroups]
-  // resident part: tiles of res_block * 4 * res_sub elements of the other segments
-  int res_block = 0;              // 64 or kBlock
-  unsigned res_grid = 0, res_lds = 0;
+  // on-chip part: tiles of kOneshotBlock * 4 * kOneshotSub elements of the other segments
+  unsigned res_lds = 0;
   uint32_t res_ntiles = 0;
   uint64_t res_uniform_seg_len = 0;
-  uint32_t spin_limit = 0;
-  uint32_t withhold = 0;          // CCN_LAMB_WITHHOLD=1: test hook, see LambResident
+  uint32_t spin_limit = 0;        // bound of the one-tile kernel's waits (CCN_LAMB_KNOB_SPIN_LIMIT)
+  uint32_t withhold = 0;          // CCN_LAMB_KNOB_WITHHOLD: diagnostic, see LambResident
+  bool force_two_pass = false;    // CCN_LAMB_KNOB_TWO_PASS: every step runs on the two-pass twin
   LambTile* rtiles = nullptr;
   uint32_t* seg_rtile_begin = nullptr;
   double* rpartials = nullptr;
-  int res_sub = 0;                // packs per thread per tile
   uint32_t* sync = nullptr;       // cnt[nseg], ndeferred
   unsigned long long* ready = nullptr;
   uint32_t* deferred = nullptr;
-  int occupancy[CCN_MAX_RANKS + 1] = {0};   // resident workgroups per CU by rank count, 0 = not asked yet
   // scattered buffers: the segments' gradient and weight pointers, moved back by the segment's first element index
   std::vector<uint64_t> seg_start;
   int nbuf = 0;                         // buffers of the scattered layout (== nseg unless segments are made of several)
@@ -946,31 +737,12 @@ struct ccn_lamb_plan {
   const void** ptr_pinned = nullptr;
   std::vector<const void*> ptr_shadow;  // what the device table holds
   int ptr_ranks = 0;
-  // fp16 gradients: a plan over the same segments with every segment on the two-pass path; made on first use
+  // a plan over the same segments with every segment on the two-pass path (fp16 gradients with segments too long to
+  // stay on chip; CCN_LAMB_KNOB_TWO_PASS); made on first use
   ccn_lamb_plan* two_pass_twin = nullptr;
-  bool oneshot = false;   // resident segments run lamb_oneshot_kernel (one tile per workgroup) instead of the persistent kernel
 };
 
 namespace {
-
-long env_long(const char* name, long dflt) {
-  const char* e = std::getenv(name);
-  if (!e || !*e) return dflt;
-  char* end = nullptr;
-  const long x = std::strtol(e, &end, 10);
-  return end && *end == 0 ? x : dflt;
-}
-
-// Calls body(integral_constant<BS>, integral_constant<SUB>) for a supported resident-kernel shape; false otherwise.
-template <class Body>
-bool with_resident_shape(int block, int sub, Body body) {
-  switch (block * 10 + sub) {
-#define CCN_SHAPE(B, S) case B * 10 + S: body(std::integral_constant<int, B>{}, std::integral_constant<int, S>{}); return true;
-    CCN_SHAPE(64, 4) CCN_SHAPE(256, 4)
-#undef CCN_SHAPE
-    default: return false;
-  }
-}
 
 // Calls body(integral_constant<P>) with the rank count as a compile-time constant (0 = 9..CCN_MAX_RANKS, looped).
 template <class Body>
@@ -983,26 +755,7 @@ void with_rank_count(int P, Body body) {
   }
 }
 
-// Workgroups of the resident kernel for P ranks that one CU holds at once with `lds` bytes of LDS each (0 on error).
-int resident_occupancy(int P, int block, int sub, unsigned lds) {
-  int occ = 0;
-  with_rank_count(P, [&](auto ptag) {
-    with_resident_shape(block, sub, [&](auto bstag, auto subtag) {
-      auto* fn = lamb_resident_kernel<decltype(ptag)::value, decltype(bstag)::value, decltype(subtag)::value, false>;
-      if (lds > 64 * 1024 &&
-          hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
-        (void)hipGetLastError();
-        return;
-      }
-      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, block, lds) != hipSuccess) {
-        (void)hipGetLastError();
-        occ = 0;
-      }
-    });
-  });
-  return occ;
-}
-
+// Workgroups of the one-tile kernel for P ranks that one CU holds at once with `lds` bytes of LDS each (0 on error).
 int oneshot_occupancy(int P, unsigned lds) {
   int occ = 0;
   with_rank_count(P, [&](auto ptag) {
@@ -1074,54 +827,17 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
 
-  // Shape of the resident kernels.  CCN_LAMB_RESIDENT=0 sends every segment down the two-pass path; CCN_LAMB_ONESHOT=0
-  // selects the persistent kernel instead of the one-tile-per-workgroup kernel; CCN_LAMB_RES_BLOCK (64 | 256) and
-  // CCN_LAMB_RES_WGS (workgroups per CU) shape the persistent kernel; CCN_LAMB_SPIN bounds the waits of both.  All of
-  // them are for tuning and tests.
-  const bool resident_wanted = !two_pass_only && env_long("CCN_LAMB_RESIDENT", 1) != 0;
-  int res_block = (int)env_long("CCN_LAMB_RES_BLOCK", kBlock);
-  if (res_block != kWave && res_block != kBlock) res_block = kBlock;
-  const bool oneshot = resident_wanted && env_long("CCN_LAMB_ONESHOT", 1) != 0;
-  if (oneshot) res_block = kOneshotBlock;
-  const int res_sub = oneshot ? kOneshotSub : kResSub;
-  int lds_limit = 0;
-  if (hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, di->device) != hipSuccess) lds_limit = 65536;
-  auto lds_need = [&](int bs) {   // parked packs (r and w in two slots, or w alone), the reduction scratch, three flags
-    return (oneshot ? (size_t)bs * res_sub * 16 : (size_t)kResDepth * bs * 4 * res_sub * 8) + 2 * (kBlock / kWave) * sizeof(double) + 16;
-  };
-  if (lds_need(res_block) > (size_t)lds_limit) res_block = kWave;
-  const uint64_t res_tile = (uint64_t)res_block * 4 * res_sub;
-  const size_t res_need = lds_need(res_block);
-  long res_wgs = env_long("CCN_LAMB_RES_WGS", (long)(kLdsPerCu / res_need));
-  const long wgs_max = (long)(kLdsPerCu / res_need);
-  if (res_wgs < 1) res_wgs = 1;
-  if (res_wgs > wgs_max) res_wgs = wgs_max;
-  // Keep to even counts: with 3 workgroups of 52 KiB per CU the kernel ran into its spin limit (measured), as it
-  // does when part of the grid is not resident, although the occupancy query below reports 3; 2, 4, 6 and 8 are fine.
-  if (res_wgs > 1) res_wgs &= ~1L;
-  // LDS request that lets res_wgs workgroups, and no more where the device's limits allow, share a CU: the whole grid
-  // is then resident at once and evenly spread.  The runtime's occupancy figure has the last word (LDS is handed out
-  // in blocks): shrink the request until res_wgs fit, or settle for the workgroups that do.
-  unsigned res_lds = (unsigned)((kLdsPerCu / (size_t)res_wgs) & ~(size_t)1023);
-  if (res_lds > (unsigned)lds_limit) res_lds = (unsigned)lds_limit;
-  int occ = 0;
-  if (oneshot) {   // registers, not LDS, decide how many of these share a CU
-    res_lds = (unsigned)((res_need + 1023) & ~(size_t)1023);
-    occ = oneshot_occupancy(8, res_lds);
-    res_wgs = occ;
-  } else {
-    occ = resident_occupancy(8, res_block, res_sub, res_lds);
-    while (occ > 0 && occ < res_wgs && res_lds >= res_need + 1024) {
-      res_lds -= 1024;
-      occ = resident_occupancy(8, res_block, res_sub, res_lds);
-    }
-    if (occ > 0 && occ < res_wgs) res_wgs = occ;
-  }
+  // Shape of the one-tile kernel: registers, not LDS, decide how many of its workgroups share a CU.
+  const bool resident_wanted = !two_pass_only;
+  const uint64_t res_tile = (uint64_t)kOneshotBlock * 4 * kOneshotSub;
+  // the parked w packs, the reduction scratch, three flags
+  const size_t res_need = (size_t)kOneshotBlock * kOneshotSub * 16 + 2 * (kBlock / kWave) * sizeof(double) + 16;
+  const unsigned res_lds = (unsigned)((res_need + 1023) & ~(size_t)1023);
+  const int occ = resident_wanted ? oneshot_occupancy(8, res_lds) : 0;
   const bool resident_ok = occ > 0;
-  const unsigned res_grid_full = (unsigned)di->cu_count * (unsigned)res_wgs;
-  // Tiles a resident segment may have: what the persistent grid can park, or half of what the GPU runs at once of the
-  // one-tile workgroups (a segment's waiting tiles must leave room for the ones that complete it).
-  const uint64_t res_cap_tiles = oneshot ? res_grid_full / 2 : (uint64_t)kResDepth * res_grid_full;
+  // Tiles a segment may have to stay on chip: half of what the GPU runs at once of the one-tile workgroups (a segment's
+  // waiting tiles must leave room for the ones that complete it).
+  const uint64_t res_cap_tiles = (uint64_t)di->cu_count * (uint64_t)(occ > 0 ? occ : 0) / 2;
 
   std::vector<LambTile> tiles, rtiles;
   std::vector<uint32_t> begin((size_t)nseg + 1), rbegin((size_t)nseg + 1);
@@ -1179,15 +895,10 @@ static int lamb_plan_create(const size_t* seg_offsets, int nseg, bool two_pass_o
   p->buf_start.assign(buf_offsets, buf_offsets + nbuf);
   p->ntiles = tiles.size();
   p->uniform_seg_len = (all_two_pass && uniform % kLambTile == 0) ? uniform : 0;
-  p->res_block = res_block;
-  p->res_sub = res_sub;
   p->res_ntiles = (uint32_t)rtiles.size();
   p->res_uniform_seg_len = (all_resident && uniform % res_tile == 0) ? uniform : 0;
-  p->res_grid = p->res_ntiles < res_grid_full ? p->res_ntiles : res_grid_full;
   p->res_lds = res_lds;
-  p->oneshot = oneshot;
-  p->spin_limit = (uint32_t)env_long("CCN_LAMB_SPIN", 1 << 15);
-  p->withhold = env_long("CCN_LAMB_WITHHOLD", 0) != 0 ? 1u : 0u;
+  p->spin_limit = 1u << 15;
   hipError_t e = hipSuccess;
   auto alloc = [&](void** ptr, size_t bytes) { if (e == hipSuccess) e = hipMalloc(ptr, bytes ? bytes : 16); };
   auto upload = [&](void* dst, const void* src, size_t bytes) {
@@ -1255,6 +966,18 @@ int ccn_lamb_plan_create_parented(const size_t* buf_sizes, const size_t* buf_par
 
 namespace {
 
+// A plan over the same segments and buffers with every segment on the two-pass path, made on first use.
+int make_two_pass_twin(ccn_lamb_plan* plan) {
+  if (plan->two_pass_twin) return CCN_OK;
+  std::vector<size_t> offs(plan->seg_start.begin(), plan->seg_start.end()), boffs(plan->buf_start.begin(), plan->buf_start.end());
+  offs.push_back(plan->N);
+  boffs.push_back(plan->N);
+  return lamb_plan_create(offs.data(), plan->nseg, true, &plan->two_pass_twin, boffs.data(), plan->nbuf);
+}
+
+int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, float* const* w_seg, float* m, float* v, float lr,
+              float beta1, float beta2, float eps, float wd, int step, int mode, void* stream);
+
 // Brings the plan's device table of per-buffer pointers in line with the caller's; copies (and waits for the copy, so
 // that the staging buffer can be reused) only when they have changed since the last call.  Returns whether every
 // pointer, moved back by its buffer's first element index, is 16-byte aligned.
@@ -1299,6 +1022,16 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
   int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
   if (di->device != plan->device) return CCN_EINVAL;
+  if (plan->force_two_pass && (plan->res_ntiles || plan->two_pass_twin)) {
+    rc = make_two_pass_twin(plan);
+    if (rc != CCN_OK) return rc;
+    rc = lamb_step(plan->two_pass_twin, g, P, w_flat, w_seg, m, v, lr, beta1, beta2, eps, wd, step, mode, stream);
+    if (rc != CCN_OK) return rc;
+    // the norms land in the caller's plan, where ccn_lamb_plan_norms reads them
+    CCN_HIP(hipMemcpyAsync(plan->norms, plan->two_pass_twin->norms, 2 * (size_t)plan->nseg * sizeof(double),
+                           hipMemcpyDeviceToDevice, as_stream(stream)));
+    return CCN_OK;
+  }
   float* const w = w_flat;   // null for scattered buffers: the kernels then take every weight pointer from the table
 
   LambPrm k;
@@ -1343,7 +1076,7 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
     lay.tiles = plan->rtiles;
     lay.seg_len = plan->res_uniform_seg_len;
     lay.seg_len_f = (float)plan->res_uniform_seg_len;
-    lay.tile = (uint32_t)(plan->res_block * 4 * plan->res_sub);
+    lay.tile = (uint32_t)(kOneshotBlock * 4 * kOneshotSub);
     lay.gtab = gtab;
     lay.wtab = wtab;
     lay.nbuf = (uint32_t)plan->nbuf;
@@ -1362,57 +1095,21 @@ int lamb_step(ccn_lamb_plan* plan, const float* const* g, int P, float* w_flat, 
                          rs.ndeferred, plan->rpartials, plan->res_ntiles);
     }
     CCN_HIP(hipGetLastError());
-    if (plan->oneshot) {
-      with_ranks([&](auto ptag) {
-        constexpr int PP = decltype(ptag)::value;
-        const auto tbl = table(ptag);
-        hipLaunchKernelGGL((scattered ? lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, true> : lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, false>),
-                           dim3(plan->res_ntiles), dim3(kOneshotBlock), plan->res_lds, s, tbl, P, w, (uint16_t*)nullptr, m, v, lay, plan->rpartials,
-                           (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
-      });
-      CCN_HIP(hipGetLastError());
-      const unsigned dg = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
-      hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<kOneshotBlock, kOneshotSub, true> : lamb_deferred_kernel<kOneshotBlock, kOneshotSub, false>),
-                         dim3(dg), dim3(kOneshotBlock), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v, lay, plan->scale,
-                         (const unsigned long long*)plan->ready, (const double*)plan->rpartials, (const uint32_t*)plan->seg_rtile_begin,
-                         (const uint64_t*)plan->seg_len, plan->norms, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
-                         vec_ok, k);
-      CCN_HIP(hipGetLastError());
-    } else {
-    // The wait in the kernel is bounded either way, but it only pays when the whole grid is resident.
-    if (plan->occupancy[P] == 0) plan->occupancy[P] = resident_occupancy(P, plan->res_block, plan->res_sub, plan->res_lds);
-    const int occ = plan->occupancy[P];
-    if (occ < 1) return CCN_EHIP;
-    const unsigned fit = (unsigned)occ * (unsigned)di->cu_count;
-    const unsigned rgrid = plan->res_grid < fit ? plan->res_grid : fit;
-    const unsigned dgrid = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
     with_ranks([&](auto ptag) {
       constexpr int PP = decltype(ptag)::value;
       const auto tbl = table(ptag);
-      with_resident_shape(plan->res_block, plan->res_sub, [&](auto bstag, auto subtag) {
-        constexpr int BS = decltype(bstag)::value;
-        constexpr int SUB = decltype(subtag)::value;
-        auto* flat = lamb_resident_kernel<PP, BS, SUB, false>;
-        auto* scat = lamb_resident_kernel<PP, BS, SUB, true>;
-        if (scattered && plan->res_lds > 64 * 1024 &&
-            hipFuncSetAttribute((const void*)scat, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan->res_lds) != hipSuccess)
-          return;   // the launch below then fails and reports
-        hipLaunchKernelGGL(scattered ? scat : flat, dim3(rgrid), dim3(BS), plan->res_lds, s, tbl, P, w, m, v, lay,
-                           plan->rpartials, (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
-      });
+      hipLaunchKernelGGL((scattered ? lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, true> : lamb_oneshot_kernel<PP, kOneshotBlock, kOneshotSub, false>),
+                         dim3(plan->res_ntiles), dim3(kOneshotBlock), plan->res_lds, s, tbl, P, w, (uint16_t*)nullptr, m, v, lay, plan->rpartials,
+                         (const uint64_t*)plan->seg_len, plan->norms, plan->scale, rs, vec_ok, k);
     });
     CCN_HIP(hipGetLastError());
-    with_resident_shape(plan->res_block, plan->res_sub, [&](auto bstag, auto subtag) {
-      constexpr int BS = decltype(bstag)::value;
-      constexpr int SUB = decltype(subtag)::value;
-      hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<BS, SUB, true> : lamb_deferred_kernel<BS, SUB, false>), dim3(dgrid),
-                         dim3(BS), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v, lay, plan->scale,
-                         (const unsigned long long*)plan->ready, (const double*)plan->rpartials, (const uint32_t*)plan->seg_rtile_begin,
-                         (const uint64_t*)plan->seg_len, plan->norms, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
-                         vec_ok, k);
-    });
+    const unsigned dg = plan->res_ntiles < 1024u ? plan->res_ntiles : 1024u;
+    hipLaunchKernelGGL((scattered ? lamb_deferred_kernel<kOneshotBlock, kOneshotSub, true> : lamb_deferred_kernel<kOneshotBlock, kOneshotSub, false>),
+                       dim3(dg), dim3(kOneshotBlock), 0, s, w, (uint16_t*)nullptr, (const float*)m, (const float*)v, lay, plan->scale,
+                       (const unsigned long long*)plan->ready, (const double*)plan->rpartials, (const uint32_t*)plan->seg_rtile_begin,
+                       (const uint64_t*)plan->seg_len, plan->norms, (const uint32_t*)plan->deferred, (const uint32_t*)rs.ndeferred,
+                       vec_ok, k);
     CCN_HIP(hipGetLastError());
-    }
   }
 
   if (plan->ntiles) {
@@ -1482,12 +1179,12 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
   const dim3 block(kBlock);
 
   // Every segment short enough to stay on chip: the one-tile kernel, as for fp32 gradients.
-  if (plan->oneshot && plan->ntiles == 0 && plan->res_ntiles) {
+  if (!plan->force_two_pass && plan->ntiles == 0 && plan->res_ntiles) {
     LambLayout lay;
     lay.tiles = plan->rtiles;
     lay.seg_len = plan->res_uniform_seg_len;
     lay.seg_len_f = (float)plan->res_uniform_seg_len;
-    lay.tile = (uint32_t)(plan->res_block * 4 * plan->res_sub);
+    lay.tile = (uint32_t)(kOneshotBlock * 4 * kOneshotSub);
     lay.gtab = nullptr;
     lay.wtab = nullptr;
     lay.nbuf = (uint32_t)plan->nbuf;
@@ -1524,13 +1221,8 @@ int lamb_step_f16g(ccn_lamb_plan* plan, const uint16_t* const* g, int P, float* 
     return CCN_OK;
   }
 
-  if (!plan->two_pass_twin) {
-    std::vector<size_t> offs(plan->seg_start.begin(), plan->seg_start.end()), boffs(plan->buf_start.begin(), plan->buf_start.end());
-    offs.push_back(plan->N);
-    boffs.push_back(plan->N);
-    rc = lamb_plan_create(offs.data(), plan->nseg, true, &plan->two_pass_twin, boffs.data(), plan->nbuf);
-    if (rc != CCN_OK) return rc;
-  }
+  rc = make_two_pass_twin(plan);
+  if (rc != CCN_OK) return rc;
   ccn_lamb_plan* tp = plan->two_pass_twin;
   const dim3 grid((unsigned)tp->ntiles);
   LambLayout lay;
@@ -1688,6 +1380,19 @@ int ccn_lamb_f32_static(const float* const* g, int P, float* w, float* m, float*
                      (const float*)sc->scale, vec_ok, k);
   CCN_HIP(hipGetLastError());
   return CCN_OK;
+}
+
+int ccn_lamb_plan_tune(ccn_lamb_plan* plan, int knob, long value) {
+  if (!plan || value < 0) return CCN_EINVAL;
+  switch (knob) {
+    case CCN_LAMB_KNOB_SPIN_LIMIT:
+      if (value > 0x7fffffffL) return CCN_ERANGE;
+      plan->spin_limit = (uint32_t)value;
+      return CCN_OK;
+    case CCN_LAMB_KNOB_TWO_PASS: plan->force_two_pass = value != 0; return CCN_OK;
+    case CCN_LAMB_KNOB_WITHHOLD: plan->withhold = value != 0 ? 1u : 0u; return CCN_OK;
+    default: return CCN_EINVAL;
+  }
 }
 
 int ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream) {

@@ -51,6 +51,7 @@ __device__ __forceinline__ void epilogue_load(EpiIn<NP>& in, const SrcTable<floa
 }
 // [0, 1] clamp of the reference's __hadd2_sat (NaN gives 0)
 __device__ __forceinline__ float sat01(float x) { return x > 0.0f ? (x < 1.0f ? x : 1.0f) : 0.0f; }
+__device__ __forceinline__ float f16_round(float x) { return f16_bits_to_f32(f32_to_f16_bits(x)); }
 
 // Two 16-bit halves into one word: the upper halves of lo and hi (lo in bits 0-15)
 __device__ __forceinline__ uint32_t pack_upper_halves(uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); }
@@ -91,8 +92,12 @@ __device__ __forceinline__ u32x2 epilogue_quad(f32x4 acc, const EpiIn<NP>& in, c
     } else {
       // the reference's fused kernel (nccl-overlap/src/collectives/device/reduce_kernel.h:192-213):
       // ((u < p ? sum : 0) + bias) + residual; its half specialisation adds with saturation to [0, 1]
+      // (value and bias are halves there and each __hadd2_sat rounds to half: restated for IEEE-half operands; an fp32
+      // sum of two halves converted to half is the correctly rounded half sum)
       const float d = !g ? s[e] : 0.0f;
-      y[e] = k.mode == CCN_DROPOUT_REF_NCCL_SAT ? sat01(sat01(d + bv[e]) + rs[e]) : (d + bv[e]) + rs[e];
+      if (k.mode != CCN_DROPOUT_REF_NCCL_SAT) y[e] = (d + bv[e]) + rs[e];
+      else if constexpr (F16) y[e] = sat01(f16_round(sat01(f16_round(d) + f16_round(bv[e]))) + rs[e]);
+      else y[e] = sat01(sat01(d + bv[e]) + rs[e]);
     }
   }
   u32x2 o;
@@ -448,7 +453,8 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
     tbl.p[q] = q < nPartials ? partials[q] : nullptr;
     if (q < nPartials && (!partials[q] || !aligned16(partials[q]))) return CCN_EINVAL;
   }
-  if (!aligned16(X) || !aligned16(W) || !aligned16(bias) || !aligned16(out) || (resid && !aligned16(resid))) return CCN_EINVAL;
+  // the 16-bit residual and output move 8 bytes at a time (a tile starts on a multiple of 4 columns)
+  if (!aligned16(X) || !aligned16(W) || !aligned16(bias) || !aligned8(out) || (resid && !aligned8(resid))) return CCN_EINVAL;
   EpiPrm ep;
   int rc = make_epi(p_drop, seed, mode, &ep);
   if (rc != CCN_OK) return rc;

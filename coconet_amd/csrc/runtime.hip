@@ -241,6 +241,12 @@ int ccn_event_record(void* ev, void* stream) {
   return CCN_OK;
 }
 
+int ccn_stream_wait_event(void* stream, void* ev) {
+  if (!ev) return CCN_EINVAL;
+  CCN_HIP(hipStreamWaitEvent(as_stream(stream), (hipEvent_t)ev, 0));
+  return CCN_OK;
+}
+
 int ccn_event_elapsed_ms(void* start, void* stop, float* ms) {
   if (!start || !stop || !ms) return CCN_EINVAL;
   CCN_HIP(hipEventSynchronize((hipEvent_t)stop));

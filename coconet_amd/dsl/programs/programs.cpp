@@ -1,6 +1,6 @@
 // DSL programs for the benchmark configurations, written against the CoCoNet API.
 //   ccn-programs <program> <schedule> [output.hip]
-// program: sgd | biasadd | clipsgd | reduction | adam | adamf16 | lamb | mlp | mlpepi
+// program: sgd | biasadd | biasstage | clipsgd | reduction | adam | adamf16 | lamb | mlp | mlpepi
 // schedule: unfused | fused (adamf16, mlpepi: fused only)
 #include <dsl.hpp>
 #include <pipeline.hpp>
@@ -34,6 +34,22 @@ static void biasadd(bool fused, const std::string& out) {
   Stage wnew = Update(w, w - lr * (gsum + b));
   Pipeline pl("biasadd", {g, w, b, lr}, {wnew});
   if (fused) pl.fuse({gsum, wnew});
+  pl.codegen(out);
+}
+
+// The same with the per-column term a STAGE value: an Update over [H] (the bias decays first) that a kernel over [B, H]
+// reads, broadcast, from the updated tensor's buffer.  Stages of different dimensions do not fuse: unfused only.
+static void biasstage(bool fused, const std::string& out) {
+  ASSERT(!fused, "biasstage has an unfused schedule only");
+  Variable B(Int32, "B"), H(Int32, "H");
+  Variable lr(Float32, "lr"), decay(Float32, "decay");
+  Tensor g(Float32, {B, H}, Local, "g");
+  Tensor w(Float32, {B, H}, Replicated, "w");
+  Tensor b(Float32, H, Replicated, "b");
+  Stage gsum = AllReduce(Summation, g);
+  Stage bnew = Update(b, b * decay);
+  Stage wnew = Update(w, w - lr * (gsum + bnew));
+  Pipeline pl("biasstage", {g, w, b, lr, decay}, {bnew, wnew});
   pl.codegen(out);
 }
 
@@ -153,7 +169,7 @@ static void mlp(bool fused, bool epilogueOnly, const std::string& out) {
 
 int main(int argc, char** argv) {
   if (argc < 3) {
-    std::cout << "usage: " << argv[0] << " <sgd|biasadd|clipsgd|reduction|adam|adamf16|lamb|mlp|mlpepi> <unfused|fused> [output.hip]" << std::endl;
+    std::cout << "usage: " << argv[0] << " <sgd|biasadd|biasstage|clipsgd|reduction|adam|adamf16|lamb|mlp|mlpepi> <unfused|fused> [output.hip]" << std::endl;
     return 1;
   }
   const std::string prog = argv[1], sched = argv[2];
@@ -162,6 +178,7 @@ int main(int argc, char** argv) {
   const std::string out = argc > 3 ? argv[3] : prog + "-" + sched + ".hip";
   if (prog == "sgd") sgd(fused, out);
   else if (prog == "biasadd") biasadd(fused, out);
+  else if (prog == "biasstage") biasstage(fused, out);
   else if (prog == "clipsgd") clipsgd(fused, out);
   else if (prog == "reduction") reduction(fused, out);
   else if (prog == "adam") adam(fused, out);

@@ -156,7 +156,7 @@ struct BodyBuilder {
 
   // Reads `array`, whose values have dimensions `dims`, inside this kernel: at the element index when the dimensions
   // are the kernel's, modulo its element count when they are a trailing part of them (the front end has checked that).
-  std::string read(const std::string& array, const std::string& hint, const NodePtr& owner) {
+  std::string read(const std::string& array, const std::string& hint, const NodePtr& owner, bool f32 = true) {
     if (owner->dims == domain || owner->dims.empty()) return input(array, hint);
     ASSERT(owner->dims.size() < domain.size() &&
                std::equal(owner->dims.begin(), owner->dims.end(), domain.end() - (long)owner->dims.size()),
@@ -164,7 +164,11 @@ struct BodyBuilder {
     bool known = false;
     for (auto& b : body.bcArrays) known = known || b.first == array;
     if (!known) body.bcArrays.push_back({array, count_expr(owner)});
-    return "s.bc_" + hint + "[idx % s.bcn_" + hint + "]";
+    // the broadcast pointer is declared and filled as a const float* named after the ARRAY (a stage's buffer may be
+    // another tensor or an S<k> buffer, not the stage's own name)
+    ASSERT(f32, "HIP target: broadcast operand '" << hint << "' must hold Float32 elements");
+    const std::string field = array.substr(0, array.find('['));
+    return "s.bc_" + field + "[idx % s.bcn_" + field + "]";
   }
 
   std::string input(const std::string& array, const std::string& hint) {
@@ -235,7 +239,9 @@ struct BodyBuilder {
         }
         ASSERT(!inGroup.count(k) || phase2, "stage " << n->name << " used before it is computed");
         ASSERT(prog.stageBuf.count(k), "stage " << n->name << " has no buffer but is read by another kernel");
-        return stageValue[k] = read(prog.stageBuf[k], n->name, n);
+        const NodePtr& def = n->args[0];
+        const bool f32 = !(def->kind == Kind::Update && def->args[0]->elem == Float16);
+        return stageValue[k] = read(prog.stageBuf[k], n->name, n, f32);
       }
       case Kind::Update:
       case Kind::Norm:
@@ -882,6 +888,10 @@ std::string generateHIP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   o << ind << "if (dump__) {\n";
   for (auto& t : updated)
     o << ind << "  ccn_gen::dump(dump__, \"" << t << "\", " << t << ", " << count_expr(*std::find_if(prog.tensors.begin(), prog.tensors.end(), [&](const NodePtr& q) { return q->name == t; })) << ");\n";
+  // ... and every output stage that lives in a buffer of its own (a final value no Update writes back)
+  for (int k : prog.ownBuffers)
+    if (p.isOutput(k))
+      o << ind << "  ccn_gen::dump(dump__, \"" << p.stages()[k]->name << "\", " << p.stages()[k]->name << ", " << count_expr(p.stages()[k]) << ");\n";
   o << ind << "}\n";
   o << ind << "CCNCHECK(ccn_stream_sync(stream));\n";
   for (auto& t : prog.tensors) {

@@ -61,6 +61,8 @@ int  ccn_stream_sync(void* stream);
 int  ccn_event_create(void** ev);
 int  ccn_event_destroy(void* ev);
 int  ccn_event_record(void* ev, void* stream);
+int  ccn_stream_wait_event(void* stream, void* ev);   /* work queued on `stream` after this call starts after `ev` (the
+                                                         cudaStreamWaitEvent of the overlapped schedules' two streams) */
 int  ccn_event_elapsed_ms(void* start, void* stop, float* ms);        /* synchronises on `stop` */
 int  ccn_last_hip_error(void);
 const char* ccn_strerror(int code);
@@ -209,6 +211,19 @@ int  ccn_lamb_f32_static(const float* const* g, int P, float* w, float* m, float
                          double* norms, void* stream);
 /* copies W_b, R_b of the last LAMB step on this plan to a HOST array of 2*nseg doubles (synchronises) */
 int  ccn_lamb_plan_norms(ccn_lamb_plan* plan, double* norms_host, void* stream);
+/* Tuning and diagnostics of a plan (no counterpart in the reference; results do not depend on any of them beyond the
+ * association of the float64 norm sums).  Takes effect from the next step on.  value >= 0.
+ *   CCN_LAMB_KNOB_SPIN_LIMIT  how long a tile of the on-chip kernel waits for its segment's scale before it leaves its
+ *                             update to the trailing kernel (default 32768 polls; 0: every tile is finished by the
+ *                             trailing kernel, what a GPU shared with other work degrades to)
+ *   CCN_LAMB_KNOB_TWO_PASS    non-zero: every segment takes the two streaming passes, also those short enough to stay on
+ *                             chip (the first step after setting it makes a second tile table: it allocates)
+ *   CCN_LAMB_KNOB_WITHHOLD    diagnostic: non-zero makes the on-chip kernel compute its scales but never announce them,
+ *                             as if a tile sum had not arrived in time, so that the trailing kernel adds every segment up */
+#define CCN_LAMB_KNOB_SPIN_LIMIT 0
+#define CCN_LAMB_KNOB_TWO_PASS   1
+#define CCN_LAMB_KNOB_WITHHOLD   2
+int  ccn_lamb_plan_tune(ccn_lamb_plan* plan, int knob, long value);
 
 /* ---- model-parallel MLP out-projection, one rank's K-slice, epilogue fused into the GEMM write-back:
  *      out = bf16( dropout( X[MxK].W[KxN] + sum_q partials[q] + bias[col] ) + resid )
@@ -242,7 +257,10 @@ int  ccn_bias_dropout_residual(const float* acc, const float* const* partials, i
  *        CCN_DROPOUT_REF_NCCL      out = ((u < p ? s : 0) + b) + r             the reference's fused kernel, FuncDropout<T>
  *                                  (nccl-overlap/src/collectives/device/reduce_kernel.h:192-197, common_kernel.h:1037-1057)
  *        CCN_DROPOUT_REF_NCCL_SAT  out = sat(sat((u < p ? s : 0) + b) + r), sat = clamp to [0,1], as its half
- *                                  specialisation adds with __hadd2_sat (reduce_kernel.h:199-213)
+ *                                  specialisation adds with __hadd2_sat (reduce_kernel.h:199-213).  The IEEE-half entry
+ *                                  points (_f16_ex) also reproduce its roundings: s and b rounded to half, a rounding
+ *                                  to half after each add.  The bfloat16 ones (no counterpart there) add in fp32 and
+ *                                  round once.
  *      The reference's forms take p in [0,1]: p = 0 keeps nothing, p = 1 everything.
  *      first_row (epilogue call): row of the whole output that row 0 of this call is, for calls that cover a band of
  *      rows each (one rank's slice): the mask of an element depends on its index in the whole output only. ---- */

@@ -91,8 +91,14 @@ def _declare(L):
     L.orc_mlp_outproj_mode.argtypes = [_vp, _vp, _pp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, C.c_uint64, _i]
     L.orc_mlp_outproj_typed.restype = None
     L.orc_mlp_outproj_typed.argtypes = [_vp, _vp, _pp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, C.c_uint64, _i, _i]
+    L.orc_dsl_lamb_f32.restype = None
+    L.orc_dsl_lamb_f32.argtypes = [_pp, _i, _vp, _vp, _vp, _vp, C.c_size_t, _f, _f, _f, _f, _f, _f, _i, _f, _vp]
+    L.orc_mlp_outproj_rows.restype = None
+    L.orc_mlp_outproj_rows.argtypes = [_vp, _vp, _pp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, C.c_uint64, _i, _i, _vp]
     L.orc_epilogue_value.restype = _f
     L.orc_epilogue_value.argtypes = [_f, _f, _f, _i, _f, _i]
+    L.orc_epilogue_value_typed.restype = _f
+    L.orc_epilogue_value_typed.argtypes = [_f, _f, _f, _i, _f, _i, _i]
 
 
 def _ptr(a, dtype):
@@ -174,6 +180,20 @@ def pseudo_adam_f32(g, w, m, v, lr, beta1, beta2):
     lib().orc_pseudo_adam_f32(p, len(g), _ptr(w, f32), _ptr(m, f32), _ptr(v, f32), w.size, lr, beta1, beta2)
 
 
+def dsl_lamb_f32(g, w, m, v, lr, beta1, beta2, gamma, c1=None, c2=None, eps=None):
+    """The DSL example's LAMB (examples/lamb/lamb.cpp:20-28): m, v updated in place; returns (new weights, (rNorm, wNorm)).
+    c1, c2 default to the example's fp32 (1 - beta); eps=None leaves the square root alone as the example does."""
+    one = np.float32(1)
+    c1 = np.float32(one - np.float32(beta1)) if c1 is None else np.float32(c1)
+    c2 = np.float32(one - np.float32(beta2)) if c2 is None else np.float32(c2)
+    p, _k = _ptrs(g, f32)
+    out = np.empty_like(w)
+    norms = np.empty(2, np.float32)
+    lib().orc_dsl_lamb_f32(p, len(g), _ptr(w, f32), _ptr(m, f32), _ptr(v, f32), _ptr(out, f32), w.size, lr, beta1, beta2,
+                           float(c1), float(c2), 0.0 if eps is None else eps, 0 if eps is None else 1, gamma, _ptr(norms, f32))
+    return out, norms
+
+
 def fused_adam_a3(g16, w, m, v, halfw, lr, beta1, beta2):
     p, _k = _ptrs(g16, u16)
     lib().orc_fused_adam_a3(p, len(g16), _ptr(w, f32), _ptr(m, f32), _ptr(v, f32), _ptr(halfw, u16), w.size,
@@ -242,21 +262,30 @@ def dropout_mask(seed, first_idx, n, p_drop):
     return keep
 
 
-def epilogue_value(s, b, r, kept_inverted, p_drop, mode):
-    """One output element of the epilogue under dropout form `mode`; kept_inverted is the draw's u >= p."""
+def epilogue_value(s, b, r, kept_inverted, p_drop, mode, half=False):
+    """One output element of the epilogue under dropout form `mode`; kept_inverted is the draw's u >= p.
+    half=True: IEEE-half operands (only the saturating form then differs: it rounds to half after each add)."""
+    if half:
+        return float(lib().orc_epilogue_value_typed(s, b, r, int(kept_inverted), p_drop, mode, 1))
     return float(lib().orc_epilogue_value(s, b, r, int(kept_inverted), p_drop, mode))
 
 
-def mlp_outproj(X, W, partials, bias, resid, M, N, K, p_drop, seed, mode=0, half=False):
+def mlp_outproj(X, W, partials, bias, resid, M, N, K, p_drop, seed, mode=0, half=False, row_ids=None):
     """X, W, resid: uint16 bit patterns, bfloat16 or (half=True) IEEE half. Returns (out_bits, out_f32).
-    mode: dropout form, 0 = standard."""
+    mode: dropout form, 0 = standard.  row_ids: the M rows handed in are these rows of a larger output (the dropout
+    draw of an element depends on its index in the whole output)."""
     out = np.empty((M, N), np.uint16)
     outf = np.empty((M, N), np.float32)
     if partials:
         p, _k = _ptrs(partials, f32)
     else:
         p, _k = C.cast(None, _pp), None
-    lib().orc_mlp_outproj_typed(_ptr(X, u16), _ptr(W, u16), p, len(partials), _ptr(bias, f32),
-                                _ptr(resid, u16) if resid is not None else None, _ptr(out, u16), _ptr(outf, f32),
-                                M, N, K, p_drop, seed, mode, 1 if half else 0)
+    ids = None
+    if row_ids is not None:
+        ids = np.ascontiguousarray(row_ids, dtype=np.int64)
+        assert ids.shape == (M,)
+    lib().orc_mlp_outproj_rows(_ptr(X, u16), _ptr(W, u16), p, len(partials), _ptr(bias, f32),
+                               _ptr(resid, u16) if resid is not None else None, _ptr(out, u16), _ptr(outf, f32),
+                               M, N, K, p_drop, seed, mode, 1 if half else 0,
+                               ids.ctypes.data_as(C.c_void_p) if ids is not None else None)
     return out, outf

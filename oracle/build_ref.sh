@@ -9,15 +9,18 @@ HERE="$(cd "$(dirname "$0")" && pwd)"
 OUT="$HERE/_ref"
 mkdir -p "$OUT"
 CXX=${CXX:-g++}
-FLAGS="-std=c++14 -O1 -w -I $REF/src"
+FLAGS="-std=c++14 -O1 -w -fPIC -I $REF/src"
 for o in codegen dsl pipeline utils; do
   if [ ! -f "$OUT/$o.o" ] || [ "$REF/src/$o.cpp" -nt "$OUT/$o.o" ]; then
     $CXX $FLAGS -c "$REF/src/$o.cpp" -o "$OUT/$o.o" &
   fi
 done
 wait
+# one shared object for the generator, so that the four example programs stay a few KB each (the directory travels with
+# every GPU run although only CPU tests use it)
+$CXX -shared -s -o "$OUT/libccnref.so" "$OUT"/codegen.o "$OUT"/dsl.o "$OUT"/pipeline.o "$OUT"/utils.o
 for ex in sgd adam lamb model-parallel; do
-  $CXX $FLAGS "$REF/examples/$ex/$ex.cpp" "$OUT"/codegen.o "$OUT"/dsl.o "$OUT"/pipeline.o "$OUT"/utils.o -o "$OUT/ref-$ex" &
+  $CXX $FLAGS "$REF/examples/$ex/$ex.cpp" -L"$OUT" -lccnref -Wl,-rpath,'$ORIGIN' -s -o "$OUT/ref-$ex" &
 done
 wait
 echo "built: $(ls "$OUT" | tr '\n' ' ')"

@@ -5,6 +5,7 @@
  */
 #include "ccn_oracle.h"
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 /* ------------------------------------------------------------------------------------------------
@@ -132,6 +133,44 @@ void orc_pseudo_adam_f32(const float* const* g, int P, float* w, float* m, float
     float S5 = (w[i] - ((lr * S3) / S4));
     v[i] = S2; m[i] = S1; w[i] = S5;
   }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * The LAMB of the DSL example, examples/lamb/lamb.cpp:20-28, stage by stage as the reference's generated
+ * checker re-executes a pipeline (src/codegen.cpp:4421-4581), every stage value an fp32 array:
+ *   g1 = AllReduce(g);  m1 = Update(m, beta1*m + (1.0-beta1)*g1);  v1 = Update(v, beta2*v + (1.0-beta2)*g1*g1);
+ *   m_ = m1/(1.0-beta1);  v_ = v1/(1.0-beta2);  r = m_/Sqrt(v_) + gamma*w;
+ *   rNorm = Norm(r);  wNorm = Norm(w);  w1 = w - lr*(wNorm/rNorm)*r
+ * The constant 1.0 prints as "1" in the reference's kernels ((1 - beta1), float arithmetic); a*b*c is (a*b)*c.
+ * Norm is the L2 norm of the WHOLE tensor; the reference's generated kernel never got its accumulation (it stores the
+ * constant 1 into the norm), so the sum is build-defined: squares taken in fp32, added in float64 in index order,
+ * square root in float64, rounded to fp32.  c1, c2: what m1 and v1 are divided by (1-beta1, 1-beta2 computed in fp32
+ * for the example; a caller's bias corrections for programs that pass them).  has_eps adds eps to the square root
+ * (the example has none).  w is not written: the new weights go to w_out (the example's w1 is a stage of its own;
+ * its RS_C_AG schedules then Update w with it).  norms_out (may be NULL): rNorm, wNorm.
+ * ---------------------------------------------------------------------------------------------- */
+void orc_dsl_lamb_f32(const float* const* g, int P, const float* w, float* m, float* v, float* w_out, size_t N,
+                      float lr, float beta1, float beta2, float c1, float c2, float eps, int has_eps, float gamma,
+                      float* norms_out) {
+  float* r = (float*)malloc((N ? N : 1) * sizeof(float));
+  double r2 = 0.0, w2 = 0.0;
+  for (size_t i = 0; i < N; i++) {
+    const float g1 = reduce_at(g, P, i);
+    const float m1 = ((beta1 * m[i]) + ((1 - beta1) * g1));
+    const float v1 = ((beta2 * v[i]) + (((1 - beta2) * g1) * g1));
+    m[i] = m1;
+    v[i] = v1;
+    const float m_ = (m1 / c1);
+    const float v_ = (v1 / c2);
+    const float root = has_eps ? (sqrtf(v_) + eps) : sqrtf(v_);
+    r[i] = ((m_ / root) + (gamma * w[i]));
+    { const float x = r[i]; r2 += (double)(x * x); }
+    { const float x = w[i]; w2 += (double)(x * x); }
+  }
+  const float rNorm = (float)sqrt(r2), wNorm = (float)sqrt(w2);
+  if (norms_out) { norms_out[0] = rNorm; norms_out[1] = wNorm; }
+  for (size_t i = 0; i < N; i++) w_out[i] = (w[i] - ((lr * (wNorm / rNorm)) * r[i]));
+  free(r);
 }
 
 /* ------------------------------------------------------------------------------------------------
@@ -478,28 +517,55 @@ float orc_epilogue_value(float s, float b, float r, int kept_inverted, float p_d
   return sat01(sat01(v + b) + r);
 }
 
+/* The same with the operand type known.  For IEEE half and the saturating form, the reference's half specialisation
+ * (reduce_kernel.h:199-213) holds the value and the bias as halves and rounds to half after EACH of its two
+ * __hadd2_sat; an fp32 sum of two halves rounded to half is the correctly rounded half sum (24 >= 2*11+2 bits), so the
+ * roundings are restated with the fp32 add followed by a conversion. */
+static float f16_round(float x) { return orc_f16_to_f32(orc_f32_to_f16(x)); }
+float orc_epilogue_value_typed(float s, float b, float r, int kept_inverted, float p_drop, int mode, int half) {
+  if (!(half && mode == 3)) return orc_epilogue_value(s, b, r, kept_inverted, p_drop, mode);
+  const float v = !kept_inverted ? f16_round(s) : 0.0f;
+  const float t = f16_round(sat01(v + f16_round(b)));
+  return f16_round(sat01(t + r));
+}
+
 /* half = 0: X, W, resid and out are bfloat16; half = 1: IEEE half (the type the reference's model-parallel example
  * declares, examples/model-parallel/model-parallel.cpp:10-15).  Same arithmetic between the conversions. */
-void orc_mlp_outproj_typed(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
-                           const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
-                           int M, int N, int K, float p_drop, uint64_t seed, int mode, int half) {
+void orc_mlp_outproj_rows(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                          const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                          int M, int N, int K, float p_drop, uint64_t seed, int mode, int half, const int64_t* row_ids) {
+  /* Row i of X, partials, resid and out is row row_ids[i] of the whole output (i itself without a table): the dropout
+   * draw of an element depends on its index in the whole output.  The product of a row is accumulated in float64 in
+   * ascending k for every column (k outer, j inner: the same sum per element as a k-innermost loop, read along W's rows). */
+  double* acc = (double*)malloc((size_t)N * sizeof(double));
   for (int i = 0; i < M; i++) {
+    for (int j = 0; j < N; j++) acc[j] = 0.0;
+    for (int k = 0; k < K; k++) {
+      const uint16_t xb = X[(size_t)i * K + k];
+      const double x = half ? (double)orc_f16_to_f32(xb) : (double)orc_bf16_to_f32(xb);
+      const uint16_t* wrow = W + (size_t)k * N;
+      if (half) for (int j = 0; j < N; j++) acc[j] += x * (double)orc_f16_to_f32(wrow[j]);
+      else for (int j = 0; j < N; j++) acc[j] += x * (double)orc_bf16_to_f32(wrow[j]);
+    }
+    const uint64_t row = row_ids ? (uint64_t)row_ids[i] : (uint64_t)i;
     for (int j = 0; j < N; j++) {
-      double acc = 0.0;
-      for (int k = 0; k < K; k++) {
-        const uint16_t x = X[(size_t)i * K + k], w = W[(size_t)k * N + j];
-        acc += half ? (double)orc_f16_to_f32(x) * (double)orc_f16_to_f32(w) : (double)orc_bf16_to_f32(x) * (double)orc_bf16_to_f32(w);
-      }
-      float s = (float)acc;
+      float s = (float)acc[j];
       size_t idx = (size_t)i * N + j;
       for (int q = 0; q < nPartials; q++) s = s + partials[q][idx];
-      const int kept_inverted = orc_dropout_keep(seed, idx, p_drop);   /* u >= p; p = 0: always */
+      const int kept_inverted = orc_dropout_keep(seed, row * (uint64_t)N + (uint64_t)j, p_drop);   /* u >= p; p = 0: always */
       const float r = !resid ? 0.0f : (half ? orc_f16_to_f32(resid[idx]) : orc_bf16_to_f32(resid[idx]));
-      float y = orc_epilogue_value(s, bias[j], r, kept_inverted, p_drop, mode);
+      float y = orc_epilogue_value_typed(s, bias[j], r, kept_inverted, p_drop, mode, half);
       if (out_f32) out_f32[idx] = y;
       if (out) out[idx] = half ? orc_f32_to_f16(y) : orc_f32_to_bf16(y);
     }
   }
+  free(acc);
+}
+
+void orc_mlp_outproj_typed(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                           const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                           int M, int N, int K, float p_drop, uint64_t seed, int mode, int half) {
+  orc_mlp_outproj_rows(X, W, partials, nPartials, bias, resid, out, out_f32, M, N, K, p_drop, seed, mode, half, NULL);
 }
 
 void orc_mlp_outproj_mode(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,

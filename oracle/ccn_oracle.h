@@ -18,6 +18,9 @@
  *   orc_sgd_f32           examples/test-sgd.cu:17-18; numpy axpy identity       pinned
  *   orc_sgd_axpby_f32     nccl-overlap/samples/single-process-wX.cu:141        pinned (numpy identity)
  *   orc_pseudo_adam_f32   examples/test-adam.cu:14-38; known answer w=-1/P      pinned
+ *   orc_dsl_lamb_f32      examples/lamb/lamb.cpp:20-28 stage by stage (src/codegen.cpp:4421-4581 re-executes that way);
+ *                         all-ones closed form w1 = 1 - lr, independent float64 numpy restatement           pinned
+ *                         (the reference's generated kernel stores 1 into its norms: the norm sum is build-defined)
  *   orc_fused_adam_a3     nccl/.../reduce_kernel.h:36-68 functors; known answer w=-1, half 0xBC00; two steps by hand at
  *                         beta1 != beta2 (the first moment decays with beta2, common_kernel.h:878)          pinned
  *   orc_adam_f32          nccl-overlap/samples/multi-process-adam-scattered.cpp:112-136;
@@ -73,6 +76,10 @@ void orc_sgd_axpby_f32(const float* const* g, int P, float* w, size_t N, float a
 /* ---- the DSL example's pseudo-Adam (no sqrt, "bias correction" = divide by beta) ---- */
 void orc_pseudo_adam_f32(const float* const* g, int P, float* w, float* m, float* v, size_t N,
                          float lr, float beta1, float beta2);
+/* the DSL example's LAMB (examples/lamb/lamb.cpp:20-28), whole-tensor L2 norms; new weights to w_out, w untouched */
+void orc_dsl_lamb_f32(const float* const* g, int P, const float* w, float* m, float* v, float* w_out, size_t N,
+                      float lr, float beta1, float beta2, float c1, float c2, float eps, int has_eps, float gamma,
+                      float* norms_out);
 
 /* ---- the modified-NCCL fused mixed-precision Adam (fp16 ring sum, square in half, beta2 used for m) ---- */
 void orc_fused_adam_a3(const uint16_t* const* g, int P, float* w, float* m, float* v, uint16_t* halfw,
@@ -114,6 +121,9 @@ void orc_dropout_mask(uint64_t seed, uint64_t first_idx, size_t n, float p_drop,
  *      out_f32 (optional) receives y before the bf16 rounding. ---- */
 /* one element of the epilogue under dropout form `mode` (0 standard, 1-3 the reference's; see ccn_oracle.c) */
 float orc_epilogue_value(float s, float b, float r, int kept_inverted, float p_drop, int mode);
+/* half != 0 with mode 3: value and bias held as IEEE halves, a rounding to half after each saturating add, as the
+ * reference's FuncDropout<half> (nccl-overlap/src/collectives/device/reduce_kernel.h:199-213) */
+float orc_epilogue_value_typed(float s, float b, float r, int kept_inverted, float p_drop, int mode, int half);
 void orc_mlp_outproj_mode(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
                           const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
                           int M, int N, int K, float p_drop, uint64_t seed, int mode);
@@ -121,6 +131,11 @@ void orc_mlp_outproj(const uint16_t* X, const uint16_t* W, const float* const* p
                      const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
                      int M, int N, int K, float p_drop, uint64_t seed);
 /* the same with the 16-bit type as an argument: half = 0 bfloat16, 1 IEEE half */
+/* the same on a gathered subset of rows: row i of X, partials, resid, out is row row_ids[i] of the whole output (the
+ * dropout draw depends on the element's index there); row_ids == NULL: rows 0..M-1 */
+void orc_mlp_outproj_rows(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
+                          const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
+                          int M, int N, int K, float p_drop, uint64_t seed, int mode, int half, const int64_t* row_ids);
 void orc_mlp_outproj_typed(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
                            const float* bias, const uint16_t* resid, uint16_t* out, float* out_f32,
                            int M, int N, int K, float p_drop, uint64_t seed, int mode, int half);

@@ -83,6 +83,19 @@ def test_trailing_dimensions_broadcast(dsl_build):
     assert "NIN = 1" in text            # x alone is streamed; g comes through the rank fold
 
 
+def test_broadcast_of_a_stage_value_is_named_after_its_buffer(dsl_build, tmp_path):
+    """An Update stage over [H] read by a kernel over [B, H]: the value lives in the updated tensor's buffer, and the
+    broadcast pointer is declared, filled and read under that buffer's name (the stage's own name would not compile)."""
+    out = tmp_path / "biasstage.hip"
+    r = run(os.path.join(dsl_build, "ccn-programs"), "biasstage", "unfused", str(out))
+    assert r.returncode == 0, r.stderr
+    text = out.read_text()
+    assert "const float* bc_b; size_t bcn_b;" in text and "s.bc_b[idx % s.bcn_b]" in text
+    assert ".s.bc_b = b;" in text and ".s.bcn_b = (size_t)H;" in text
+    assert not re.search(r"bc_S\d", text)
+    assert "h.b[i0 % h.b.size()]" in text or "h.S1[i0 % h.S1.size()]" in text
+
+
 def test_matmul_chain_is_matched_by_structure_and_lowered_by_schedule(dsl_build, tmp_path):
     """The chain may be written with its sums' operands in either order and without bias and dropout; what is emitted
     follows the schedule: separate steps when nothing is fused (the reference emits a cuBLAS call, an all-reduce and

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GEN = os.path.join(ROOT, "coconet_amd", "dsl", "build", "gen")
 LINE = re.compile(r"^\{SZ: (\d+), Epochs: (\d+)((?:, \w+: [0-9.eE+-]+)+)\}$")
 
-OWN = ["sgd-fused", "sgd-unfused", "biasadd-fused", "biasadd-unfused", "clipsgd-fused", "clipsgd-unfused", "reduction-fused", "reduction-unfused", "adam-fused", "adam-unfused", "adamf16-fused", "lamb-fused", "lamb-unfused"]
+OWN = ["sgd-fused", "sgd-unfused", "biasadd-fused", "biasadd-unfused", "biasstage-unfused", "clipsgd-fused", "clipsgd-unfused", "reduction-fused", "reduction-unfused", "adam-fused", "adam-unfused", "adamf16-fused", "lamb-fused", "lamb-unfused"]
 REF = ["ref-sgd-ar-c", "ref-sgd-rs-c-ag", "ref-sgd-fuse-rs-c-ag", "ref-adam-ar-c", "ref-adam-rs-c-ag",
        "ref-adam-fuse-rs-c-ag", "ref-lamb-ar-c", "ref-lamb-rs-c-ag", "ref-lamb-fuse-rs-c-ag"]
 
@@ -55,7 +55,7 @@ def run_program(name, *args, env=None):
 @pytest.mark.parametrize("ranks", [1, 4, 8, 11])
 def test_own_programs_check_themselves(name, ranks):
     # sizes 2^10 .. 2^21 with the CPU re-execution switched on (biasadd walks a B x H matrix with B = H = 2^k)
-    if name.startswith("biasadd"):
+    if name.startswith("bias"):
         rows = run_program(name, 2, ranks, 1, 10, 1)
         assert [r[0] for r in rows] == [1 << (2 * k) for k in range(1, 11)]
     else:
@@ -64,7 +64,10 @@ def test_own_programs_check_themselves(name, ranks):
     for size, epochs, f in rows:
         assert epochs == 2 and abs(sum(v for k, v in f.items() if k != "Total") - f["Total"]) < 1e-3
     steps = set(rows[0][2]) - {"Total"}
-    assert steps == ({"kernel0"} if name.endswith("-fused") else {"AllReduce", "kernel0"})
+    if name == "biasstage-unfused":     # the [H] update and the [B, H] update are kernels of their own
+        assert steps == {"AllReduce", "kernel0", "kernel1"}
+    else:
+        assert steps == ({"kernel0"} if name.endswith("-fused") else {"AllReduce", "kernel0"})
 
 
 @pytest.mark.parametrize("name", REF)
@@ -131,6 +134,119 @@ def test_emitted_sgd_and_adam_against_the_oracle(tmp_path, schedule, n, ranks):
     for name, want in (("w", w), ("m", m), ("v", v)):
         got = np.fromfile(f"{prefix}.{name}.{n}.f32", dtype=np.float32)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), ("adam", schedule, name)
+
+
+def dumped(prefix, name, count):
+    return np.fromfile(f"{prefix}.{name}.{count}.f32", dtype=np.float32)
+
+
+def same_bits(a, b):
+    return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@pytest.mark.parametrize("schedule", ["ar-c", "rs-c-ag", "fuse-rs-c-ag"])
+@pytest.mark.parametrize("n,ranks", [(4099, 4), (4099, 7), (1 << 16, 4), (1 << 16, 7), (5, 8)])
+def test_emitted_lamb_against_the_oracle(tmp_path, schedule, n, ranks):
+    """The programs emitted from the reference's examples/lamb/lamb.cpp, every schedule, against the oracle's restatement
+    of that text (whole-tensor norms): m and v bit for bit; the norms' float64 sums are added up in another order by the
+    two-pass kernels, so the new weights are held to 1e-6.  The AR_C schedule leaves its result in a stage buffer (S8)
+    and w untouched, the RS_C_AG ones write it back into w."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    lr, b1, b2, gamma = 0.25, 0.75, 0.5, 0.125
+    env = {"CCN_GEN_N": n, "CCN_GEN_DUMP": prefix, "CCN_GEN_lr": lr, "CCN_GEN_beta1": b1, "CCN_GEN_beta2": b2, "CCN_GEN_gamma": gamma}
+    run_program(f"ref-lamb-{schedule}", 1, ranks, 10, 10, 1, env=env)
+    g, (w, m, v) = emitted_inputs(ranks, n, 3)
+    want_w, _ = orc.dsl_lamb_f32(g, w, m, v, lr, b1, b2, gamma)
+    assert same_bits(dumped(prefix, "m", n), m) and same_bits(dumped(prefix, "v", n), v), schedule
+    got_w = dumped(prefix, "S8" if schedule == "ar-c" else "w", n)
+    assert np.max(np.abs(got_w - want_w)) <= 1e-6 * np.max(np.abs(want_w)), schedule
+    assert np.max(np.abs(got_w - w)) > 1e-3                                  # ... and it is an update, not the old weights
+
+
+@pytest.mark.parametrize("name", ["lamb-fused", "lamb-unfused"])
+@pytest.mark.parametrize("n,ranks", [(4099, 3), (1 << 16, 8)])
+def test_own_lamb_program_against_the_oracle(tmp_path, name, n, ranks):
+    """The build's own LAMB program (bias corrections and epsilon passed as scalars, one global trust ratio)."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    sc = {"lr": 0.25, "beta1": 0.75, "beta2": 0.5, "eps": 0.015625, "wd": 0.125, "bias1": 0.25, "bias2": 0.5}
+    env = {"CCN_GEN_N": n, "CCN_GEN_DUMP": prefix}
+    env.update({f"CCN_GEN_{k}": x for k, x in sc.items()})
+    run_program(name, 1, ranks, 10, 10, 1, env=env)
+    g, (w, m, v) = emitted_inputs(ranks, n, 3)
+    want_w, _ = orc.dsl_lamb_f32(g, w, m, v, sc["lr"], sc["beta1"], sc["beta2"], sc["wd"], c1=sc["bias1"], c2=sc["bias2"], eps=sc["eps"])
+    assert same_bits(dumped(prefix, "m", n), m) and same_bits(dumped(prefix, "v", n), v)
+    assert np.max(np.abs(dumped(prefix, "w", n) - want_w)) <= 1e-6 * np.max(np.abs(want_w))
+
+
+@pytest.mark.parametrize("n,ranks", [(4099, 4), (1 << 16, 7), (3, 2)])
+def test_emitted_fp16_gradient_adam_against_the_oracle(tmp_path, n, ranks):
+    """The pipeline of the reference's examples/test-adamf16.cu (fp16 gradients widened and summed in fp32, the DSL
+    example's Adam, an fp16 copy of the new weights): its checker there is the loop of examples/test-adam.cu on the widened
+    gradients, i.e. the oracle's orc_pseudo_adam_f32.  Bit for bit, the fp16 copy included."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    run_program("adamf16-fused", 1, ranks, 10, 10, 1, env={"CCN_GEN_N": n, "CCN_GEN_DUMP": prefix, "CCN_GEN_lr": 1.0})
+    g = [orc.f16_to_f32(orc.f32_to_f16(splitmix_uniform(1234 + 100 + p, n))) for p in range(ranks)]
+    w, m, v = (splitmix_uniform(1234 + k, n) for k in (101, 103, 104))
+    orc.pseudo_adam_f32(g, w, m, v, 1.0, 0.5, 0.5)
+    for name, want in (("w", w), ("m", m), ("v", v)):
+        assert same_bits(dumped(prefix, name, n), want), name
+    assert same_bits(dumped(prefix, "halfw", n), orc.f16_to_f32(orc.f32_to_f16(w)))
+
+
+@pytest.mark.parametrize("name", ["reduction-fused", "reduction-unfused"])
+@pytest.mark.parametrize("n,ranks", [(4099, 4), (1 << 16, 7)])
+def test_emitted_reduction_against_a_float64_sum(tmp_path, name, n, ranks):
+    """The pipeline of the reference's examples/test-reduction.cu: S1 = w + sum_p g, S2 = the sum of S1 over the tensor,
+    w <- w - (damp * S2) * S0.  The whole-tensor sum against numpy's float64 sum rounded to fp32."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    damp = 2.0 ** -18
+    run_program(name, 1, ranks, 10, 10, 1, env={"CCN_GEN_N": n, "CCN_GEN_DUMP": prefix, "CCN_GEN_damp": damp})
+    g, (w,) = emitted_inputs(ranks, n, 1)
+    s0 = orc.reduce_f32(g)
+    s2 = np.float32(np.sum((w + s0).astype(np.float64)))
+    want = w - (np.float32(damp) * s2) * s0
+    got = dumped(prefix, "w", n)
+    assert np.max(np.abs(got - want)) <= 1e-6 * np.max(np.abs(want)) and np.max(np.abs(got - w)) > 1e-3
+
+
+@pytest.mark.parametrize("name", ["clipsgd-fused", "clipsgd-unfused"])
+def test_emitted_clipped_sgd_against_numpy(tmp_path, name):
+    """Ite and comparisons: the summed gradient clipped to [-clip, clip] element by element, bit for bit against numpy's
+    select on the oracle's fixed-order sum (uniform inputs on 4 ranks sum to (0, 4]: the upper clip at 2 cuts half)."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    n, ranks, lr, clip = 4099, 4, 0.25, 2.0
+    run_program(name, 1, ranks, 10, 10, 1, env={"CCN_GEN_N": n, "CCN_GEN_DUMP": prefix, "CCN_GEN_lr": lr, "CCN_GEN_clip": clip})
+    g, (w,) = emitted_inputs(ranks, n, 1)
+    gs = orc.reduce_f32(g)
+    c = np.float32(clip)
+    gc = np.where(gs > c, c, np.where(-c > gs, -c, gs)).astype(np.float32)
+    assert 0.2 < float((gs > c).mean()) < 0.8
+    assert same_bits(dumped(prefix, "w", n), w - np.float32(lr) * gc)
+
+
+@pytest.mark.parametrize("name", ["biasadd-fused", "biasadd-unfused", "biasstage-unfused"])
+def test_emitted_broadcast_programs_against_numpy(tmp_path, name):
+    """A [H] operand broadcast over the rows of a [B, H] update, as a tensor (biasadd) and as the value of an Update stage
+    over [H] read from the updated tensor's buffer (biasstage): bit for bit against numpy broadcasting.  B = H = 67."""
+    import oracle as orc
+    prefix = str(tmp_path / "out")
+    B = H = 67
+    ranks, lr, decay = 3, 0.25, 0.75
+    run_program(name, 1, ranks, 1, 1, 1, env={"CCN_GEN_N": B, "CCN_GEN_DUMP": prefix, "CCN_GEN_lr": lr, "CCN_GEN_decay": decay})
+    g = [splitmix_uniform(1234 + 100 + p, B * H) for p in range(ranks)]
+    w = splitmix_uniform(1234 + 101, B * H)
+    b = splitmix_uniform(1234 + 102, H)
+    if name.startswith("biasstage"):
+        b = b * np.float32(decay)
+        assert same_bits(dumped(prefix, "b", H), b)
+    gs = orc.reduce_f32(g).reshape(B, H)
+    want = w.reshape(B, H) - np.float32(lr) * (gs + b[None, :])
+    assert same_bits(dumped(prefix, "w", B * H), want.reshape(-1).astype(np.float32))
 
 
 @pytest.mark.parametrize("schedule", ["rs-c-ag", "fuse-rs-c-ag"])

@@ -164,16 +164,27 @@ def test_half_product_and_standalone_epilogue(ccn):
     parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(2)]
     bias = r.standard_normal(N, dtype=np.float32)
     resid = r.standard_normal((M, N)).astype(np.float16)
-    for mode in (0, 1, 2, 3):
+    for mode in (0, 1, 2, 3, 3):
+        if mode == 3:       # values inside and around [0, 1]: both clamps and the roundings between the two adds matter
+            acc, parts, bias = acc * np.float32(0.2), [q * np.float32(0.2) for q in parts], bias * np.float32(0.3)
         out = torch.zeros(M, N, dtype=torch.int16, device=DEV)
         ccn.bias_dropout_residual(torch.from_numpy(acc).to(DEV), [torch.from_numpy(q).to(DEV) for q in parts],
                                   torch.from_numpy(bias).to(DEV), u16_dev(resid.view(np.uint16)), out, M, N, 0.3, 7,
                                   dropout_mode=mode, half=True)
         s = (acc + parts[0]) + parts[1]
         kept = orc.dropout_mask(7, 0, M * N, 0.3).reshape(M, N)
-        y = np.array([[orc.epilogue_value(s[i, j], bias[j], np.float32(resid[i, j]), int(kept[i, j]), 0.3, mode)
+        y = np.array([[orc.epilogue_value(s[i, j], bias[j], np.float32(resid[i, j]), int(kept[i, j]), 0.3, mode, half=True)
                        for j in range(N)] for i in range(M)], np.float32)
         assert np.array_equal(bf16_host(out).reshape(M, N), y.astype(np.float16).view(np.uint16)), mode
+        if mode == 3:
+            # the reference's half specialisation rounds to half after each saturating add: float16 arithmetic throughout
+            # (numpy's, an independent library) gives the same bits, one fp32 sum rounded once does not
+            sat = lambda x: np.clip(x, np.float16(0), np.float16(1))
+            v = np.where(kept.astype(bool), np.float16(0), s.astype(np.float16))
+            assert np.array_equal(y.astype(np.float16), sat(sat(v + bias.astype(np.float16)[None, :]) + resid))
+            once = np.array([[orc.epilogue_value(s[i, j], bias[j], np.float32(resid[i, j]), int(kept[i, j]), 0.3, 3)
+                              for j in range(N)] for i in range(M)], np.float32).astype(np.float16)
+            assert (once != y.astype(np.float16)).any()
 
 
 def test_outproj_all_ones_known_answer(ccn):
@@ -295,9 +306,10 @@ def test_outproj_config5_shape_in_ieee_half(ccn):
 
 
 def test_outproj_config5_full_size(ccn):
-    """benchmark configuration 5 at full size (8192 x 1024 x 8192, 7 partials, p = 0.1, seed 0).  Checked by:
-    the exact dropout mask over all 2^26 outputs (torch recomputes nothing: dropped outputs equal the
-    residual, kept ones almost never do), and the oracle on sampled rows."""
+    """benchmark configuration 5 at full size (8192 x 1024 x 8192, 7 partials, p = 0.1, seed 0).  Checked by the oracle
+    itself on every row of three 128-row tile rows (the first, one in the middle, the last: every row position inside a
+    tile, so every wavefront and both halves of its walk, over all 64 tile columns), and over the whole output by the
+    drop rate (dropped outputs equal the residual, kept ones almost never do)."""
     M = N = 8192
     K = 1024
     gen = torch.Generator(device=DEV)
@@ -310,29 +322,78 @@ def test_outproj_config5_full_size(ccn):
     out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     ccn.mlp_outproj_bf16(X, W, parts, bias, resid, out, M, N, K, 0.1, 0)
     torch.cuda.synchronize()
-    rows = [0, 1, 127, 128, 4095, 4096, 8191]
-    keep_rows = np.stack([orc.dropout_mask(0, r * N, N, 0.1) for r in rows]).astype(bool)
-    Xh = X[rows].view(torch.int16).cpu().numpy().view(np.uint16)
+    rows = np.concatenate([np.arange(0, 128), np.arange(37 * 128, 38 * 128), np.arange(M - 128, M)])
+    ridx = torch.from_numpy(rows).to(DEV)
+    bits = lambda t: t[ridx].view(torch.int16).cpu().numpy().view(np.uint16)
+    Xh, rh, got = bits(X), bits(resid), bits(out)
     Wh = W.view(torch.int16).cpu().numpy().view(np.uint16)
-    ph = [q[rows].cpu().numpy() for q in parts]
-    rh = resid[rows].view(torch.int16).cpu().numpy().view(np.uint16)
-    got = out[rows].view(torch.int16).cpu().numpy().view(np.uint16)
-    # oracle on the sampled rows: numpy float64 GEMM for the product, then the oracle's epilogue order
-    acc = (orc.bf16_to_f32(Xh).astype(np.float64) @ orc.bf16_to_f32(Wh).astype(np.float64)).astype(np.float32)
-    s = acc
-    for q in ph:
-        s = s + q
-    t = s + bias.cpu().numpy()[None, :]
-    scale = np.float32(1.0) / (np.float32(1.0) - np.float32(0.1))
-    y = np.where(keep_rows, t * scale, np.float32(0)) + orc.bf16_to_f32(rh)
-    want = orc.f32_to_bf16(y.astype(np.float32))
+    ph = [q[ridx].cpu().numpy() for q in parts]
+    want, _ = orc.mlp_outproj(Xh, Wh, ph, bias.cpu().numpy(), rh, len(rows), N, K, 0.1, 0, row_ids=rows)
+    keep_rows = np.stack([orc.dropout_mask(0, int(r) * N, N, 0.1) for r in rows]).astype(bool)
     assert np.array_equal(got[~keep_rows], rh[~keep_rows])                 # mask exact on the sampled rows
     d = bf16_ulp_distance(got, want)
     assert d.max() <= 1 and (d > 0).mean() < 0.02
-    # over the whole output: the fraction of outputs equal to the residual is the drop rate (kept outputs equal
-    # the residual only when the scaled sum rounds away, which is rare)
+    per_row = (d > 0).reshape(3, 128, N).mean(axis=(0, 2))                 # no row position inside a tile stands out
+    assert per_row.max() < 0.03, f"in-tile row {int(per_row.argmax())}: {per_row.max():.4f} of its outputs differ"
     dropped = float((out == resid).float().mean())
     assert abs(dropped - 0.1) < 2e-3
+
+
+def test_fused_call_takes_8_byte_aligned_residual_and_output(ccn):
+    """The 16-bit residual and output of the fused call need 8-byte alignment only (they move a quad of columns at a
+    time), as the header says: both 8 bytes off a 16-byte boundary, whole-tile shape (matrix-core kernel) and an odd
+    one (any-shape kernel)."""
+    for (M, N, K) in [(128, 256, 128), (100, 36, 70)]:
+        X, W, parts, bias, resid = make_case(33, M, N, K, 2)
+        rbuf = torch.zeros(M * N + 4, dtype=torch.int16, device=DEV)
+        obuf = torch.zeros(M * N + 4, dtype=torch.int16, device=DEV)
+        rbuf[4:] = bf16_dev(resid).reshape(-1)
+        rview, oview = rbuf[4:], obuf[4:]
+        assert rview.data_ptr() % 16 == 8 and oview.data_ptr() % 16 == 8
+        ccn.mlp_outproj_bf16(bf16_dev(X), bf16_dev(W), [torch.from_numpy(q).to(DEV) for q in parts], torch.from_numpy(bias).to(DEV),
+                             rview, oview, M, N, K, 0.2, 4)
+        got = bf16_host(oview).reshape(M, N)
+        want, _ = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, 0.2, 4)
+        d = bf16_ulp_distance(got, want)
+        assert d.max() <= 1 and (d > 0).mean() < 0.03
+        assert np.array_equal(bf16_host(obuf)[:4], np.zeros(4, np.uint16))     # nothing written in front of the output
+        with pytest.raises(ccn.CoconetError) as e:                              # 4 bytes off is refused
+            ccn.mlp_outproj_bf16(bf16_dev(X), bf16_dev(W), [], torch.from_numpy(bias).to(DEV), None, obuf[2:], M, N, K, 0.0, 0)
+        assert e.value.code == ccn.CCN_EINVAL
+
+
+def test_rows_longer_than_a_buffer_descriptor_spans(ccn):
+    """N = 2^21 + 128 (whole tiles, but a row of fp32 partials is longer than the 2 GiB window the matrix-core kernel
+    addresses 128 rows through): the entry point hands over to the any-shape kernel.  Oracle on a few rows."""
+    M, K = 128, 64
+    N = (1 << 21) + 128
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(12)
+    X = torch.randn(M, K, device=DEV, generator=gen).to(torch.bfloat16)
+    W = (torch.randn(K, N, device=DEV, generator=gen) * 0.1).to(torch.bfloat16)
+    part = torch.randn(M, N, device=DEV, generator=gen)
+    bias = torch.randn(N, device=DEV, generator=gen)
+    resid = torch.randn(M, N, device=DEV, generator=gen).to(torch.bfloat16)
+    out = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+    ccn.mlp_outproj_bf16(X, W, [part], bias, resid, out, M, N, K, 0.1, 3)
+    torch.cuda.synchronize()
+    rows = np.array([0, 1, 63, 126, 127])
+    ridx = torch.from_numpy(rows).to(DEV)
+    bits = lambda t: t.view(torch.int16).cpu().numpy().view(np.uint16)
+    want, _ = orc.mlp_outproj(bits(X[ridx]), bits(W), [part[ridx].cpu().numpy()], bias.cpu().numpy(), bits(resid[ridx]),
+                              len(rows), N, K, 0.1, 3, row_ids=rows)
+    got = bits(out[ridx])
+    d = bf16_ulp_distance(got, want)
+    assert d.max() <= 1 and (d > 0).mean() < 0.02
+    keep_rows = np.stack([orc.dropout_mask(3, int(r) * N, N, 0.1) for r in rows]).astype(bool)
+    assert np.array_equal(got[~keep_rows], bits(resid[ridx])[~keep_rows])
+    dropped = float((out == resid).float().mean())
+    assert abs(dropped - 0.1) < 2e-3
+    Cd = torch.empty(M, N, device=DEV)                                          # the plain product hands over as well
+    ccn.matmul_bf16_f32(X, W, Cd, M, N, K)
+    torch.cuda.synchronize()
+    ref = X[ridx].double() @ W.double()
+    assert float((Cd[ridx].double() - ref).abs().max()) <= K * 2.0 ** -24 * float((X[ridx].double().abs() @ W.double().abs()).max())
 
 
 @pytest.mark.parametrize("case", range(8))

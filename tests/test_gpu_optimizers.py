@@ -408,34 +408,25 @@ def _lamb_compare(ccn, g, w0, segs, lr, b1, b2, eps, wd_, steps, mode, what, m0=
     return ulp_diff_f32(gw, w)
 
 
-# How a plan runs its segments is fixed when the plan is created, from these variables: the one-tile-per-workgroup
-# kernel (the default), the persistent segment-resident kernel with 256-thread or single-wavefront workgroups, each of
-# them also with a spin limit of zero (every tile whose segment is not ready at the first poll goes through the
-# deferred list), or the two-pass kernels only.
+# How a plan runs its segments: the one-tile-per-workgroup kernel for segments short enough to stay on chip (the
+# default), the same with a spin limit of zero (every tile whose segment is not ready at the first poll goes through the
+# deferred list), or the two-pass kernels only.  Knobs of ccn_lamb_plan_tune, applied to every plan the tests create.
+SPIN, TWO_PASS, WITHHOLD = 0, 1, 2
 LAMB_VARIANTS = {
     "one-tile": {},
-    "one-tile-deferred": {"CCN_LAMB_SPIN": "0"},
-    "resident": {"CCN_LAMB_ONESHOT": "0"},
-    "resident-wave": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_RES_BLOCK": "64"},
-    "deferred": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0"},
-    "deferred-wave": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "0", "CCN_LAMB_RES_BLOCK": "64"},
-    "two-pass": {"CCN_LAMB_RESIDENT": "0"},
+    "one-tile-deferred": {SPIN: 0},
+    "two-pass": {TWO_PASS: 1},
     # a patience of a poll or two: some tiles see their segment's scale in time, the others go to the trailing kernel
-    "one-tile-short-patience": {"CCN_LAMB_SPIN": "6"},
-    "resident-short-patience": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_SPIN": "3"},
+    "one-tile-short-patience": {SPIN: 6},
     # the workgroup that adds a segment up keeps the result to itself, as it does when a tile sum has not arrived: every
     # tile runs out of patience and the trailing kernel adds the segments up from the sums in memory
-    "one-tile-withheld": {"CCN_LAMB_WITHHOLD": "1", "CCN_LAMB_SPIN": "8"},
-    "resident-withheld": {"CCN_LAMB_ONESHOT": "0", "CCN_LAMB_WITHHOLD": "1", "CCN_LAMB_SPIN": "8"},
+    "one-tile-withheld": {WITHHOLD: 1, SPIN: 8},
 }
 
 
 @pytest.fixture(params=list(LAMB_VARIANTS))
-def lamb_variant(request, monkeypatch):
-    for k in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT", "CCN_LAMB_WITHHOLD"):
-        monkeypatch.delenv(k, raising=False)
-    for k, val in LAMB_VARIANTS[request.param].items():
-        monkeypatch.setenv(k, val)
+def lamb_variant(request, ccn, monkeypatch):
+    monkeypatch.setattr(ccn, "LAMB_DEFAULT_KNOBS", dict(LAMB_VARIANTS[request.param]))
     return request.param
 
 
@@ -451,16 +442,11 @@ def test_lamb_ragged_segments(ccn, mode, lamb_variant):
 
 
 @pytest.mark.parametrize("P", [1, 5, 7, 9, 16])
-@pytest.mark.parametrize("path", ["one-tile", "persistent", "two-pass"])
+@pytest.mark.parametrize("path", ["one-tile", "two-pass"])
 def test_lamb_rank_counts(ccn, monkeypatch, P, path):
     """Every rank count has its own instantiation up to 8 and a looped one beyond; segments around the 8192-element
     tile of the one-tile kernel."""
-    for name in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT"):
-        monkeypatch.delenv(name, raising=False)
-    if path == "persistent":
-        monkeypatch.setenv("CCN_LAMB_ONESHOT", "0")
-    if path == "two-pass":
-        monkeypatch.setenv("CCN_LAMB_RESIDENT", "0")
+    monkeypatch.setattr(ccn, "LAMB_DEFAULT_KNOBS", {TWO_PASS: 1} if path == "two-pass" else {})
     segs = [0, 8192, 8192 + 8191, 3 * 8192 + 5, 5 * 8192 + 5]
     N = segs[-1]
     g = grads_f32(40 + P, P, N, 1e-3)
@@ -499,14 +485,11 @@ def test_lamb_unaligned_buffers(ccn, lamb_variant):
     assert ulp_diff_f32(host(wd), w) <= 2
 
 
-@pytest.mark.parametrize("kernel,long_seg", [("one-tile", 4_000_000), ("persistent", 2_500_000)])
-def test_lamb_mixed_resident_and_two_pass(ccn, monkeypatch, kernel, long_seg):
+@pytest.mark.parametrize("long_seg", [4_000_000])
+def test_lamb_mixed_resident_and_two_pass(ccn, long_seg):
     """One segment too long to stay on chip between short ones: the long one takes the two-pass kernels, the others
-    the resident kernel, in one call.  The one-tile kernel keeps segments of up to half the tiles the GPU runs at once
-    (384 tiles of 8192 elements); the persistent kernel, held to one workgroup per CU here, 2 * 256 tiles of 4096."""
-    if kernel == "persistent":
-        monkeypatch.setenv("CCN_LAMB_ONESHOT", "0")
-        monkeypatch.setenv("CCN_LAMB_RES_WGS", "1")
+    the one-tile kernel, in one call.  The one-tile kernel keeps segments of up to half the tiles the GPU runs at once
+    (384 tiles of 8192 elements)."""
     P = 2
     segs = [0, 3000, 3000 + long_seg, 3000 + long_seg + 8192, 3000 + long_seg + 8192 + 100_001]
     N = segs[-1]
@@ -593,16 +576,7 @@ def test_lamb_full_size_segments(ccn):
         ref[b] = [float(w0[sl].double().pow(2).mean().sqrt()), float(r.pow(2).mean().sqrt())]
     assert rel_err(norms, ref) < 1e-6, rel_err(norms, ref)
     w2, m2, v2 = w0, torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
-    import os
-    saved = os.environ.get("CCN_LAMB_RESIDENT")
-    os.environ["CCN_LAMB_RESIDENT"] = "0"
-    try:
-        plan2 = ccn.LambPlan([i * seglen for i in range(nseg + 1)])
-    finally:
-        if saved is None:
-            del os.environ["CCN_LAMB_RESIDENT"]
-        else:
-            os.environ["CCN_LAMB_RESIDENT"] = saved
+    plan2 = ccn.LambPlan([i * seglen for i in range(nseg + 1)], knobs={TWO_PASS: 1})
     plan2.step(g, w2, m2, v2, 1e-3, 0.9, 0.999, 1e-6, 0.01, 1, ccn.LAMB_TRUST_RATIO)
     norms2 = plan2.norms()
     plan2.close()
@@ -684,7 +658,7 @@ def test_recorded_steps_replay_like_eager_calls(ccn):
 
 
 def test_recorded_lamb_step_replays(ccn):
-    """A LAMB step through the segment-resident kernel, recorded after one eager call and replayed twice."""
+    """A LAMB step through the one-tile kernel (segments that stay on chip), recorded after one eager call and replayed twice."""
     P, segs = 3, [0, 5000, 5000 + 40960, 5000 + 40960 + 12289]
     N = segs[-1]
     g = grads_f32(83, P, N, 1e-3)
@@ -712,9 +686,9 @@ def test_recorded_lamb_step_replays(ccn):
     stream.close()
 
 
-def test_lamb_resident_kernel_shares_the_gpu(ccn):
-    """The resident kernel assumes its whole grid is on the chip at once.  With another stream keeping the GPU busy that
-    need not hold: waits may run out and tiles go through the deferred list.  Whatever happens, the result is the same."""
+def test_lamb_on_chip_kernel_shares_the_gpu(ccn):
+    """The one-tile kernel counts on a segment's tiles running at the same time.  With another stream keeping the GPU busy
+    that need not hold: waits may run out and tiles go through the deferred list.  Whatever happens, the result is the same."""
     P, nseg, seglen = 4, 16, 1 << 20
     N = nseg * seglen
     segs = [i * seglen for i in range(nseg + 1)]
@@ -747,23 +721,20 @@ def test_lamb_resident_kernel_shares_the_gpu(ccn):
 
 
 # ---------------------------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("P,segs,shift", [(8, [0, 1 << 18], 0), (3, [0, 700, 701, 5000, 8192 + 3], 0),
-                                          (8, [0, 4096, 8192, 12288], 0), (11, [0, 1000, 70001], 0),
-                                          (2, [0, 4099], 1), (1, [0, 1], 0), (8, [0, 5 * 1024 * 4096 + 17], 0)])
-@pytest.mark.parametrize("path", ["one-tile", "one-tile-deferred", "two-pass"])
+MIXED_LAMB_SHAPES = [(8, [0, 1 << 18], 0), (3, [0, 700, 701, 5000, 8192 + 3], 0), (8, [0, 4096, 8192, 12288], 0),
+                     (11, [0, 1000, 70001], 0), (2, [0, 4099], 1), (1, [0, 1], 0)]
+# ... and one segment of more than 4096 tiles, which takes the two-pass kernels whatever the path: run once
+MIXED_LAMB_CASES = [(P, segs, shift, path) for (P, segs, shift) in MIXED_LAMB_SHAPES
+                    for path in ("one-tile", "one-tile-deferred", "two-pass")] + [(8, [0, 5 * 1024 * 4096 + 17], 0, "one-tile")]
+
+
+@pytest.mark.parametrize("P,segs,shift,path", MIXED_LAMB_CASES)
 def test_lamb_nccl_mixed_precision(ccn, monkeypatch, P, segs, shift, path):
     """The modified NCCL's LAMB with fp16 gradients: m and v bit for bit, w within the fp32 bar (the order of the
     float64 norm sums differs), the fp16 weight copy within one fp16 ulp and equal to fp16 of the kernel's own w.
     shift = 1: every array starts one element past an aligned address (scalar path).  The last case has a segment of
     more than 4096 tiles: it takes the two-pass kernels whatever the path, with its partial sums folded in two levels."""
-    for name in ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT"):
-        monkeypatch.delenv(name, raising=False)
-    if path == "one-tile-deferred":
-        monkeypatch.setenv("CCN_LAMB_SPIN", "0")
-    if path == "two-pass":
-        monkeypatch.setenv("CCN_LAMB_RESIDENT", "0")
-    if path != "one-tile" and segs[-1] > (1 << 22):
-        pytest.skip("the long segment takes the two-pass kernels in every path: run once")
+    monkeypatch.setattr(ccn, "LAMB_DEFAULT_KNOBS", {"one-tile": {}, "one-tile-deferred": {SPIN: 0}, "two-pass": {TWO_PASS: 1}}[path])
     N = segs[-1]
     g16 = [orc.f32_to_f16(x) for x in grads_f32(71 + P, P, N, 0.5)]
     w0 = weights_f32(71, N, 0.05)

@@ -628,3 +628,106 @@ def test_reference_saturating_dropout_form():
     assert orc.epilogue_value(-2.0, 0.5, 0.25, 0, 0.5, 2) == -1.25      # unsaturated: (-2 + 0.5) + 0.25
     assert orc.epilogue_value(0.25, 0.25, 0.25, 0, 0.5, 3) == 0.75 and orc.epilogue_value(0.25, 0.25, -1.0, 0, 0.5, 3) == 0.0
     assert orc.epilogue_value(float("nan"), 0.0, 0.0, 0, 0.5, 3) == 0.0  # NaN saturates to zero
+
+
+def test_saturating_form_in_half_rounds_after_each_add():
+    """FuncDropout<half> (nccl-overlap/src/collectives/device/reduce_kernel.h:199-213) holds value, bias and residual as
+    halves and each __hadd2_sat rounds to half.  Hand-computed: at 0.5 a half's spacing is 2^-11, so 0.5 + 2^-12 is a
+    tie and rounds to even (0.5) -- twice; one fp32 sum rounded once would give 0.5 + 2^-11.  numpy's float16
+    arithmetic (an independent library) rounds after each add too."""
+    h = np.float32(2.0 ** -12)
+    assert orc.epilogue_value(0.5, h, h, 0, 0.5, 3, half=True) == 0.5
+    assert orc.epilogue_value(0.5, h, h, 0, 0.5, 3) == 0.5 + 2.0 ** -11           # the fp32 form adds first, rounds never
+    # the sum itself is rounded to half before the first add (the reference's value is a half): 0.5 + 2^-13 -> 0.5
+    assert orc.epilogue_value(0.5 + 2.0 ** -13, 0.0, 0.0, 0, 0.5, 3, half=True) == 0.5
+    # the other forms do not change with the operand type
+    for mode in (0, 1, 2):
+        assert orc.epilogue_value(0.3, 0.2, 0.1, 0, 0.5, mode, half=True) == orc.epilogue_value(0.3, 0.2, 0.1, 0, 0.5, mode)
+    r = rng(62)
+    s = (r.standard_normal(4000) * 0.3).astype(np.float16)
+    b = (r.standard_normal(4000) * 0.3).astype(np.float16)
+    res = (r.standard_normal(4000) * 0.3).astype(np.float16)
+    sat = lambda x: np.clip(x, np.float16(0), np.float16(1))
+    want = sat(sat(s + b) + res)                                                   # float16 arithmetic throughout
+    got = np.array([orc.epilogue_value(float(s[i]), float(b[i]), float(res[i]), 0, 0.5, 3, half=True) for i in range(4000)])
+    assert np.array_equal(got.astype(np.float16), want) and np.array_equal(got, want.astype(np.float64))
+
+
+def test_row_subset_of_the_out_projection_equals_the_whole_call():
+    """orc.mlp_outproj(row_ids=...) on gathered rows gives the rows of the whole-output call, mask included; and the
+    product behind it is the float64 brute force whatever the loop order."""
+    r = rng(63)
+    M, N, K, nP, p = 24, 16, 40, 2, 0.4
+    X = orc.f32_to_bf16(r.standard_normal((M, K), dtype=np.float32))
+    W = orc.f32_to_bf16(r.standard_normal((K, N), dtype=np.float32))
+    parts = [r.standard_normal((M, N), dtype=np.float32) for _ in range(nP)]
+    bias = r.standard_normal(N, dtype=np.float32)
+    resid = orc.f32_to_bf16(r.standard_normal((M, N), dtype=np.float32))
+    whole, whole_f = orc.mlp_outproj(X, W, parts, bias, resid, M, N, K, p, 11)
+    rows = np.array([23, 0, 7, 8, 15])
+    sub, sub_f = orc.mlp_outproj(np.ascontiguousarray(X[rows]), W, [np.ascontiguousarray(q[rows]) for q in parts], bias,
+                                 np.ascontiguousarray(resid[rows]), len(rows), N, K, p, 11, row_ids=rows)
+    assert np.array_equal(sub, whole[rows]) and np.array_equal(sub_f, whole_f[rows])
+    # brute force, k innermost, float64: the product of one element
+    xf, wf = orc.bf16_to_f32(X).astype(np.float64), orc.bf16_to_f32(W).astype(np.float64)
+    keep = orc.dropout_mask(11, 0, M * N, p).reshape(M, N).astype(bool)
+    for (i, j) in [(0, 0), (23, 15), (7, 3)]:
+        acc = 0.0
+        for k in range(K):
+            acc += xf[i, k] * wf[k, j]
+        s = np.float32(acc)
+        for q in parts:
+            s = np.float32(s + q[i, j])
+        t = np.float32(s + bias[j])
+        y = np.float32((np.float32(t * (np.float32(1) / (np.float32(1) - np.float32(p)))) if keep[i, j] else np.float32(0))
+                       + orc.bf16_to_f32(resid[i:i + 1, j:j + 1])[0, 0])
+        assert whole_f[i, j] == y
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the LAMB of the DSL example (examples/lamb/lamb.cpp:20-28): what the programs emitted from it are checked against
+# ---------------------------------------------------------------------------------------------------------------------
+def test_dsl_lamb_all_ones_closed_form():
+    """g = 1 on P ranks, m = v = 0, w = 1, beta = 1/2, gamma = 1: m1 = P/2, v1 = P^2/2, m_ = P, v_ = P^2, r = 1 + 1 = 2,
+    rNorm = 2 sqrt(N), wNorm = sqrt(N), w1 = 1 - lr * (1/2) * 2 = 1 - lr; every step exact for N a power of four."""
+    for P in (1, 4, 8):
+        N = 4096
+        g = [np.ones(N, np.float32) for _ in range(P)]
+        w, m, v = np.ones(N, np.float32), np.zeros(N, np.float32), np.zeros(N, np.float32)
+        w1, norms = orc.dsl_lamb_f32(g, w, m, v, 0.25, 0.5, 0.5, 1.0)
+        assert np.all(m == P / 2) and np.all(v == P * P / 2)
+        assert norms[0] == 2 * 64 and norms[1] == 64
+        assert np.all(w1 == 0.75) and np.all(w == 1.0)
+    # gamma = 0 and a known r: w = 3, P = 2, g = 1: r = 1, wNorm/rNorm = 3, w1 = 3 - lr*3
+    g = [np.ones(16, np.float32) for _ in range(2)]
+    w1, norms = orc.dsl_lamb_f32(g, np.full(16, 3, np.float32), np.zeros(16, np.float32), np.zeros(16, np.float32), 0.5, 0.5, 0.5, 0.0)
+    assert norms[0] == 4 and norms[1] == 12 and np.all(w1 == 1.5)
+
+
+def test_dsl_lamb_against_a_float64_restatement():
+    """An independent numpy restatement in float64 from the text of examples/lamb/lamb.cpp:20-28: fp32 results within
+    a few ulp; a wrong operand order, a missing square root, a norm over r instead of w or the division the other way
+    round are all far outside."""
+    r = rng(71)
+    N, P = 5000, 4
+    g = [r.uniform(0, 1, N).astype(np.float32) for _ in range(P)]
+    w, m0, v0 = (r.uniform(0, 1, N).astype(np.float32) for _ in range(3))
+    lr, b1, b2, gamma = 0.01, 0.9, 0.99, 0.1
+    m, v = m0.copy(), v0.copy()
+    w1, norms = orc.dsl_lamb_f32(g, w, m, v, lr, b1, b2, gamma)
+    G = np.sum(np.stack(g).astype(np.float64), axis=0)
+    fb1, fb2 = np.float64(np.float32(b1)), np.float64(np.float32(b2))
+    M = fb1 * m0 + (1.0 - fb1) * G
+    V = fb2 * v0 + (1.0 - fb2) * G * G
+    R = (M / (1.0 - fb1)) / np.sqrt(V / (1.0 - fb2)) + np.float64(np.float32(gamma)) * w
+    rn, wn = np.sqrt(np.sum(R * R)), np.sqrt(np.sum(w.astype(np.float64) ** 2))
+    W1 = w - np.float64(np.float32(lr)) * (wn / rn) * R
+    assert np.max(np.abs(m - M) / np.abs(M)) < 4e-7 and np.max(np.abs(v - V) / np.abs(V)) < 4e-7
+    assert abs(norms[0] - rn) / rn < 2e-7 and abs(norms[1] - wn) / wn < 2e-7
+    assert np.max(np.abs(w1 - W1)) < 1e-6 * np.max(np.abs(W1))
+    # with bias corrections and an epsilon handed in (the build's own lamb program)
+    m, v = m0.copy(), v0.copy()
+    w2, _ = orc.dsl_lamb_f32(g, w, m, v, lr, b1, b2, gamma, c1=0.3, c2=0.7, eps=1e-3)
+    R2 = (M / np.float64(np.float32(0.3))) / (np.sqrt(V / np.float64(np.float32(0.7))) + np.float64(np.float32(1e-3))) + np.float64(np.float32(gamma)) * w
+    W2 = w - np.float64(np.float32(lr)) * (wn / np.sqrt(np.sum(R2 * R2))) * R2
+    assert np.max(np.abs(w2 - W2)) < 1e-6 * np.max(np.abs(W2))

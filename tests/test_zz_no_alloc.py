@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 import torch
 
+import oracle as orc
 from util import grads_f32, rel_err, weights_f32
 
 pytestmark = pytest.mark.gpu
@@ -17,7 +18,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 FP32_TOL = 1e-6
 HYPER = (1e-3, 0.9, 0.999, 1e-6, 0.01)
-LAMB_ENV = ("CCN_LAMB_RES_BLOCK", "CCN_LAMB_SPIN", "CCN_LAMB_RESIDENT", "CCN_LAMB_RES_WGS", "CCN_LAMB_ONESHOT")
+TWO_PASS = {1: 1}      # ccn_lamb_plan_tune(CCN_LAMB_KNOB_TWO_PASS, 1): every segment through the two-pass kernels
 
 
 def dev(a):
@@ -29,11 +30,11 @@ def host(t):
     return t.cpu().numpy()
 
 
-def run_plan(ccn, g, w0, seg_len, steps, mode):
+def run_plan(ccn, g, w0, seg_len, steps, mode, knobs=None):
     N = w0.size
     gd = [dev(x) for x in g]
     wd, md, vd = dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
-    plan = ccn.LambPlan(list(range(0, N + 1, seg_len)))
+    plan = ccn.LambPlan(list(range(0, N + 1, seg_len)), knobs=knobs or {})
     for t in range(1, steps + 1):
         plan.step(gd, wd, md, vd, *HYPER, t, mode)
     norms = plan.norms()
@@ -62,22 +63,18 @@ CASES = [
 
 @pytest.mark.parametrize("first,second", CASES)
 @pytest.mark.parametrize("mode", [0, 1])
-def test_static_scratch_lamb_matches_the_plan_entry_point(ccn, monkeypatch, first, second, mode):
+def test_static_scratch_lamb_matches_the_plan_entry_point(ccn, first, second, mode):
     for case_no, (P, nseg, seg_len) in enumerate((first, second)):
         N = nseg * seg_len
         g = grads_f32(90 + case_no, P, N, 1e-3)
         w0 = weights_f32(90 + case_no, N, 0.05)
         got = run_static(ccn, g, w0, seg_len, 2, mode)
         # the same kernels through a plan: bit for bit, the norms included
-        for name in LAMB_ENV:
-            monkeypatch.delenv(name, raising=False)
-        monkeypatch.setenv("CCN_LAMB_RESIDENT", "0")
-        want = run_plan(ccn, g, w0, seg_len, 2, mode)
+        want = run_plan(ccn, g, w0, seg_len, 2, mode, TWO_PASS)
         for name, a, b in zip("wmv", got[:3], want[:3]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (case_no, name, rel_err(a, b))
         assert np.array_equal(got[3], want[3]), (case_no, "norms")
         # the entry point as it is by default (segments that fit stay on chip: other summation order for the norms)
-        monkeypatch.delenv("CCN_LAMB_RESIDENT", raising=False)
         dflt = run_plan(ccn, g, w0, seg_len, 2, mode)
         assert np.array_equal(got[1].view(np.uint32), dflt[1].view(np.uint32)), (case_no, "m")
         assert np.array_equal(got[2].view(np.uint32), dflt[2].view(np.uint32)), (case_no, "v")
@@ -86,7 +83,63 @@ def test_static_scratch_lamb_matches_the_plan_entry_point(ccn, monkeypatch, firs
         assert rel_err(got[3], dflt[3]) < 1e-12, (case_no, "norms against the default plan")
 
 
-def test_static_scratch_lamb_without_a_norms_array_and_unaligned(ccn, monkeypatch):
+@pytest.mark.parametrize("mode", [0, 1])
+def test_static_scratch_lamb_against_the_oracle(ccn, mode):
+    """Directly against the CPU oracle (not only against the plan entry point): two calls in a row, the second on a smaller
+    input; m and v bit for bit, w to 1e-6, the norms to 1e-9 (float64 sums in another order)."""
+    for case_no, (P, nseg, seg_len) in enumerate(((5, 12, 1 << 14), (3, 2, 3072))):
+        N = nseg * seg_len
+        g = grads_f32(93 + case_no, P, N, 1e-3)
+        w0 = weights_f32(93 + case_no, N, 0.05)
+        got = run_static(ccn, g, w0, seg_len, 2, mode)
+        w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+        segs = list(range(0, N + 1, seg_len))
+        for t in (1, 2):
+            norms = orc.lamb_f32(g, w, m, v, segs, *HYPER, t, mode)
+        assert np.array_equal(got[1].view(np.uint32), m.view(np.uint32)), (case_no, "m")
+        assert np.array_equal(got[2].view(np.uint32), v.view(np.uint32)), (case_no, "v")
+        assert np.max(np.abs(got[0].astype(np.float64) - w)) <= FP32_TOL * float(np.max(np.abs(w))), (case_no, "w")
+        assert rel_err(got[3], np.asarray(norms).reshape(-1, 2)) < 1e-9, (case_no, "norms")
+
+
+def test_static_scratch_lamb_calls_on_two_streams_in_order(ccn):
+    """All calls on a GPU share the one static array, so calls on different streams must be ordered by the caller: a call
+    on stream A, an event, stream B waits for it, a call on stream B on other buffers, and back.  Each result equals the
+    same call made alone."""
+    shapes = [(4, 8, 8192), (2, 3, 2048)]
+    data = []
+    for k, (P, nseg, seg_len) in enumerate(shapes):
+        N = nseg * seg_len
+        g, w0 = grads_f32(98 + k, P, N, 1e-3), weights_f32(98 + k, N, 0.05)
+        data.append((g, w0, N, seg_len, run_static(ccn, g, w0, seg_len, 2, 0, with_norms=False)))
+    a, b = ccn.Stream(), ccn.Stream()
+    ev = [ccn.Event() for _ in range(4)]
+    state = []
+    for (g, w0, N, seg_len, _want) in data:
+        state.append(([dev(x) for x in g], dev(w0), torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)))
+    torch.cuda.synchronize()
+    k = 0
+    for t in (1, 2):
+        for which, stream, other in ((0, a, b), (1, b, a)):
+            gd, wd, md, vd = state[which]
+            _g, _w0, N, seg_len, _want = data[which]
+            ccn.lamb_f32_static(gd, wd, md, vd, N, seg_len, *HYPER, t, 0, None, stream.h)
+            ev[k].record(stream)
+            other.wait_event(ev[k])          # the next call, on the other stream, starts after this one has finished
+            k += 1
+    a.sync()
+    b.sync()
+    for which, (gd, wd, md, vd) in enumerate(state):
+        want = data[which][4]
+        for name, t_, w_ in zip("wmv", (wd, md, vd), want[:3]):
+            assert np.array_equal(host(t_).view(np.uint32), w_.view(np.uint32)), (which, name)
+    for e in ev:
+        e.close()
+    a.close()
+    b.close()
+
+
+def test_static_scratch_lamb_without_a_norms_array_and_unaligned(ccn):
     """norms = NULL keeps the norms in the static array; buffers 4 bytes off a 16-byte boundary take the scalar path."""
     P, nseg, seg_len = 3, 4, 2048
     N = nseg * seg_len
@@ -96,8 +149,7 @@ def test_static_scratch_lamb_without_a_norms_array_and_unaligned(ccn, monkeypatc
     wd = dev(np.concatenate([[np.float32(0)], w0]))[1:]
     md, vd = torch.zeros(N + 1, device=DEV)[1:], torch.zeros(N + 1, device=DEV)[1:]
     ccn.lamb_f32_static(gd, wd, md, vd, N, seg_len, *HYPER, 1, 0, None)
-    monkeypatch.setenv("CCN_LAMB_RESIDENT", "0")
-    want = run_plan(ccn, g, w0, seg_len, 1, 0)
+    want = run_plan(ccn, g, w0, seg_len, 1, 0, TWO_PASS)
     for name, a, b in zip("wmv", (host(wd), host(md), host(vd)), want[:3]):
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), name
 
