@@ -5,10 +5,13 @@
 // Wavefront w owns the 32 tile rows 8j + 2w, 8j + 2w + 1 (j = 0..15) over all 128 columns, as four
 // v_mfma_f32_32x32x16_bf16 blocks.  The MFMA computes C^T blocks (rows = n from W, columns = m from X)
 // so that every lane ends up with four CONSECUTIVE n of one row m in its accumulator quads.
-// W is [K x N] row-major (n contiguous) while the MFMA wants k contiguous per lane, so the W tile is
-// transposed in registers on its way into LDS.  LDS rows are 128 bytes (64 k) with the eight 16-byte
-// chunks XOR-swizzled by (row%8)^((row/8)%8): conflict-free for the 8-byte transposed writes and the
-// 16-byte fragment reads (also with the rows a wavefront owns: they differ in row/8).
+// X tile in LDS: rows of 128 bytes (64 k), the eight 16-byte chunks XOR-swizzled by (row%8)^((row/8)%8): conflict-free
+// for the 16-byte fragment reads with the rows a wavefront owns (they differ in row/8).
+// W is [K x N] row-major (n contiguous) while the MFMA wants k contiguous per lane.  The W tile goes into LDS as it
+// lies in memory (64 rows of 256 bytes, the sixteen 16-byte chunks of row k XOR-swizzled by 4*(k%4)) and comes back
+// transposed through gfx950's ds_read_b64_tr_b16: within 16 lanes, lane j receives element j%4 of the four 8-byte
+// pieces addressed by lanes j/4, j/4+4, j/4+8, j/4+12, so a 4(k) x 16(n) block arrives as 4 consecutive k per lane;
+// with the swizzle the 32 lanes of half a wavefront touch all 64 banks once.
 #include "ccn_common.hpp"
 
 #include <type_traits>
@@ -20,6 +23,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 128, BN = 128, BK = 64;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
 
 struct EpiPrm {
   float p_drop, keep_scale;
@@ -189,19 +195,10 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
       const int row = xr + 32 * j;
       *reinterpret_cast<u32x4*>(lds_x + row * 128 + ((xc ^ swz(row)) << 4)) = r.x[j];
     }
-    // transpose 4(k) x 8(n) -> 8 rows of 4 k, one byte permute per word
+    // W as it lies in memory: row k = wq*4 + j of 256 bytes, the 16-byte chunk wg at position wg ^ 4*(k%4)
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const uint32_t a0 = r.w[0][q], a1 = r.w[1][q], a2 = r.w[2][q], a3 = r.w[3][q];
-      u32x2 lo, hi;   // lo: column 2q, hi: column 2q+1; each k0..k3
-      lo[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100u);
-      lo[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100u);
-      hi[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302u);
-      hi[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
-      const int r0 = wg * 8 + 2 * q, r1 = r0 + 1;
-      *reinterpret_cast<u32x2*>(lds_w + r0 * 128 + (((wq >> 1) ^ swz(r0)) << 4) + ((wq & 1) << 3)) = lo;
-      *reinterpret_cast<u32x2*>(lds_w + r1 * 128 + (((wq >> 1) ^ swz(r1)) << 4) + ((wq & 1) << 3)) = hi;
-    }
+    for (int j = 0; j < 4; j++)
+      *reinterpret_cast<u32x4*>(lds_w + ((wq * 4 + j) * 16 + (wg ^ (4 * j))) * 16) = r.w[j];
   };
 
   f32x16 acc[4];   // [bn]: register 4*i4+e is C[rho][bn*32 + i4*8 + lh*4 + e]
@@ -213,9 +210,14 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
   // One K-step: four rounds of 16 k, each one X fragment against four W fragments: 16 MFMAs.  The W fragment of MFMA
   // i+2 (and the X fragment of the next round) is read from LDS before MFMA i is issued, so that an MFMA does not wait
   // for the read just before it; two fragments ahead is what the register budget of three workgroups per CU allows.
+  const int a16 = lane & 15, g2 = (lane >> 4) & 1;
+  const int waddr = ((lh * 8 + (a16 >> 2)) * 16 + ((2 * g2 + ((a16 >> 1) & 1)) ^ (4 * (a16 >> 2)))) * 16 + 8 * (a16 & 1);
   auto read_w = [&](int i) {
-    const int c = (i >> 2) * 2 + lh, row = (i & 3) * 32 + li;
-    return *reinterpret_cast<const bf16x8*>(lds_w + row * 128 + ((c ^ swz(row)) << 4));
+    // fragment i%4 (32 columns), round i/4: k = 16*(i/4) + 8*lh + 0..7 in two transposing reads of 4 k each
+    const uint8_t* p = lds_w + (waddr ^ ((i & 3) * 64)) + (i >> 2) * 4096;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 1024));
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
   auto read_x = [&](int ks) {
     const int c = ks * 2 + lh;
@@ -227,12 +229,14 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
     fb[0] = read_x(0);
 #pragma unroll
     for (int i = 0; i < kAhead; i++) fa[i] = read_w(i);
-    __builtin_amdgcn_sched_group_barrier(0x100, 1 + kAhead, 0);
+    constexpr int kWReads = 2;   // LDS instructions per W fragment
+    __builtin_amdgcn_sched_group_barrier(0x100, 1 + kAhead * kWReads, 0);
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       int reads = 0;
-      if (i + kAhead < 16) { fa[(i + kAhead) % (kAhead + 1)] = read_w(i + kAhead); reads++; }
+      if (i + kAhead < 16) { fa[(i + kAhead) % (kAhead + 1)] = read_w(i + kAhead); reads += kWReads; }
       if ((i & 3) == 4 - kAhead && (i >> 2) + 1 < 4) { fb[((i >> 2) + 1) & 1] = read_x((i >> 2) + 1); reads++; }
+      if (reads == 3) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
       if (reads == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       if (reads == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       const bf16x8 a = fa[i % (kAhead + 1)], b = fb[(i >> 2) & 1];

@@ -139,8 +139,10 @@ __host__ __device__ inline float dropout_ref(float x, float p_keep, uint64_t see
 }
 // One output element of the MLP epilogue from the sum s over the ranks' products, bias b and residual r, under dropout
 // form `mode` (CCN_DROPOUT_* of coconet_hip.h); host mirror of the library's epilogue for the emitted self-check.
-inline float epilogue_value(float s, float b, float r, float p, uint64_t seed, uint64_t idx, int mode) {
+// half: the operands are IEEE half; the saturating form then rounds to half after each add, as the library does.
+inline float epilogue_value(float s, float b, float r, float p, uint64_t seed, uint64_t idx, int mode, bool half = false) {
   auto sat = [](float x) { return x > 0.0f ? (x < 1.0f ? x : 1.0f) : 0.0f; };
+  auto h16 = [](float x) { return f16_bits_to_f32(f32_to_f16_bits(x)); };
   if (mode == CCN_DROPOUT_INVERTED) {
     const float t = s + b;
     const float d = p > 0.0f ? dropout(t, p, seed, idx) : t;
@@ -152,6 +154,7 @@ inline float epilogue_value(float s, float b, float r, float p, uint64_t seed, u
     return (kept ? t : 0.0f) + r;
   }
   const float d = kept ? s : 0.0f;
+  if (mode == CCN_DROPOUT_REF_NCCL_SAT && half) return sat(h16(sat(h16(d) + h16(b))) + r);
   return mode == CCN_DROPOUT_REF_NCCL_SAT ? sat(sat(d + b) + r) : (d + b) + r;
 }
 

@@ -321,7 +321,7 @@ std::string generateMLP(const Pipeline& p, const std::vector<CodeGenVarBounds>& 
   o << ind << "        float s = (float)acc;\n";
   o << ind << "        for (int q = 0; q < nPartials; q++) { s = s + hP[q][m * N + n]; mag += fabs((double)hP[q][m * N + n]); }\n";
   o << ind << "        const float r = " << (c.resid ? cv_from + "(hR[m * N + n])" : std::string("0.0f")) << ";\n";
-  o << ind << "        const float y = ccn_gen::epilogue_value(s, hB[n], r, p_drop, seed__, m * N + n, mode__);\n";
+  o << ind << "        const float y = ccn_gen::epilogue_value(s, hB[n], r, p_drop, seed__, m * N + n, mode__, " << (half ? "true" : "false") << ");\n";
   o << ind << "        mag = (mag + fabs((double)hB[n])) * (mode__ == CCN_DROPOUT_INVERTED ? 1.0 / (1.0 - (double)p_drop) : 1.0) + fabs((double)r);\n";
   o << ind << "        const int want = " << cv_to << "(y), have = got[m * N + n];\n";
   o << ind << "        seen++;\n";

@@ -43,6 +43,21 @@ def bf16_ulp_distance(a, b):
     return np.abs(key(a) - key(b))
 
 
+def assert_within_fp32_sum_error(got_bits, want_bits, want_f32, mag, terms):
+    """The fused kernel's bar on many outputs: the same bfloat16 or its neighbour, except where the sum cancels (a small
+    result of large terms), where the error must stay within what an fp32 sum of `terms` terms of total magnitude `mag`
+    may be off by, plus the rounding to bfloat16."""
+    d = bf16_ulp_distance(got_bits, want_bits)
+    assert (d > 0).mean() < 0.02, f"{(d > 0).mean():.4f} of the outputs differ"
+    far = d > 1
+    assert far.mean() < 1e-4, f"{far.mean():.6f} of the outputs differ by more than one ulp"
+    if far.any():
+        err = np.abs(orc.bf16_to_f32(got_bits[far]).astype(np.float64) - want_f32[far])
+        ulp = np.abs(want_f32[far]).astype(np.float64) * 2.0 ** -8 + 1e-38
+        assert np.all(err <= terms * 2.0 ** -24 * mag[far] + ulp), float(np.max(err / (terms * 2.0 ** -24 * mag[far] + ulp)))
+    return d
+
+
 @pytest.mark.parametrize("M,N,K,nP,p", [(128, 128, 64, 7, 0.1), (256, 384, 192, 7, 0.1), (128, 256, 1024, 3, 0.5),
                                          (384, 128, 128, 0, 0.0), (128, 128, 64, 1, 0.0)])
 def test_outproj_against_oracle(ccn, M, N, K, nP, p):
@@ -328,11 +343,12 @@ def test_outproj_config5_full_size(ccn):
     Xh, rh, got = bits(X), bits(resid), bits(out)
     Wh = W.view(torch.int16).cpu().numpy().view(np.uint16)
     ph = [q[ridx].cpu().numpy() for q in parts]
-    want, _ = orc.mlp_outproj(Xh, Wh, ph, bias.cpu().numpy(), rh, len(rows), N, K, 0.1, 0, row_ids=rows)
+    want, want_f32 = orc.mlp_outproj(Xh, Wh, ph, bias.cpu().numpy(), rh, len(rows), N, K, 0.1, 0, row_ids=rows)
     keep_rows = np.stack([orc.dropout_mask(0, int(r) * N, N, 0.1) for r in rows]).astype(bool)
     assert np.array_equal(got[~keep_rows], rh[~keep_rows])                 # mask exact on the sampled rows
-    d = bf16_ulp_distance(got, want)
-    assert d.max() <= 1 and (d > 0).mean() < 0.02
+    mag = (torch.abs(X[ridx].float()) @ torch.abs(W.float())).cpu().numpy().astype(np.float64)
+    mag = (mag + sum(np.abs(q).astype(np.float64) for q in ph) + np.abs(bias.cpu().numpy())) / 0.9 + np.abs(orc.bf16_to_f32(rh))
+    d = assert_within_fp32_sum_error(got, want, want_f32, mag, K + 11)
     per_row = (d > 0).reshape(3, 128, N).mean(axis=(0, 2))                 # no row position inside a tile stands out
     assert per_row.max() < 0.03, f"in-tile row {int(per_row.argmax())}: {per_row.max():.4f} of its outputs differ"
     dropped = float((out == resid).float().mean())
@@ -380,11 +396,12 @@ def test_rows_longer_than_a_buffer_descriptor_spans(ccn):
     rows = np.array([0, 1, 63, 126, 127])
     ridx = torch.from_numpy(rows).to(DEV)
     bits = lambda t: t.view(torch.int16).cpu().numpy().view(np.uint16)
-    want, _ = orc.mlp_outproj(bits(X[ridx]), bits(W), [part[ridx].cpu().numpy()], bias.cpu().numpy(), bits(resid[ridx]),
-                              len(rows), N, K, 0.1, 3, row_ids=rows)
+    want, want_f32 = orc.mlp_outproj(bits(X[ridx]), bits(W), [part[ridx].cpu().numpy()], bias.cpu().numpy(), bits(resid[ridx]),
+                                     len(rows), N, K, 0.1, 3, row_ids=rows)
     got = bits(out[ridx])
-    d = bf16_ulp_distance(got, want)
-    assert d.max() <= 1 and (d > 0).mean() < 0.02
+    mag = (torch.abs(X[ridx].float()) @ torch.abs(W.float())).cpu().numpy().astype(np.float64)
+    mag = (mag + np.abs(part[ridx].cpu().numpy()) + np.abs(bias.cpu().numpy())) / 0.9 + np.abs(orc.bf16_to_f32(bits(resid[ridx])))
+    assert_within_fp32_sum_error(got, want, want_f32, mag, K + 5)
     keep_rows = np.stack([orc.dropout_mask(3, int(r) * N, N, 0.1) for r in rows]).astype(bool)
     assert np.array_equal(got[~keep_rows], bits(resid[ridx])[~keep_rows])
     dropped = float((out == resid).float().mean())
