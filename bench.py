@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adam_f32",
                     choices=["adam_f32", "adam_f32_scattered", "sgd_f32", "adam_f16g", "adam_bf16g", "lamb_f32",
-                             "lamb_nccl_f16g", "mlp_outproj", "copy"])
+                             "lamb_nccl_f16g", "mlp_outproj", "matmul_bf16", "copy"])
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -67,55 +67,70 @@ class Buffers:
         return a
 
 
+def source_sha256(rel):
+    import hashlib
+    with open(os.path.join(ROOT, rel), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
 def traffic_from_profiles(name):
-    """HBM bytes per launch measured with rocprofv3 --pmc, if a summary for this workload was committed."""
+    """HBM bytes per launch measured with rocprofv3 --pmc, from the committed summary of this workload -- or None when
+    there is none, or when the kernel's source file has changed since the summary was taken (every summary records the
+    SHA-256 of the source file its kernel is compiled from: a stale figure is not passed on)."""
     path = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(path):
         return None
-    vals = {}
+    vals, fresh = {}, False
     for line in open(path):
+        if line.startswith("SOURCE_SHA256="):
+            digest, rel = line.split("=", 1)[1].split()[:2]
+            try:
+                fresh = source_sha256(rel) == digest
+            except OSError:
+                fresh = False
         if "=" in line and line.split("=")[0].strip() in ("FETCH_BYTES_PER_LAUNCH", "WRITE_BYTES_PER_LAUNCH"):
             k, v = line.split("=", 1)
             try:
                 vals[k.strip()] = float(v.split()[0])
             except ValueError:
                 pass
-    if len(vals) == 2:
+    if len(vals) == 2 and fresh:
         return vals["FETCH_BYTES_PER_LAUNCH"] + vals["WRITE_BYTES_PER_LAUNCH"]
     return None
 
 
 def cpu_baseline(wl, P, budget_s=8.0):
     """The oracle's restatement of the reference loops (for Adam: multi-process-adam-scattered.cpp:112-136 with a
-    fixed-order P-way sum) on a bounded sample of the same workload: once on one thread, as the reference runs it, and
-    once with the work cut into one slice per host thread (index ranges, whole segments for LAMB, rows for the MLP:
-    the loops are independent across those, so the results are the same)."""
+    fixed-order P-way sum), C compiled -O2 -ffp-contract=off -fopenmp, on a bounded sample of the same workload: once on
+    one thread, as the reference runs its checker, and once as an OpenMP parallel-for over the elements (whole segments
+    for LAMB, rows for the MLP) on the host threads this box gives a job.  Same arithmetic and results either way."""
     import oracle as orc
-    from concurrent.futures import ThreadPoolExecutor
     threads = max(1, min(16, os.cpu_count() or 1))     # a one-GPU box gives a job 16 host threads
     r = np.random.Generator(np.random.Philox(key=[5, 0]))
     f32 = np.float32
-    if wl == "mlp_outproj":
+    if wl in ("mlp_outproj", "matmul_bf16"):
         # a band of rows of the 8192 x 1024 x 8192 product with its 7 partial buffers
-        rows, Nn, Kd, nP = 8 * threads, 8192, 1024, 7
+        rows, Nn, Kd, nP = 8 * threads, 8192, 1024, (7 if wl == "mlp_outproj" else 0)
         X = orc.f32_to_bf16(r.standard_normal((rows, Kd), dtype=f32))
         Wm = orc.f32_to_bf16(r.standard_normal((Kd, Nn), dtype=f32) * f32(0.02))
         parts = [r.standard_normal((rows, Nn), dtype=f32) for _ in range(nP)]
         bias = r.standard_normal(Nn, dtype=f32)
         resid = orc.f32_to_bf16(r.standard_normal((rows, Nn), dtype=f32))
-        units, per_unit = rows * Nn, (7 * 4 + 2 + 2) + (Kd * 2 * 2.0) / 8192   # bytes per output, X and W amortised
-        what = f"oracle orc_mlp_outproj on {rows} of the 8192 rows (K=1024, 7 partials, p=0.1)"
+        units, per_unit = rows * Nn, (nP * 4 + 2 + 2) + (Kd * 2 * 2.0) / 8192   # bytes per output, X and W amortised
+        what = f"oracle orc_mlp_outproj (a float64 brute-force product, a checker and not a tuned CPU GEMM) on {rows} of the 8192 rows (K=1024, {nP} partials)"
 
-        def piece(lo, hi, t):
-            orc.mlp_outproj(X[lo:hi], Wm, [q[lo:hi] for q in parts], bias, resid[lo:hi], hi - lo, Nn, Kd, 0.1, 0)
-        cuts = [rows * k // threads for k in range(threads + 1)]
+        def piece(t):
+            orc.mlp_outproj(X, Wm, parts, bias, resid, rows, Nn, Kd, 0.1 if nP else 0.0, 0)
     else:
-        n = 1 << 24
+        # the headline workload on a quarter of its elements (2^26: 3 GB of host memory), the others on 2^24
+        n = 1 << (26 if wl in ("adam_f32", "adam_f32_scattered") else 24)
         nseg = 16
         segs = [k * (n // nseg) for k in range(nseg + 1)]
         half = wl in ("adam_f16g", "adam_bf16g", "lamb_nccl_f16g")
         scale = f32(2.0 ** 7 if wl == "adam_bf16g" else 2.0 ** 16 if wl == "adam_f16g" else 1.0)
-        g = [(r.standard_normal(n, dtype=f32) * f32(1e-3)) for _ in range(P)]
+        base = r.standard_normal(n, dtype=f32) * f32(1e-3)
+        g = [np.roll(base, 1000003 * p) for p in range(P)]      # one draw, shifted per rank: distinct arrays, same statistics
+        del base
         if half:
             g = [(orc.f32_to_bf16 if wl == "adam_bf16g" else orc.f32_to_f16)(x * scale) for x in g]
         w = r.uniform(-0.05, 0.05, n).astype(f32)
@@ -125,57 +140,45 @@ def cpu_baseline(wl, P, budget_s=8.0):
         units = n
         per_unit = {"sgd_f32": (P + 1) * 4 + 4, "adam_f32": (P + 3) * 4 + 12, "adam_f32_scattered": (P + 3) * 4 + 12,
                     "lamb_f32": (P + 3) * 4 + 12}.get(wl, P * 2 + 12 + 12 + 2)
-        what = f"oracle loop of {wl}, P={P}, N=2^24 sample of the 2^28 workload" + (" in 16 segments" if "lamb" in wl else "")
+        what = (f"oracle loop of {wl}, P={P}, N=2^{int(np.log2(n))} sample of the 2^28 workload"
+                + (" in 16 segments" if "lamb" in wl else ""))
 
-        def piece(lo, hi, t):
-            gs = [x[lo:hi] for x in g]
+        def piece(t):
             if wl == "sgd_f32":
-                orc.sgd_f32(gs, w[lo:hi], 0.01)
+                orc.sgd_f32(g, w, 0.01)
             elif wl in ("adam_f32", "adam_f32_scattered"):
-                orc.adam_f32(gs, w[lo:hi], m[lo:hi], v[lo:hi], 1e-3, 0.9, 0.999, 1e-6, t)
+                orc.adam_f32(g, w, m, v, 1e-3, 0.9, 0.999, 1e-6, t)
             elif wl == "adam_f16g":
-                orc.adam_f16g(gs, w[lo:hi], m[lo:hi], v[lo:hi], w16[lo:hi], 1e-3, 0.9, 0.999, 1e-6, t, f32(1.0) / scale)
+                orc.adam_f16g(g, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, t, f32(1.0) / scale)
             elif wl == "adam_bf16g":
-                orc.adam_bf16g(gs, w[lo:hi], m[lo:hi], v[lo:hi], w16[lo:hi], 1e-3, 0.9, 0.999, 1e-6, t, f32(1.0) / scale)
+                orc.adam_bf16g(g, w, m, v, w16, 1e-3, 0.9, 0.999, 1e-6, t, f32(1.0) / scale)
+            elif wl == "lamb_f32":
+                orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
             else:
-                local = [x - lo for x in segs if lo <= x <= hi]
-                if wl == "lamb_f32":
-                    orc.lamb_f32(gs, w[lo:hi], m[lo:hi], v[lo:hi], local, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
-                else:
-                    orc.lamb_nccl_f16g(gs, w[lo:hi], w16[lo:hi], m[lo:hi], v[lo:hi], local, 1e-3, 0.9, 0.999, 1.0)
-        if "lamb" in wl:      # whole segments per thread
-            cuts = [segs[nseg * k // threads] for k in range(threads + 1)]
-        else:
-            cuts = [n * k // threads for k in range(threads + 1)]
-    top = cuts[-1]
-    piece(0, top, 1)          # warm the pages
+                orc.lamb_nccl_f16g(g, w, w16, m, v, segs, 1e-3, 0.9, 0.999, 1.0)
+    orc.set_num_threads(threads)
+    piece(1)          # warm the pages
 
-    def timed(step_fn):
+    def timed(nthreads):
+        orc.set_num_threads(nthreads)
         t0 = time.perf_counter()
         reps = 0
         while True:
-            step_fn(reps + 2)
+            piece(reps + 2)
             reps += 1
             el = time.perf_counter() - t0
             if el > budget_s or reps >= 400:
                 return el / (reps * units), reps
 
-    one, reps1 = timed(lambda t: piece(0, top, t))
-    pool = ThreadPoolExecutor(threads)
-
-    def sliced(t):
-        jobs = [pool.submit(piece, a, b, t) for a, b in zip(cuts[:-1], cuts[1:]) if b > a]
-        for j in jobs:
-            j.result()
-
-    many, repsT = timed(sliced)
-    pool.shutdown()
+    many, repsT = timed(threads)
+    one, reps1 = timed(1)
+    orc.set_num_threads(1)
     return {
         "value": round(per_unit / many / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
         "params_per_s": round(1.0 / many, 1),
         "single_thread": {"value": round(per_unit / one / 1e9, 3), "unit": "GB/s", "params_per_s": round(1.0 / one, 1)},
-        "sample": f"{what}; {repsT} steps on {threads} threads (one slice each), {reps1} steps on 1 thread "
-                  f"({os.cpu_count()} host cpus visible)",
+        "sample": f"{what}; C loop (-O2 -ffp-contract=off -fopenmp): {repsT} steps as an OpenMP parallel-for on {threads} threads, "
+                  f"{reps1} steps on 1 thread as the reference runs it ({os.cpu_count()} host cpus visible)",
     }
 
 
@@ -285,6 +288,19 @@ def build_workload(a, wl, capi, torch, stream, allocator):
         kernel = "mlp_outproj_kernel<7>"
         config = {"workload": "mlp_outproj bf16 8192x1024x8192 + 7 fp32 partials + bias + dropout(0.1) + residual",
                   "M": M, "N": Nn, "K": Kd}
+    elif wl == "matmul_bf16":
+        # the MatMul step of the unfused schedules alone (the reference: cublasGemmEx, src/codegen.cpp:1058-1136)
+        M = Nn = 8192
+        Kd = 1024
+        X = torch.randn(M, Kd, device="cuda", generator=gen).to(torch.bfloat16)
+        Wm = (torch.randn(Kd, Nn, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+        Cm = torch.empty(M, Nn, device="cuda")
+        step = lambda t: capi.matmul_bf16_f32(X, Wm, Cm, M, Nn, Kd, stream)
+        alg_bytes = float(M * Kd * 2 + Kd * Nn * 2 + M * Nn * 4)
+        flops = 2.0 * M * Nn * Kd
+        units = M * Nn
+        kernel = "mlp_outproj_kernel<0, true>"
+        config = {"workload": "matmul bf16 8192x1024x8192 -> fp32 (the unfused schedule's MatMul step)", "M": M, "N": Nn, "K": Kd}
     else:   # plain device copy, the practical HBM ceiling of this box
         N = 1 << (a.log2n or 30)
         src = torch.empty(N, dtype=torch.float32, device="cuda").normal_(generator=gen)
@@ -349,19 +365,39 @@ def other_workloads(a, capi, torch, stream):
                      "algorithmic_bytes_per_launch": c["roofline"]["algorithmic_bytes_per_launch"], "traffic": None})
     except (ValueError, KeyError, IndexError):
         rows.append({"workload": "adam_f32 on plain allocations", "error": (child.stderr or child.stdout)[-300:]})
-    for wl, allocator in (("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_large", "ccn"), ("adam_f16g", "ccn"),
-                          ("lamb_f32", "ccn"), ("mlp_outproj", "ccn")):
-        step, alg_bytes, units, kernel, config, flops, P, keep = build_workload(a, wl, capi, torch, stream, allocator)
+    for wl, allocator in (("copy", "torch"), ("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_graph", "ccn"),
+                          ("sgd_f32_large", "ccn"), ("adam_f16g", "ccn"), ("lamb_f32", "ccn"), ("mlp_outproj", "ccn"),
+                          ("matmul_bf16", "ccn")):
+        replay = 64 if wl == "sgd_f32_graph" else 0      # configuration 1 again, 64 recorded steps per graph launch
+        own = capi.Stream() if replay else None          # the null stream cannot be recorded
+        st = own.h if own else stream
+        step, alg_bytes, units, kernel, config, flops, P, keep = build_workload(a, "sgd_f32" if replay else wl, capi, torch, st,
+                                                                                allocator)
         steps, warm = (200, 20) if alg_bytes < 1e9 else (30, 10)
-        wall_ms, ev_ms = timed_steps(step, steps, warm, capi, torch, stream)
+        if replay:
+            step(1)
+            torch.cuda.synchronize()
+            with capi.Graph(own) as graph:
+                for t in range(replay):
+                    step(2 + t)
+            wall_ms, ev_ms = timed_steps(lambda t: graph.launch(), steps, warm, capi, torch, st)
+            wall_ms, ev_ms, steps = wall_ms / replay, ev_ms / replay, steps * replay
+            config["workload"] += f", {replay} recorded steps per ccn_graph_launch"
+        else:
+            wall_ms, ev_ms = timed_steps(step, steps, warm, capi, torch, st)
         ach = alg_bytes / (ev_ms * 1e-3) / 1e9
         row = {"workload": config["workload"], "allocator": allocator, "steps": steps, "warmup": warm,
                "ms_per_step": round(wall_ms, 5), "avg_launch_ms": round(ev_ms, 5), "algorithmic_GBps": round(ach, 2),
                "frac_of_hbm_peak": round(ach / HBM_PEAK_GBPS, 4), "kernel": kernel,
                "algorithmic_bytes_per_launch": alg_bytes,
                "traffic": traffic_from_profiles(f"{'sgd_f32' if wl == 'sgd_f32_large' else wl}.pmc.txt") if allocator == "ccn" else None}
-        if alg_bytes < 1e9:
+        if alg_bytes < 1e9 and wl != "matmul_bf16":
             row["note"] = "fits the caches and is bound by launches: not a roofline figure"
+        if wl == "copy":
+            row["note"] = "the measured ceiling of a 1R:1W stream on this box, to read the fractions of the 8 TB/s nominal peak against"
+        if replay:
+            graph.close()
+            own.close()
         if flops:
             row["mfma_TFLOPs"] = round(flops / (ev_ms * 1e-3) / 1e12, 2)
             row["frac_of_mfma_peak"] = round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
@@ -424,7 +460,7 @@ def main():
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"adam_f16g": "f16 gradients, f32 state", "adam_bf16g": "bf16 gradients, f32 state",
                   "lamb_nccl_f16g": "f16 gradients (f16 sum), f32 state",
-                  "mlp_outproj": "bf16 x bf16 -> f32"}.get(wl, "f32"),
+                  "mlp_outproj": "bf16 x bf16 -> f32", "matmul_bf16": "bf16 x bf16 -> f32"}.get(wl, "f32"),
         "data": "synthetic", "config": config,
         "params_per_s": round(units / (wall_ms * 1e-3), 1),
         "device": info,
@@ -437,13 +473,16 @@ def main():
     if flops:
         line["mfma"] = {"achieved": round(flops / (ev_ms * 1e-3) / 1e12, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                         "unit": "TFLOP/s", "frac": round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    if wl == "matmul_bf16":     # the one compute-bound kernel of the path: its roofline is the matrix cores'
+        line["roofline"].update({"bound": "mfma", "achieved": line["mfma"]["achieved"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                                 "unit": "TFLOP/s", "frac": line["mfma"]["frac"], "algorithmic_flops_per_launch": flops})
     default_run = (wl == "adam_f32" and a.allocator == "ccn" and a.graph_steps == 0 and a.log2n is None and a.ranks is None)
     if default_run and not a.no_others:
         del step
         release(keep, capi, torch)
         line["other_workloads"] = other_workloads(a, capi, torch, stream)
     if wl != "copy" and not a.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(wl, P if wl != "mlp_outproj" else 8)
+        line["cpu_baseline"] = cpu_baseline(wl, P if wl not in ("mlp_outproj", "matmul_bf16") else 8)
     print(json.dumps(line), flush=True)
 
 

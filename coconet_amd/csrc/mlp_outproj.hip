@@ -327,6 +327,192 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
   }
 }
 
+// ---- the plain product on large tiles ------------------------------------------------------------------------------------
+// C[M x N] (fp32) = X . W alone is bound by the matrix cores, and a 128 x 128 tile moves too many operand bytes per MFMA
+// to keep them busy.  For whole multiples of 256 rows and columns: a 512-thread workgroup owns a 256(m) x 256(n) tile,
+// its 8 wavefronts as 2(m) x 4(n), each 128 x 64 as eight 32 x 32 blocks (128 accumulator registers); per 16-k round a
+// wavefront reads four X and two W fragments from LDS for eight MFMAs.  Two LDS stages of 64 KiB (X: rows of 128 bytes,
+// chunks swizzled by (row/2)%8; W as it lies in memory, rows of 512 bytes, chunks swizzled by 4*(k%4), read back through
+// ds_read_b64_tr_b16), operands staged through registers one K-step ahead, one barrier per K-step, one workgroup per CU.
+// Workgroups are numbered so that the 32 an XCD runs at a time form a block of 4 x 8 tiles: their X and W panels are
+// shared inside that XCD's L2.  The accumulators leave through wavefront-private pieces of LDS as whole 256-byte rows.
+constexpr int TM = 256, TN = 256;
+constexpr int kBigBlock = 512;
+constexpr int kBigStage = (TM + TN) * BK * 2;     // one K-step of X and W: 64 KiB
+constexpr int kBigLds = 2 * kBigStage;
+
+template <bool F16>
+__global__ __launch_bounds__(kBigBlock) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ C, const int N,
+                           const int K, const int tilesM, const int tilesN) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_big[];
+  // tile of this workgroup: blocks of 4 x 8 tiles dealt to the XCDs (workgroup b runs on XCD b % 8) when the grid divides
+  int tm, tn;
+  {
+    const int b = blockIdx.x;
+    if (tilesM % 4 == 0 && tilesN % 8 == 0 && ((tilesM / 4) * (tilesN / 8)) % 8 == 0) {
+      const int xcd = b & 7, s_ = b >> 3, blk = (s_ >> 5) * 8 + xcd, j = s_ & 31;
+      const int bcols = tilesN / 8;
+      tm = (blk / bcols) * 4 + (j >> 3);
+      tn = (blk % bcols) * 8 + (j & 7);
+    } else {
+      tm = b / tilesN;
+      tn = b % tilesN;
+    }
+  }
+  const size_t m0 = (size_t)tm * TM, n0 = (size_t)tn * TN;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);   // a scalar: it goes into descriptors
+  const int wm = wave >> 2, wn = wave & 3;
+  const int li = lane & 31, lh = lane >> 5;
+
+  // staging: X rows (t/8) + 64*j, chunk t%8; W rows (t/32) + 16*j, chunk t%32 (memory chunk c lives at position c ^ 4*(k%4))
+  const int xr_ = t >> 3, xc = t & 7, wk = t >> 5, wc = t & 31;
+  const uint32_t xoff = (uint32_t)((xr_ * K + xc * 8) * 2), xrow64 = (uint32_t)(64 * K * 2);
+  const uint32_t woff = (uint32_t)((wk * N + 8 * (wc ^ (4 * (wk & 3)))) * 2), wrow16 = (uint32_t)(16 * N * 2);
+  const rsrc_t x_rs = buffer_at(X + m0 * (size_t)K);
+  const uint16_t* const wbase = W + n0;
+  // two sets of staging registers: the operands of step s wait in set s%2, requested two K-steps before their use
+  u32x4 sx[2][4], sw[2][4];
+  auto load_stage = [&](auto set, int k0) {
+    constexpr int S = decltype(set)::value;
+    const rsrc_t w_rs = buffer_at(wbase + (size_t)k0 * N);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      sx[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rs, xoff, (uint32_t)j * xrow64 + (uint32_t)k0 * 2u, 0));
+      sw[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w_rs, woff, (uint32_t)j * wrow16, 0));
+    }
+  };
+  auto store_quarter = [&](auto set, int buf, int j) {
+    constexpr int S = decltype(set)::value;
+    uint8_t* const lx = lds_big + buf * kBigStage;
+    uint8_t* const lw = lx + TM * BK * 2;
+    const int row = xr_ + 64 * j;
+    *reinterpret_cast<u32x4*>(lx + row * 128 + ((xc ^ ((row >> 1) & 7)) << 4)) = sx[S][j];
+    *reinterpret_cast<u32x4*>(lw + ((wk + 16 * j) * 32 + wc) * 16) = sw[S][j];
+  };
+  auto store_stage = [&](auto set, int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) store_quarter(set, buf, j);
+  };
+  // fragment addresses: X rows 128*wm + 32*bm + li, chunk 2*ks + lh; W fragment bn of this wavefront's 64 columns
+  int xaddr[4];
+#pragma unroll
+  for (int bm = 0; bm < 4; bm++) {
+    const int row = 128 * wm + 32 * bm + li;
+    xaddr[bm] = row * 128;   // + ((2*ks + lh) ^ swizzle) * 16
+  }
+  const int xsw = (li >> 1) & 7;   // (row/2) % 8: the rows of a fragment start at a multiple of 32
+  const int a16 = lane & 15, g2 = (lane >> 4) & 1;
+  const int waddr = ((lh * 8 + (a16 >> 2)) * 32 + ((8 * wn + 2 * g2 + ((a16 >> 1) & 1)) ^ (4 * (a16 >> 2)))) * 16 + 8 * (a16 & 1);
+  auto read_x = [&](int buf, int bm, int ks) {
+    return *reinterpret_cast<const s16x8*>(lds_big + buf * kBigStage + xaddr[bm] + (((2 * ks + lh) ^ xsw) << 4));
+  };
+  auto read_w = [&](int buf, int bn, int ks) {
+    const uint8_t* p = lds_big + buf * kBigStage + TM * BK * 2 + (waddr ^ (bn * 64)) + ks * (16 * 512);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * 512));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+
+  f32x16 acc[2][4];   // [bn][bm]: register 4*i4+e is C[128*wm + 32*bm + li][64*wn + 32*bn + 8*i4 + 4*lh + e]
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
+
+  // One K-step from LDS stage `buf` as 16 phases (round ks, row block bm) of two MFMAs each.  A phase reads the X fragment
+  // of the next phase, and the last two phases of a round the two W fragments of the next round, so that the fragments
+  // in flight stay at 6 registers sets; `write_next(i)` is called in phase i of the last round (i = 0..3) to move a
+  // quarter of the next step's operands from their staging registers into the other stage.
+  auto mfma_step = [&](int buf, auto&& write_next) {
+    s16x8 fw[2][2], fx[2];
+    fw[0][0] = read_w(buf, 0, 0);
+    fw[0][1] = read_w(buf, 1, 0);
+    fx[0] = read_x(buf, 0, 0);
+#pragma unroll
+    for (int ph = 0; ph < 16; ph++) {
+      const int ks = ph >> 2, bm = ph & 3;
+      int reads = 0;
+      if (ph + 1 < 16) { fx[(ph + 1) & 1] = read_x(buf, (ph + 1) & 3, (ph + 1) >> 2); reads += 1; }
+      if (ks + 1 < 4 && bm >= 2) { fw[(ks + 1) & 1][bm - 2] = read_w(buf, bm - 2, ks + 1); reads += 2; }
+      if (ks == 3) write_next(bm);
+#pragma unroll
+      for (int bn = 0; bn < 2; bn++) {
+        if constexpr (F16)
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fw[ks & 1][bn]), __builtin_bit_cast(f16x8, fx[ph & 1]), acc[bn][bm], 0, 0, 0);
+        else
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fw[ks & 1][bn]), __builtin_bit_cast(bf16x8, fx[ph & 1]), acc[bn][bm], 0, 0, 0);
+      }
+      // issue order of the phase: its LDS reads (and writes), then its two MFMAs
+      if (reads == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (reads == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      if (reads == 3) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+      if (ks == 3) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto lds_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): this wavefront's LDS writes are done; global loads stay in flight
+    __builtin_amdgcn_s_barrier();
+  };
+
+  // main loop, two steps per turn so that the staging sets are compile-time names: step kt multiplies from LDS stage
+  // kt%2, requests the operands of step kt+2 (past the end: the last step's again, unused) and, under its last round,
+  // moves those of step kt+1 from their registers into the other stage
+  const int nk = K / BK;
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  auto clamp_k = [&](int kt) { return (kt < nk ? kt : nk - 1) * BK; };
+  load_stage(Set0{}, 0);
+  load_stage(Set1{}, clamp_k(1));
+  store_stage(Set0{}, 0);
+  lds_barrier();
+  auto step = [&](auto set, int kt) {   // set = kt % 2
+    constexpr int S = decltype(set)::value;
+    load_stage(set, clamp_k(kt + 2));
+    __builtin_amdgcn_sched_barrier(0);   // the requests go out first, two K-steps ahead of their use
+    mfma_step(S, [&](int j) { store_quarter(std::integral_constant<int, 1 - S>{}, 1 - S, j); });
+    lds_barrier();
+  };
+  // (the last step's requests and LDS writes are redundant and harmless: nothing reads that stage any more)
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    step(Set0{}, kt);
+    step(Set1{}, kt + 1);
+  }
+  if (kt < nk) step(Set0{}, kt);   // an odd number of steps
+  // every wavefront is past the last step's barrier and done with the operand stages: LDS becomes eight private C pieces
+  constexpr int kCS = 64 + 4;   // floats per row of a piece: 32 rows x 64 columns at a time
+  float* const cw = reinterpret_cast<float*>(lds_big) + wave * (32 * kCS);
+  const int r4 = lane >> 4, c16 = lane & 15;
+  const rsrc_t c_rs = buffer_at(C + (m0 + 128 * wm) * (size_t)N + n0 + 64 * wn);
+#pragma unroll
+  for (int bm = 0; bm < 4; bm++) {
+#pragma unroll
+    for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        f32x4 v;
+        v[0] = acc[bn][bm][i4 * 4 + 0];
+        v[1] = acc[bn][bm][i4 * 4 + 1];
+        v[2] = acc[bn][bm][i4 * 4 + 2];
+        v[3] = acc[bn][bm][i4 * 4 + 3];
+        *reinterpret_cast<f32x4*>(cw + li * kCS + bn * 32 + i4 * 8 + lh * 4) = v;
+      }
+    __builtin_amdgcn_wave_barrier();   // a wavefront's LDS operations complete in order
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(cw + (4 * jj + r4) * kCS + 4 * c16);
+      const uint32_t off = (uint32_t)(((32 * bm + 4 * jj + r4) * N + 4 * c16) * 4);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), c_rs, off, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
 // Standalone epilogue over an fp32 product in memory: one quad per thread, no loop, the launch shape of the other
 // streaming kernels (the y dimension of the grid only comes into play beyond 2^30 workgroups).
 template <int NP, int BS, bool REF, bool F16 = false>
@@ -564,6 +750,16 @@ int matmul_launch(const uint16_t* X, const uint16_t* W, float* C, int M, int N, 
     if (tiles > 0x7fffffffull) return CCN_ERANGE;
     hipLaunchKernelGGL((outproj_any_shape_kernel<true, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, as_stream(stream), X, W,
                        tbl, 0, (const float*)nullptr, (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), M, N, K, ep);
+    CCN_HIP(hipGetLastError());
+    return CCN_OK;
+  }
+  if (M % TM == 0 && N % TN == 0 && (size_t)128 * (size_t)N * 4 < 0x7fffffffull) {   // whole large tiles: the matrix-core-bound kernel
+    static const hipError_t attr = hipFuncSetAttribute((const void*)matmul_tile256_kernel<F16>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBigLds);
+    if (attr != hipSuccess) return hip_fail(attr);
+    const int tilesM = M / TM, tilesN = N / TN;
+    hipLaunchKernelGGL((matmul_tile256_kernel<F16>), dim3((unsigned)(tilesM * tilesN)), dim3(kBigBlock), kBigLds, as_stream(stream),
+                       X, W, C, N, K, tilesM, tilesN);
     CCN_HIP(hipGetLastError());
     return CCN_OK;
   }

@@ -101,6 +101,11 @@ def _declare(L):
     L.orc_epilogue_value_typed.argtypes = [_f, _f, _f, _i, _f, _i, _i]
 
 
+def set_num_threads(n):
+    """Host threads for the oracle's element-, segment- and row-parallel loops (1 = as the reference runs its checker)."""
+    lib().orc_set_num_threads(int(n))
+
+
 def _ptr(a, dtype):
     assert isinstance(a, np.ndarray) and a.dtype == dtype and a.flags["C_CONTIGUOUS"], (a.dtype, dtype)
     return a.ctypes.data_as(C.c_void_p)

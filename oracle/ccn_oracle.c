@@ -95,12 +95,21 @@ static inline float reduce_at(const float* const* g, int P, size_t i) {
   return s;
 }
 
+/* Host threads for the loops that are independent across elements (or across segments, or rows): 1 = the reference's
+ * single-threaded checker; more = the same loops under "omp parallel for" (static schedule, same arithmetic per
+ * element, same results), which is how bench.py times the CPU baseline on all cores of the GPU box. */
+static int orc_threads = 1;
+void orc_set_num_threads(int n) { orc_threads = n > 1 ? n : 1; }
+int orc_get_num_threads(void) { return orc_threads; }
+#define ORC_PARALLEL_FOR _Pragma("omp parallel for schedule(static) num_threads(orc_threads) if (orc_threads > 1)")
+
 void orc_reduce_f32(const float* const* g, int P, size_t N, float* out) {
   for (size_t i = 0; i < N; i++) out[i] = reduce_at(g, P, i);
 }
 
 /* examples/test-sgd.cu:17-18   __S1[i0] = (__w[i0] - (__lr * __S0[i0])) */
 void orc_sgd_f32(const float* const* g, int P, float* w, size_t N, float lr) {
+  ORC_PARALLEL_FOR
   for (size_t i = 0; i < N; i++) {
     float s0 = reduce_at(g, P, i);
     w[i] = (w[i] - (lr * s0));
@@ -220,6 +229,7 @@ void orc_adam_f32(const float* const* g, int P, float* w, float* m, float* v, si
   const double bc1 = 1 - pow((double)beta1, (double)step);
   const double bc2 = 1 - pow((double)beta2, (double)step);
   const float stepsize = -lr;
+  ORC_PARALLEL_FOR
   for (size_t i = 0; i < N; i++) {
     float gs = reduce_at(g, P, i);
     float mi = beta1 * m[i] + (1 - beta1) * gs;
@@ -250,6 +260,7 @@ uint32_t orc_adam_f16g(const uint16_t* const* g, int P, float* w, float* m, floa
   const double bc2 = 1 - pow((double)beta2, (double)step);
   const float stepsize = -lr;
   uint32_t flag = 0;
+  _Pragma("omp parallel for schedule(static) num_threads(orc_threads) if (orc_threads > 1) reduction(|:flag)")
   for (size_t i = 0; i < N; i++) {
     int bad = 0;
     float gs = 0.0f;
@@ -284,6 +295,7 @@ uint32_t orc_adam_bf16g(const uint16_t* const* g, int P, float* w, float* m, flo
   const double bc2 = 1 - pow((double)beta2, (double)step);
   const float stepsize = -lr;
   uint32_t flag = 0;
+  _Pragma("omp parallel for schedule(static) num_threads(orc_threads) if (orc_threads > 1) reduction(|:flag)")
   for (size_t i = 0; i < N; i++) {
     int bad = 0;
     float gs = 0.0f;
@@ -376,6 +388,7 @@ static void lamb_nccl_segment(const float* const* g, int P, float* w, float* m, 
 void orc_lamb_nccl_f16g(const uint16_t* const* g, int P, float* w, uint16_t* halfw, float* m, float* v,
                         const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2, float wd,
                         double* norms_out) {
+  ORC_PARALLEL_FOR
   for (int b = 0; b < nseg; b++) {
     const size_t lo = seg_offsets[b], hi = seg_offsets[b + 1];
     double rr = 0.0, ww = 0.0;
@@ -408,6 +421,7 @@ void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
                   const size_t* seg_offsets, int nseg, float lr, float beta1, float beta2,
                   float eps, float wd, int step, int mode, double* norms_out) {
   if (mode == 2) {
+    ORC_PARALLEL_FOR
     for (int b = 0; b < nseg; b++)
       lamb_nccl_segment(g, P, w, m, v, seg_offsets[b], seg_offsets[b + 1], lr, beta1, beta2, wd,
                         norms_out ? norms_out + 2 * b : NULL);
@@ -416,6 +430,7 @@ void orc_lamb_f32(const float* const* g, int P, float* w, float* m, float* v,
   const double bc1 = 1 - pow((double)beta1, (double)step);
   const double bc2 = 1 - pow((double)beta2, (double)step);
   const float stepsize = lr;
+  ORC_PARALLEL_FOR
   for (int b = 0; b < nseg; b++) {
     const size_t lo = seg_offsets[b], hi = seg_offsets[b + 1];
     const uint64_t n = (uint64_t)(hi - lo);
@@ -537,8 +552,9 @@ void orc_mlp_outproj_rows(const uint16_t* X, const uint16_t* W, const float* con
   /* Row i of X, partials, resid and out is row row_ids[i] of the whole output (i itself without a table): the dropout
    * draw of an element depends on its index in the whole output.  The product of a row is accumulated in float64 in
    * ascending k for every column (k outer, j inner: the same sum per element as a k-innermost loop, read along W's rows). */
-  double* acc = (double*)malloc((size_t)N * sizeof(double));
+  ORC_PARALLEL_FOR
   for (int i = 0; i < M; i++) {
+    double* acc = (double*)malloc((size_t)N * sizeof(double));
     for (int j = 0; j < N; j++) acc[j] = 0.0;
     for (int k = 0; k < K; k++) {
       const uint16_t xb = X[(size_t)i * K + k];
@@ -558,8 +574,8 @@ void orc_mlp_outproj_rows(const uint16_t* X, const uint16_t* W, const float* con
       if (out_f32) out_f32[idx] = y;
       if (out) out[idx] = half ? orc_f32_to_f16(y) : orc_f32_to_bf16(y);
     }
+    free(acc);
   }
-  free(acc);
 }
 
 void orc_mlp_outproj_typed(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,

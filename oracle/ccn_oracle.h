@@ -52,6 +52,11 @@
 extern "C" {
 #endif
 
+/* Host threads for the element-, segment- and row-parallel loops (default 1, the reference's single-threaded checker);
+ * results do not depend on it. */
+void orc_set_num_threads(int n);
+int  orc_get_num_threads(void);
+
 /* ---- scalar conversions (IEEE binary16 / bfloat16, round-to-nearest-even) ---- */
 uint16_t orc_f32_to_f16(float f);
 float    orc_f16_to_f32(uint16_t h);

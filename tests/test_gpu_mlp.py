@@ -522,3 +522,56 @@ def test_plain_product(ccn):
     with pytest.raises(ccn.CoconetError) as e:
         ccn.matmul_bf16_f32(bf16_dev(X), bf16_dev(W), Cd, M, N - 2, K)   # a quad of columns must stay inside a row
     assert e.value.code == ccn.CCN_ERANGE
+
+
+@pytest.mark.parametrize("M,N,K,half", [(256, 256, 64, False), (512, 768, 192, False), (1024, 2048, 128, False), (256, 512, 1024, True),
+                                        (2048, 256, 64, False), (768, 1280, 320, False)])
+def test_plain_product_on_large_tiles(ccn, M, N, K, half):
+    """Whole multiples of 256 rows and columns take the 256 x 256-tile kernel of the plain product: exact on small integers
+    (a one-hot X picks rows of an integer W: any transposed, swizzled or mis-dealt index shows as a wrong integer; all-ones
+    gives K, the reference's own check at this boundary), within the fp32-accumulation bound of float64 on random operands.
+    Tile counts that do and do not divide into the blocks of 4 x 8 tiles the workgroups are dealt in."""
+    r = rng(300 + M // 256 + N // 256)
+    to16 = (lambda a: a.astype(np.float16).view(np.uint16)) if half else (lambda a: orc.f32_to_bf16(a.astype(np.float32)))
+    wide = (lambda b: b.view(np.float16).astype(np.float64)) if half else (lambda b: orc.bf16_to_f32(b).astype(np.float64))
+    Cd = torch.full((M, N), -7.0, device=DEV)
+    sel = r.integers(0, K, M)
+    Xf = np.zeros((M, K), np.float32)
+    Xf[np.arange(M), sel] = 1.0
+    Wf = r.integers(-64, 64, (K, N)).astype(np.float32)
+    ccn.matmul_bf16_f32(u16_dev(to16(Xf)), u16_dev(to16(Wf)), Cd, M, N, K, half=half)
+    torch.cuda.synchronize()
+    assert np.array_equal(Cd.cpu().numpy(), Wf[sel])
+    ones = lambda shape: u16_dev(to16(np.ones(shape, np.float32)))
+    ccn.matmul_bf16_f32(ones((M, K)), ones((K, N)), Cd, M, N, K, half=half)
+    torch.cuda.synchronize()
+    assert torch.all(Cd == K)
+    X = to16(r.standard_normal((M, K)))
+    W = to16(r.standard_normal((K, N)) * 0.02)
+    ccn.matmul_bf16_f32(u16_dev(X), u16_dev(W), Cd, M, N, K, half=half)
+    torch.cuda.synchronize()
+    xf, wf = wide(X), wide(W)
+    bound = K * 2.0 ** -24 * (np.abs(xf) @ np.abs(wf))
+    assert np.all(np.abs(Cd.cpu().numpy().astype(np.float64) - xf @ wf) <= bound + 1e-30)
+
+
+def test_plain_product_config5_shape(ccn):
+    """8192 x 1024 x 8192 through the large-tile kernel: sampled rows against float64 (every row position inside a tile in
+    the first and the last tile row), and a checksum over the whole product: sum_ij C_ij = sum_k (sum_i X_ik)(sum_j W_kj)."""
+    M = N = 8192
+    K = 1024
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(15)
+    X = torch.randn(M, K, device=DEV, generator=gen).to(torch.bfloat16)
+    W = (torch.randn(K, N, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+    Cd = torch.empty(M, N, device=DEV)
+    ccn.matmul_bf16_f32(X, W, Cd, M, N, K)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, 256), torch.arange(M - 256, M)]).to(DEV)
+    ref = X[rows].double() @ W.double()
+    bound = K * 2.0 ** -24 * (X[rows].double().abs() @ W.double().abs())
+    assert bool(((Cd[rows].double() - ref).abs() <= bound + 1e-30).all())
+    total = float(Cd.double().sum())
+    want = float((X.double().sum(dim=0) * W.double().sum(dim=1)).sum())
+    mag = float((X.double().abs().sum(dim=0) * W.double().abs().sum(dim=1)).sum())
+    assert abs(total - want) <= K * 2.0 ** -24 * mag
