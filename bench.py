@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adam_f32",
                     choices=["adam_f32", "adam_f32_scattered", "sgd_f32", "adam_f16g", "adam_bf16g", "lamb_f32",
-                             "lamb_nccl_f16g", "mlp_outproj", "matmul_bf16", "copy"])
+                             "lamb_nccl_f16g", "mlp_outproj", "matmul_bf16", "copy", "copy_stream"])
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -301,6 +301,19 @@ def build_workload(a, wl, capi, torch, stream, allocator):
         units = M * Nn
         kernel = "mlp_outproj_kernel<0, true>"
         config = {"workload": "matmul bf16 8192x1024x8192 -> fp32 (the unfused schedule's MatMul step)", "M": M, "N": Nn, "K": Kd}
+    elif wl == "copy_stream":
+        # a 1R:1W stream through the library's own streaming kernel (ccn_reduce_f32 over one rank buffer is a copy): the
+        # ceiling of this box for the launch shape the fused kernels use
+        N = 1 << (a.log2n or 30)
+        bufs = Buffers(capi, torch, allocator == "torch")
+        src = bufs.from_tensor(torch.empty(N, dtype=torch.float32, device="cuda").normal_(generator=gen))
+        dst = bufs.from_tensor(torch.empty(N, dtype=torch.float32, device="cuda"))
+        step = lambda t: capi.reduce_f32([src], dst, N, stream)
+        alg_bytes = 8.0 * N
+        units = N
+        kernel = "fused_stream_kernel<ReduceMath, 1, 4, 1, 256>"
+        config = {"workload": f"copy of 2^{int(np.log2(N))} fp32 through the library's streaming kernel (ccn_reduce_f32, P=1)"}
+        keep = [bufs]
     else:   # plain device copy, the practical HBM ceiling of this box
         N = 1 << (a.log2n or 30)
         src = torch.empty(N, dtype=torch.float32, device="cuda").normal_(generator=gen)
@@ -365,7 +378,7 @@ def other_workloads(a, capi, torch, stream):
                      "algorithmic_bytes_per_launch": c["roofline"]["algorithmic_bytes_per_launch"], "traffic": None})
     except (ValueError, KeyError, IndexError):
         rows.append({"workload": "adam_f32 on plain allocations", "error": (child.stderr or child.stdout)[-300:]})
-    for wl, allocator in (("copy", "torch"), ("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_graph", "ccn"),
+    for wl, allocator in (("copy", "torch"), ("copy_stream", "ccn"), ("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_graph", "ccn"),
                           ("sgd_f32_large", "ccn"), ("adam_f16g", "ccn"), ("lamb_f32", "ccn"), ("mlp_outproj", "ccn"),
                           ("matmul_bf16", "ccn")):
         replay = 64 if wl == "sgd_f32_graph" else 0      # configuration 1 again, 64 recorded steps per graph launch
@@ -394,7 +407,10 @@ def other_workloads(a, capi, torch, stream):
         if alg_bytes < 1e9 and wl != "matmul_bf16":
             row["note"] = "fits the caches and is bound by launches: not a roofline figure"
         if wl == "copy":
-            row["note"] = "the measured ceiling of a 1R:1W stream on this box, to read the fractions of the 8 TB/s nominal peak against"
+            row["note"] = "torch's device-to-device copy_ on this box"
+        if wl == "copy_stream":
+            row["note"] = ("the measured ceiling of a 1R:1W stream on this box in the launch shape of the fused kernels: read the "
+                           "fractions of the 8 TB/s nominal peak against it")
         if replay:
             graph.close()
             own.close()
@@ -481,7 +497,7 @@ def main():
         del step
         release(keep, capi, torch)
         line["other_workloads"] = other_workloads(a, capi, torch, stream)
-    if wl != "copy" and not a.no_cpu_baseline:
+    if wl not in ("copy", "copy_stream") and not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl, P if wl not in ("mlp_outproj", "matmul_bf16") else 8)
     print(json.dumps(line), flush=True)
 
