@@ -5,6 +5,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
 
@@ -134,9 +135,10 @@ constexpr size_t kStaggerMin = 4u << 20;       // only buffers of at least 4 MiB
 constexpr size_t kStaggerStep = 4 * 1024;
 constexpr size_t kStaggerSlots = 16;
 constexpr size_t kStaggerPad = kStaggerStep * kStaggerSlots;
-std::mutex g_alloc_mu;
+std::mutex g_alloc_mu;                            // guards the map only; hipMalloc / hipFree run outside it
 std::unordered_map<void*, void*> g_alloc_base;   // pointer given to the caller -> hipMalloc base
-unsigned g_alloc_count = 0;
+std::atomic<size_t> g_alloc_count{0};             // staggered allocations so far: picks the slot
+std::atomic<size_t> g_alloc_live{0};              // staggered allocations not yet freed: ccn_free skips the map at zero
 }  // namespace
 
 int ccn_malloc(void** p, size_t bytes) {
@@ -149,15 +151,16 @@ int ccn_malloc(void** p, size_t bytes) {
   }
   void* base = nullptr;
   CCN_HIP(hipMalloc(&base, bytes + kStaggerPad));
+  // Allocation c takes slot (c + c/16 + c/256 + c/4096) mod 16: allocations 1, 16, 256 or 4096 apart in the
+  // sequence all land in different slots, so the arrays walked in lock step differ whether the caller allocated
+  // rank by rank or tensor by tensor.
+  const size_t c = g_alloc_count.fetch_add(1, std::memory_order_relaxed);
+  const size_t slot = (c + c / 16 + c / 256 + c / 4096) % kStaggerSlots;
+  void* const user = static_cast<char*>(base) + slot * kStaggerStep;
   const int rc = guarded([&] {
     std::lock_guard<std::mutex> lock(g_alloc_mu);
-    // Allocation c takes slot (c + c/16 + c/256 + c/4096) mod 16: allocations 1, 16, 256 or 4096 apart in the
-    // sequence all land in different slots, so the arrays walked in lock step differ whether the caller allocated
-    // rank by rank or tensor by tensor.
-    const size_t c = g_alloc_count++;
-    const size_t slot = (c + c / 16 + c / 256 + c / 4096) % kStaggerSlots;
-    void* user = static_cast<char*>(base) + slot * kStaggerStep;
     g_alloc_base[user] = base;
+    g_alloc_live.fetch_add(1, std::memory_order_release);
     *p = user;
     return CCN_OK;
   });
@@ -168,12 +171,13 @@ int ccn_malloc(void** p, size_t bytes) {
 int ccn_free(void* p) {
   if (!p) return CCN_OK;
   void* base = p;
-  {
+  if (g_alloc_live.load(std::memory_order_acquire) != 0) {   // small buffers, and any buffer while nothing is staggered, go straight on
     std::lock_guard<std::mutex> lock(g_alloc_mu);
     auto it = g_alloc_base.find(p);
     if (it != g_alloc_base.end()) {
       base = it->second;
       g_alloc_base.erase(it);
+      g_alloc_live.fetch_sub(1, std::memory_order_release);
     }
   }
   CCN_HIP(hipFree(base));

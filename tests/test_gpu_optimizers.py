@@ -1032,3 +1032,29 @@ def test_seeded_random_scattered_buffers(ccn, case):
     assert_f32_parity(host(vd), v, what + " lamb v")
     got = np.concatenate([host(x) for x in wd])
     assert np.max(np.abs(got.astype(np.float64) - w)) <= FP32_TOL * float(np.max(np.abs(w))), what
+
+
+def test_lamb_plan_knobs_reject_what_they_do_not_know(ccn):
+    """ccn_lamb_plan_tune: unknown knobs and negative values are CCN_EINVAL and change nothing; a spin limit beyond 2^31-1
+    is CCN_ERANGE; setting and clearing the two-pass knob between steps gives the oracle's result either way."""
+    segs = [0, 8192, 3 * 8192, 3 * 8192 + 777]
+    N = segs[-1]
+    plan = ccn.LambPlan(segs, knobs={})
+    for knob, value, code in [(7, 1, ccn.CCN_EINVAL), (-1, 0, ccn.CCN_EINVAL), (SPIN, -5, ccn.CCN_EINVAL), (SPIN, 1 << 40, ccn.CCN_ERANGE)]:
+        with pytest.raises(ccn.CoconetError) as e:
+            plan.tune(knob, value)
+        assert e.value.code == code, (knob, value)
+    g = grads_f32(97, 3, N, 1e-3)
+    w0 = weights_f32(97, N, 0.05)
+    gd, wd = [dev(x) for x in g], dev(w0)
+    md, vd = torch.zeros(N, device=DEV), torch.zeros(N, device=DEV)
+    w, m, v = w0.copy(), np.zeros(N, np.float32), np.zeros(N, np.float32)
+    for t, two_pass in ((1, 0), (2, 1), (3, 0)):
+        plan.tune(TWO_PASS, two_pass)
+        plan.step(gd, wd, md, vd, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+        want = orc.lamb_f32(g, w, m, v, segs, 1e-3, 0.9, 0.999, 1e-6, 0.01, t, 0)
+        assert rel_err(plan.norms(), want) < 1e-9, (t, two_pass)
+    assert_f32_parity(host(md), m, "knobs m")
+    assert_f32_parity(host(vd), v, "knobs v")
+    assert ulp_diff_f32(host(wd), w) <= 4
+    plan.close()
