@@ -378,9 +378,9 @@ def other_workloads(a, capi, torch, stream):
                      "algorithmic_bytes_per_launch": c["roofline"]["algorithmic_bytes_per_launch"], "traffic": None})
     except (ValueError, KeyError, IndexError):
         rows.append({"workload": "adam_f32 on plain allocations", "error": (child.stderr or child.stdout)[-300:]})
-    for wl, allocator in (("copy", "torch"), ("copy_stream", "ccn"), ("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_graph", "ccn"),
-                          ("sgd_f32_large", "ccn"), ("adam_f16g", "ccn"), ("lamb_f32", "ccn"), ("mlp_outproj", "ccn"),
-                          ("matmul_bf16", "ccn")):
+    for wl, allocator in (("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_graph", "ccn"), ("sgd_f32_large", "ccn"),
+                          ("adam_f16g", "ccn"), ("lamb_f32", "ccn"), ("mlp_outproj", "ccn"), ("matmul_bf16", "ccn"),
+                          ("copy", "torch"), ("copy_stream", "ccn")):
         replay = 64 if wl == "sgd_f32_graph" else 0      # configuration 1 again, 64 recorded steps per graph launch
         own = capi.Stream() if replay else None          # the null stream cannot be recorded
         st = own.h if own else stream
