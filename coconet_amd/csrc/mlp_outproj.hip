@@ -371,28 +371,23 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
   const uint32_t woff = (uint32_t)((wk * N + 8 * (wc ^ (4 * (wk & 3)))) * 2), wrow16 = (uint32_t)(16 * N * 2);
   const rsrc_t x_rs = buffer_at(X + m0 * (size_t)K);
   const uint16_t* const wbase = W + n0;
-  // two sets of staging registers: the operands of step s wait in set s%2, requested two K-steps before their use
-  u32x4 sx[2][4], sw[2][4];
-  auto load_stage = [&](auto set, int k0) {
-    constexpr int S = decltype(set)::value;
+  // staging registers: the operands of the next step, requested at the top of a step and moved into the other LDS stage
+  // under its last round
+  u32x4 sx[4], sw[4];
+  auto load_stage = [&](int k0) {
     const rsrc_t w_rs = buffer_at(wbase + (size_t)k0 * N);
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      sx[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rs, xoff, (uint32_t)j * xrow64 + (uint32_t)k0 * 2u, 0));
-      sw[S][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w_rs, woff, (uint32_t)j * wrow16, 0));
+      sx[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rs, xoff, (uint32_t)j * xrow64 + (uint32_t)k0 * 2u, 0));
+      sw[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w_rs, woff, (uint32_t)j * wrow16, 0));
     }
   };
-  auto store_quarter = [&](auto set, int buf, int j) {
-    constexpr int S = decltype(set)::value;
+  auto store_quarter = [&](int buf, int j) {
     uint8_t* const lx = lds_big + buf * kBigStage;
     uint8_t* const lw = lx + TM * BK * 2;
     const int row = xr_ + 64 * j;
-    *reinterpret_cast<u32x4*>(lx + row * 128 + ((xc ^ ((row >> 1) & 7)) << 4)) = sx[S][j];
-    *reinterpret_cast<u32x4*>(lw + ((wk + 16 * j) * 32 + wc) * 16) = sw[S][j];
-  };
-  auto store_stage = [&](auto set, int buf) {
-#pragma unroll
-    for (int j = 0; j < 4; j++) store_quarter(set, buf, j);
+    *reinterpret_cast<u32x4*>(lx + row * 128 + ((xc ^ ((row >> 1) & 7)) << 4)) = sx[j];
+    *reinterpret_cast<u32x4*>(lw + ((wk + 16 * j) * 32 + wc) * 16) = sw[j];
   };
   // fragment addresses: X rows 128*wm + 32*bm + li, chunk 2*ks + lh; W fragment bn of this wavefront's 64 columns
   int xaddr[4];
@@ -422,68 +417,81 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
 
-  // One K-step from LDS stage `buf` as 16 phases (round ks, row block bm) of two MFMAs each.  A phase reads the X fragment
-  // of the next phase, and the last two phases of a round the two W fragments of the next round, so that the fragments
-  // in flight stay at 6 registers sets; `write_next(i)` is called in phase i of the last round (i = 0..3) to move a
-  // quarter of the next step's operands from their staging registers into the other stage.
-  auto mfma_step = [&](int buf, auto&& write_next) {
-    s16x8 fw[2][2], fx[2];
-    fw[0][0] = read_w(buf, 0, 0);
-    fw[0][1] = read_w(buf, 1, 0);
-    fx[0] = read_x(buf, 0, 0);
+  // A round of 16 k: two W and four X fragments for eight MFMAs.  The six fragments of the NEXT round are read under this
+  // round's MFMAs (a whole round ahead: more than the LDS latency, so a wavefront rarely waits for a fragment and the
+  // second wavefront of its SIMD finds the matrix core busy, not idle).  Rounds alternate between two fragment sets.
+  s16x8 fw[2][2], fx[2][4];
+  auto read_frags = [&](int set, int buf, int ks) {
 #pragma unroll
-    for (int ph = 0; ph < 16; ph++) {
-      const int ks = ph >> 2, bm = ph & 3;
-      int reads = 0;
-      if (ph + 1 < 16) { fx[(ph + 1) & 1] = read_x(buf, (ph + 1) & 3, (ph + 1) >> 2); reads += 1; }
-      if (ks + 1 < 4 && bm >= 2) { fw[(ks + 1) & 1][bm - 2] = read_w(buf, bm - 2, ks + 1); reads += 2; }
-      if (ks == 3) write_next(bm);
+    for (int bn = 0; bn < 2; bn++) fw[set][bn] = read_w(buf, bn, ks);
+#pragma unroll
+    for (int bm = 0; bm < 4; bm++) fx[set][bm] = read_x(buf, bm, ks);
+  };
+  auto mfma_round = [&](int set) {
+#pragma unroll
+    for (int bm = 0; bm < 4; bm++)
 #pragma unroll
       for (int bn = 0; bn < 2; bn++) {
         if constexpr (F16)
-          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fw[ks & 1][bn]), __builtin_bit_cast(f16x8, fx[ph & 1]), acc[bn][bm], 0, 0, 0);
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fw[set][bn]), __builtin_bit_cast(f16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
         else
-          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fw[ks & 1][bn]), __builtin_bit_cast(bf16x8, fx[ph & 1]), acc[bn][bm], 0, 0, 0);
+          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fw[set][bn]), __builtin_bit_cast(bf16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
       }
-      // issue order of the phase: its LDS reads (and writes), then its two MFMAs
-      if (reads == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (reads == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      if (reads == 3) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
-      if (ks == 3) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+  };
+  // issue order of a round: `lds_per_mfma` LDS operations, then `vmem` loads spread over the first MFMAs, one MFMA at a time
+  auto interleave = [&](auto reads, auto writes, auto vmem) {
+    constexpr int R = decltype(reads)::value, Wr = decltype(writes)::value, V = decltype(vmem)::value;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if (R) __builtin_amdgcn_sched_group_barrier(0x100, R, 0);
+      if (Wr) __builtin_amdgcn_sched_group_barrier(0x200, Wr, 0);
+      if (V) __builtin_amdgcn_sched_group_barrier(0x020, V, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
   auto lds_barrier = [&]() {
     __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): this wavefront's LDS writes are done; global loads stay in flight
     __builtin_amdgcn_s_barrier();
   };
 
-  // main loop, two steps per turn so that the staging sets are compile-time names: step kt multiplies from LDS stage
-  // kt%2, requests the operands of step kt+2 (past the end: the last step's again, unused) and, under its last round,
-  // moves those of step kt+1 from their registers into the other stage
+  // Main loop, software-pipelined so that no LDS latency is left in the open: step kt multiplies from stage kt%2;
+  //   rounds 0, 1   MFMAs, reading the next round's fragments
+  //   round 2       the same, and the operands of step kt+1 go from their staging registers into the other stage
+  //   barrier       (every wavefront's LDS operations are complete before it arrives: nobody still reads what the next
+  //                  step's round 2 will overwrite, everybody's writes are in place)
+  //   round 3       MFMAs, reading round 0 of step kt+1 from the other stage, and requesting the operands of step kt+2
+  //                 (past the end: the last step's again, unused) a whole step ahead of their trip into LDS
   const int nk = K / BK;
-  using Set0 = std::integral_constant<int, 0>;
-  using Set1 = std::integral_constant<int, 1>;
   auto clamp_k = [&](int kt) { return (kt < nk ? kt : nk - 1) * BK; };
-  load_stage(Set0{}, 0);
-  load_stage(Set1{}, clamp_k(1));
-  store_stage(Set0{}, 0);
+  load_stage(0);
+#pragma unroll
+  for (int j = 0; j < 4; j++) store_quarter(0, j);
+  load_stage(clamp_k(1));
   lds_barrier();
-  auto step = [&](auto set, int kt) {   // set = kt % 2
-    constexpr int S = decltype(set)::value;
-    load_stage(set, clamp_k(kt + 2));
-    __builtin_amdgcn_sched_barrier(0);   // the requests go out first, two K-steps ahead of their use
-    mfma_step(S, [&](int j) { store_quarter(std::integral_constant<int, 1 - S>{}, 1 - S, j); });
+  read_frags(0, 0, 0);
+  for (int kt = 0; kt < nk; kt++) {
+    const int buf = kt & 1;
+    read_frags(1, buf, 1);
+    mfma_round(0);
+    interleave(I1{}, I0{}, I0{});
+    read_frags(0, buf, 2);
+    mfma_round(1);
+    interleave(I1{}, I0{}, I0{});
+    read_frags(1, buf, 3);
+#pragma unroll
+    for (int j = 0; j < 4; j++) store_quarter(buf ^ 1, j);
+    mfma_round(0);
+    interleave(I1{}, I1{}, I0{});
     lds_barrier();
-  };
-  // (the last step's requests and LDS writes are redundant and harmless: nothing reads that stage any more)
-  int kt = 0;
-  for (; kt + 1 < nk; kt += 2) {
-    step(Set0{}, kt);
-    step(Set1{}, kt + 1);
+    load_stage(clamp_k(kt + 2));
+    read_frags(0, buf ^ 1, 0);
+    mfma_round(1);
+    interleave(I1{}, I0{}, I1{});
   }
-  if (kt < nk) step(Set0{}, kt);   // an odd number of steps
+  lds_barrier();   // the last round's reads of LDS are done everywhere before the stages become C pieces
   // every wavefront is past the last step's barrier and done with the operand stages: LDS becomes eight private C pieces
   constexpr int kCS = 64 + 4;   // floats per row of a piece: 32 rows x 64 columns at a time
   float* const cw = reinterpret_cast<float*>(lds_big) + wave * (32 * kCS);
