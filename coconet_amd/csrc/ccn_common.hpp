@@ -196,8 +196,9 @@ unsigned stream_grid(size_t units, size_t tile);
 // 256-thread workgroups 82%; 7 wavefronts per CU as single-wavefront workgroups 85%; 4 wavefronts 63-70%.  A 2-stream
 // copy wants all the occupancy it can get.
 struct StreamShape { int block; unsigned lds_bytes; };
-// Shape for a kernel whose threads each load `load_bytes` and store `store_bytes`, one pack per array.
-StreamShape stream_shape(int load_bytes, int store_bytes);
+// Shape for a kernel whose threads each load `load_bytes` and store `store_bytes`, one pack per array; `grad_bytes` is
+// the element size of the gradient arrays (narrow elements mean more load instructions for the same bytes).
+StreamShape stream_shape(int load_bytes, int store_bytes, int grad_bytes = 4);
 // Dynamic LDS request that keeps at most `per_cu` workgroups on a CU (0 = no request).
 unsigned lds_for_residency(int per_cu);
 

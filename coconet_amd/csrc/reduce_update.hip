@@ -412,7 +412,7 @@ static int launch_one(const typename M::G* const* g, int nP, const StateTable<M:
   const size_t nvec = n / VEC;
   const int load_bytes = VEC * (nP * (int)sizeof(typename M::G) + M::NS * 4);
   const int store_bytes = VEC * (M::NS * 4 + (M::OUT16 ? 2 : 0) + (M::OUTF ? 4 : 0));
-  const StreamShape sh = stream_shape(load_bytes, store_bytes);
+  const StreamShape sh = stream_shape(load_bytes, store_bytes, (int)sizeof(typename M::G));
   size_t tiles = (nvec + (size_t)sh.block * UNROLL - 1) / ((size_t)sh.block * UNROLL);
   if (tiles < 1) tiles = 1;                                     // the n % VEC tail still needs workgroup 0
   const size_t gx = tiles < 0x40000000ull ? tiles : 0x40000000ull;
