@@ -331,15 +331,20 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
 // C[M x N] (fp32) = X . W alone is bound by the matrix cores, and a 128 x 128 tile moves too many operand bytes per MFMA
 // to keep them busy.  For whole multiples of 256 rows and columns: a 512-thread workgroup owns a 256(m) x 256(n) tile,
 // its 8 wavefronts as 2(m) x 4(n), each 128 x 64 as eight 32 x 32 blocks (128 accumulator registers); per 16-k round a
-// wavefront reads four X and two W fragments from LDS for eight MFMAs.  Two LDS stages of 64 KiB (X: rows of 128 bytes,
-// chunks swizzled by (row/2)%8; W as it lies in memory, rows of 512 bytes, chunks swizzled by 4*(k%4), read back through
-// ds_read_b64_tr_b16), operands staged through registers one K-step ahead, one barrier per K-step, one workgroup per CU.
+// wavefront reads four X and two W fragments from LDS for eight MFMAs.  One workgroup per CU.
+// The operands travel global memory -> LDS directly (no staging registers, no LDS store instructions) into a ring of
+// four stages of 32 k (X: 256 rows of 64 bytes, chunks swizzled by (row/4)%4; W as it lies in memory, 32 rows of 512
+// bytes, chunks swizzled by 4*(k%4), read back through ds_read_b64_tr_b16).  A wavefront requests one KiB every fourth
+// MFMA, all the time: the CU's address path takes 16 cycles per request, and eight wavefronts asking for a whole step
+// at once stand in its queue instead of issuing MFMAs.  A request is waited for three steps after it was made.
 // Workgroups are numbered so that the 32 an XCD runs at a time form a block of 4 x 8 tiles: their X and W panels are
 // shared inside that XCD's L2.  The accumulators leave through wavefront-private pieces of LDS as whole 256-byte rows.
 constexpr int TM = 256, TN = 256;
 constexpr int kBigBlock = 512;
-constexpr int kBigStage = (TM + TN) * BK * 2;     // one K-step of X and W: 64 KiB
-constexpr int kBigLds = 2 * kBigStage;
+constexpr int kBigK = 32;                            // k per stage
+constexpr int kBigStage = (TM + TN) * kBigK * 2;     // one step of X and W: 32 KiB
+constexpr int kBigStages = 4;
+constexpr int kBigLds = kBigStages * kBigStage;
 
 template <bool F16>
 __global__ __launch_bounds__(kBigBlock) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -365,45 +370,50 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
   const int wm = wave >> 2, wn = wave & 3;
   const int li = lane & 31, lh = lane >> 5;
 
-  // staging: X rows (t/8) + 64*j, chunk t%8; W rows (t/32) + 16*j, chunk t%32 (memory chunk c lives at position c ^ 4*(k%4))
-  const int xr_ = t >> 3, xc = t & 7, wk = t >> 5, wc = t & 31;
-  const uint32_t xoff = (uint32_t)((xr_ * K + xc * 8) * 2), xrow64 = (uint32_t)(64 * K * 2);
-  const uint32_t woff = (uint32_t)((wk * N + 8 * (wc ^ (4 * (wk & 3)))) * 2), wrow16 = (uint32_t)(16 * N * 2);
-  const rsrc_t x_rs = buffer_at(X + m0 * (size_t)K);
-  const uint16_t* const wbase = W + n0;
-  // staging registers: the operands of the next step, requested at the top of a step and moved into the other LDS stage
-  // under its last round
-  u32x4 sx[4], sw[4];
-  auto load_stage = [&](int k0) {
-    const rsrc_t w_rs = buffer_at(wbase + (size_t)k0 * N);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      sx[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rs, xoff, (uint32_t)j * xrow64 + (uint32_t)k0 * 2u, 0));
-      sw[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w_rs, woff, (uint32_t)j * wrow16, 0));
-    }
+  // A direct-to-LDS load fills 1 KiB, lane L its 16 bytes at position L, so the swizzles are applied on the global side:
+  // lane L fetches the chunk that belongs at L.  Per stage wavefront w brings the X rows 16*(w + 8j).. (16 rows of 64
+  // bytes) and the W rows 2*(w + 8j).. (2 rows of 512 bytes), j = 0, 1.  X: position (row, slot) holds memory chunk
+  // slot ^ (row/4)%4; W: position (k, slot) holds chunk slot ^ 4*(k%4).
+  const uint32_t xvoff = (uint32_t)(((lane >> 2) * K + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
+  const uint32_t wvoff = (uint32_t)(((lane >> 5) * N + 8 * ((lane & 31) ^ (4 * (2 * (wave & 1) + (lane >> 5))))) * 2);
+  // The loads are written as assembly: the compiler orders every LDS read after a direct-to-LDS load it can see behind a
+  // wait for ALL outstanding loads, which would put the memory latency into every step.  Here the only reads of a
+  // stage follow the wait and barrier below, so the waits are placed by hand.
+  auto words = [](const void* base) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    return u32x4{(uint32_t)a, (uint32_t)(a >> 32), 0x7ffffffcu, 0x00020000u};   // no stride, no bounds, as buffer_at()
   };
-  auto store_quarter = [&](int buf, int j) {
-    uint8_t* const lx = lds_big + buf * kBigStage;
-    uint8_t* const lw = lx + TM * BK * 2;
-    const int row = xr_ + 64 * j;
-    *reinterpret_cast<u32x4*>(lx + row * 128 + ((xc ^ ((row >> 1) & 7)) << 4)) = sx[j];
-    *reinterpret_cast<u32x4*>(lw + ((wk + 16 * j) * 32 + wc) * 16) = sw[j];
+  auto load_to_lds = [](u32x4 rs, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rs), "s"(soff) : "memory");
+  };
+  const u32x4 x_rs = words(X + m0 * (size_t)K), w_rs = words(W + n0);
+  typedef __attribute__((address_space(3))) void* lds_void_ptr;
+  const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((lds_void_ptr)lds_big) + (uint32_t)wave * 1024u;
+  const int nk = K / kBigK;
+  // half j (0, 1) of the X / W operands of step `kt` (past the end: the last step's again, unused), into stage `stage`
+  const uint32_t xs0 = (uint32_t)(16 * wave * K * 2), xs1 = (uint32_t)((16 * wave + 128) * K * 2);
+  const uint32_t ws0 = (uint32_t)(2 * wave * N * 2), ws1 = (uint32_t)((2 * wave + 16) * N * 2);
+  const uint32_t wstep = (uint32_t)(kBigK * N * 2);
+  auto request_x = [&](int stage, int kt, int j) {
+    const uint32_t kc = (uint32_t)(kt < nk ? kt : nk - 1);
+    load_to_lds(x_rs, lds0 + stage * kBigStage + j * 8192, xvoff, (j ? xs1 : xs0) + kc * (kBigK * 2));
+  };
+  auto request_w = [&](int stage, int kt, int j) {
+    const uint32_t kc = (uint32_t)(kt < nk ? kt : nk - 1);
+    load_to_lds(w_rs, lds0 + stage * kBigStage + TM * kBigK * 2 + j * 8192, wvoff, (j ? ws1 : ws0) + kc * wstep);
   };
   // fragment addresses: X rows 128*wm + 32*bm + li, chunk 2*ks + lh; W fragment bn of this wavefront's 64 columns
   int xaddr[4];
 #pragma unroll
-  for (int bm = 0; bm < 4; bm++) {
-    const int row = 128 * wm + 32 * bm + li;
-    xaddr[bm] = row * 128;   // + ((2*ks + lh) ^ swizzle) * 16
-  }
-  const int xsw = (li >> 1) & 7;   // (row/2) % 8: the rows of a fragment start at a multiple of 32
+  for (int bm = 0; bm < 4; bm++) xaddr[bm] = (128 * wm + 32 * bm + li) * 64;   // + ((2*ks + lh) ^ swizzle) * 16
+  const int xsw = (li >> 2) & 3;   // (row/4) % 4: the rows of a fragment start at a multiple of 32
   const int a16 = lane & 15, g2 = (lane >> 4) & 1;
   const int waddr = ((lh * 8 + (a16 >> 2)) * 32 + ((8 * wn + 2 * g2 + ((a16 >> 1) & 1)) ^ (4 * (a16 >> 2)))) * 16 + 8 * (a16 & 1);
   auto read_x = [&](int buf, int bm, int ks) {
     return *reinterpret_cast<const s16x8*>(lds_big + buf * kBigStage + xaddr[bm] + (((2 * ks + lh) ^ xsw) << 4));
   };
   auto read_w = [&](int buf, int bn, int ks) {
-    const uint8_t* p = lds_big + buf * kBigStage + TM * BK * 2 + (waddr ^ (bn * 64)) + ks * (16 * 512);
+    const uint8_t* p = lds_big + buf * kBigStage + TM * kBigK * 2 + (waddr ^ (bn * 64)) + ks * (16 * 512);
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
     const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * 512));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -417,81 +427,70 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
 
-  // A round of 16 k: two W and four X fragments for eight MFMAs.  The six fragments of the NEXT round are read under this
-  // round's MFMAs (a whole round ahead: more than the LDS latency, so a wavefront rarely waits for a fragment and the
-  // second wavefront of its SIMD finds the matrix core busy, not idle).  Rounds alternate between two fragment sets.
+  // A round of 16 k: two W and four X fragments for eight MFMAs, in two alternating fragment sets.  A round multiplies
+  // from set `set` while the six fragments of the NEXT round are read into the other set from (stage rbuf, round rks)
+  // in the order the next round's MFMAs need them, one LDS instruction per MFMA; after the fourth and the eighth MFMA the
+  // round makes request `j` for step `lkt`.  Every piece is pinned in place: the order IS the schedule.
   s16x8 fw[2][2], fx[2][4];
-  auto read_frags = [&](int set, int buf, int ks) {
-#pragma unroll
-    for (int bn = 0; bn < 2; bn++) fw[set][bn] = read_w(buf, bn, ks);
-#pragma unroll
-    for (int bm = 0; bm < 4; bm++) fx[set][bm] = read_x(buf, bm, ks);
+  auto mfma = [&](int set, int bm, int bn) {
+    if constexpr (F16)
+      acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fw[set][bn]), __builtin_bit_cast(f16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
+    else
+      acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fw[set][bn]), __builtin_bit_cast(bf16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
   };
-  auto mfma_round = [&](int set) {
-#pragma unroll
-    for (int bm = 0; bm < 4; bm++)
-#pragma unroll
-      for (int bn = 0; bn < 2; bn++) {
-        if constexpr (F16)
-          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fw[set][bn]), __builtin_bit_cast(f16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
-        else
-          acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fw[set][bn]), __builtin_bit_cast(bf16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
-      }
-  };
-  // issue order of a round: `lds_per_mfma` LDS operations, then `vmem` loads spread over the first MFMAs, one MFMA at a time
-  auto interleave = [&](auto reads, auto writes, auto vmem) {
-    constexpr int R = decltype(reads)::value, Wr = decltype(writes)::value, V = decltype(vmem)::value;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      if (R) __builtin_amdgcn_sched_group_barrier(0x100, R, 0);
-      if (Wr) __builtin_amdgcn_sched_group_barrier(0x200, Wr, 0);
-      if (V) __builtin_amdgcn_sched_group_barrier(0x020, V, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  auto lds_barrier = [&]() {
-    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): this wavefront's LDS writes are done; global loads stay in flight
-    __builtin_amdgcn_s_barrier();
+  auto pin = [] { __builtin_amdgcn_sched_barrier(0); };
+  auto round = [&](int set, int rbuf, int rks, int lstage, int lkt, int j) {
+    const int o = set ^ 1;
+    fw[o][0] = read_w(rbuf, 0, rks); mfma(set, 0, 0); pin();
+    fx[o][0] = read_x(rbuf, 0, rks); mfma(set, 0, 1); pin();
+    fw[o][1] = read_w(rbuf, 1, rks); mfma(set, 1, 0); pin();
+    fx[o][1] = read_x(rbuf, 1, rks); mfma(set, 1, 1); pin();
+    request_x(lstage, lkt, j); pin();
+    fx[o][2] = read_x(rbuf, 2, rks); mfma(set, 2, 0); pin();
+    fx[o][3] = read_x(rbuf, 3, rks); mfma(set, 2, 1); pin();
+    mfma(set, 3, 0); pin();
+    mfma(set, 3, 1); pin();
+    request_w(lstage, lkt, j); pin();
   };
 
-  // Main loop, software-pipelined so that no LDS latency is left in the open: step kt multiplies from stage kt%2;
-  //   rounds 0, 1   MFMAs, reading the next round's fragments
-  //   round 2       the same, and the operands of step kt+1 go from their staging registers into the other stage
-  //   barrier       (every wavefront's LDS operations are complete before it arrives: nobody still reads what the next
-  //                  step's round 2 will overwrite, everybody's writes are in place)
-  //   round 3       MFMAs, reading round 0 of step kt+1 from the other stage, and requesting the operands of step kt+2
-  //                 (past the end: the last step's again, unused) a whole step ahead of their trip into LDS
-  const int nk = K / BK;
-  auto clamp_k = [&](int kt) { return (kt < nk ? kt : nk - 1) * BK; };
-  load_stage(0);
+  // Main loop: step kt multiplies 32 k from stage kt%4 (four steps per trip, so that every LDS address is a constant).
+  //   round 0   MFMAs; reads round 1's fragments; second half of the requests for step kt+3
+  //   barrier   every wavefront waits for its own requests for step kt+1 (the eight newer ones stay in flight) and for
+  //             its LDS reads, then for the others: stage (kt+1)%4 is complete, nobody reads stage kt%4 any more
+  //   round 1   MFMAs; reads round 0 of step kt+1; first half of the requests for step kt+4, into stage kt%4
+  auto step = [&](int st, int kt) {
+    round(0, st, 1, (st + 3) & 3, kt + 3, 1);
+    __builtin_amdgcn_s_waitcnt(0x0078);   // vmcnt(8) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    pin();
+    round(1, (st + 1) & 3, 0, st, kt + 4, 0);
+  };
+  request_x(0, 0, 0); request_w(0, 0, 0); request_x(0, 0, 1); request_w(0, 0, 1);
+  request_x(1, 1, 0); request_w(1, 1, 0); request_x(1, 1, 1); request_w(1, 1, 1);
+  request_x(2, 2, 0); request_w(2, 2, 0); request_x(2, 2, 1); request_w(2, 2, 1);
+  request_x(3, 3, 0); request_w(3, 3, 0);
+  __builtin_amdgcn_s_waitcnt(0x007A);   // vmcnt(10) lgkmcnt(0): the requests for step 0 have landed
+  __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int j = 0; j < 4; j++) store_quarter(0, j);
-  load_stage(clamp_k(1));
-  lds_barrier();
-  read_frags(0, 0, 0);
-  for (int kt = 0; kt < nk; kt++) {
-    const int buf = kt & 1;
-    read_frags(1, buf, 1);
-    mfma_round(0);
-    interleave(I1{}, I0{}, I0{});
-    read_frags(0, buf, 2);
-    mfma_round(1);
-    interleave(I1{}, I0{}, I0{});
-    read_frags(1, buf, 3);
+  for (int bn = 0; bn < 2; bn++) fw[0][bn] = read_w(0, bn, 0);
 #pragma unroll
-    for (int j = 0; j < 4; j++) store_quarter(buf ^ 1, j);
-    mfma_round(0);
-    interleave(I1{}, I1{}, I0{});
-    lds_barrier();
-    load_stage(clamp_k(kt + 2));
-    read_frags(0, buf ^ 1, 0);
-    mfma_round(1);
-    interleave(I1{}, I0{}, I1{});
+  for (int bm = 0; bm < 4; bm++) fx[0][bm] = read_x(0, bm, 0);
+  int kt = 0;
+  for (; kt + 4 <= nk; kt += 4) {
+    step(0, kt);
+    step(1, kt + 1);
+    step(2, kt + 2);
+    step(3, kt + 3);
   }
-  lds_barrier();   // the last round's reads of LDS are done everywhere before the stages become C pieces
+  if (kt < nk) {   // K is a multiple of 64: two steps are left
+    step(0, kt);
+    step(1, kt + 1);
+  }
+  auto dma_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) and lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+  };
+  dma_barrier();   // the last round's reads of LDS and the last (unused) loads into it are done everywhere before the stages become C pieces
   // every wavefront is past the last step's barrier and done with the operand stages: LDS becomes eight private C pieces
   constexpr int kCS = 64 + 4;   // floats per row of a piece: 32 rows x 64 columns at a time
   float* const cw = reinterpret_cast<float*>(lds_big) + wave * (32 * kCS);
