@@ -329,25 +329,28 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
 
 // ---- the plain product on large tiles ------------------------------------------------------------------------------------
 // C[M x N] (fp32) = X . W alone is bound by the matrix cores, and a 128 x 128 tile moves too many operand bytes per MFMA
-// to keep them busy.  For whole multiples of 256 rows and columns: a 512-thread workgroup owns a 256(m) x 256(n) tile,
-// its 8 wavefronts as 2(m) x 4(n), each 128 x 64 as eight 32 x 32 blocks (128 accumulator registers); per 16-k round a
-// wavefront reads four X and two W fragments from LDS for eight MFMAs.  One workgroup per CU.
+// to keep them busy.  For whole multiples of 256 rows and columns: a 256-thread workgroup owns a 256(m) x 256(n) tile,
+// ONE wavefront per SIMD, each 128 x 128 as sixteen 32 x 32 blocks (256 accumulator registers, which the compiler keeps
+// in the accumulation half of the register file); per 16-k round a wavefront reads four X and four W fragments from
+// LDS for sixteen MFMAs.  (Two wavefronts per SIMD of 128 x 64 each do not share the matrix core evenly: the older one
+// is served first and then waits at every barrier for the younger one, which runs the rest alone at three quarters of
+// the rate.)  One workgroup per CU.
 // The operands travel global memory -> LDS directly (no staging registers, no LDS store instructions) into a ring of
 // four stages of 32 k (X: 256 rows of 64 bytes, chunks swizzled by (row/4)%4; W as it lies in memory, 32 rows of 512
 // bytes, chunks swizzled by 4*(k%4), read back through ds_read_b64_tr_b16).  A wavefront requests one KiB every fourth
-// MFMA, all the time: the CU's address path takes 16 cycles per request, and eight wavefronts asking for a whole step
-// at once stand in its queue instead of issuing MFMAs.  A request is waited for three steps after it was made.
+// MFMA, all the time: wavefronts asking for a whole step at once stand in the queue of the CU's address path instead
+// of issuing MFMAs.  A request is waited for three steps after it was made.
 // Workgroups are numbered so that the 32 an XCD runs at a time form a block of 4 x 8 tiles: their X and W panels are
-// shared inside that XCD's L2.  The accumulators leave through wavefront-private pieces of LDS as whole 256-byte rows.
+// shared inside that XCD's L2.  The accumulators leave through wavefront-private pieces of LDS as whole 512-byte rows.
 constexpr int TM = 256, TN = 256;
-constexpr int kBigBlock = 512;
+constexpr int kBigBlock = 256;
 constexpr int kBigK = 32;                            // k per stage
 constexpr int kBigStage = (TM + TN) * kBigK * 2;     // one step of X and W: 32 KiB
 constexpr int kBigStages = 4;
 constexpr int kBigLds = kBigStages * kBigStage;
 
 template <bool F16>
-__global__ __launch_bounds__(kBigBlock) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(kBigBlock) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ C, const int N,
                            const int K, const int tilesM, const int tilesN) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_big[];
@@ -367,12 +370,12 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
   }
   const size_t m0 = (size_t)tm * TM, n0 = (size_t)tn * TN;
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);   // a scalar: it goes into descriptors
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave >> 1, wn = wave & 1;
   const int li = lane & 31, lh = lane >> 5;
 
   // A direct-to-LDS load fills 1 KiB, lane L its 16 bytes at position L, so the swizzles are applied on the global side:
-  // lane L fetches the chunk that belongs at L.  Per stage wavefront w brings the X rows 16*(w + 8j).. (16 rows of 64
-  // bytes) and the W rows 2*(w + 8j).. (2 rows of 512 bytes), j = 0, 1.  X: position (row, slot) holds memory chunk
+  // lane L fetches the chunk that belongs at L.  Per stage wavefront w brings the X rows 16*(w + 4j).. (16 rows of 64
+  // bytes) and the W rows 2*(w + 4j).. (2 rows of 512 bytes), j = 0..3.  X: position (row, slot) holds memory chunk
   // slot ^ (row/4)%4; W: position (k, slot) holds chunk slot ^ 4*(k%4).
   const uint32_t xvoff = (uint32_t)(((lane >> 2) * K + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
   const uint32_t wvoff = (uint32_t)(((lane >> 5) * N + 8 * ((lane & 31) ^ (4 * (2 * (wave & 1) + (lane >> 5))))) * 2);
@@ -390,25 +393,25 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
   typedef __attribute__((address_space(3))) void* lds_void_ptr;
   const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((lds_void_ptr)lds_big) + (uint32_t)wave * 1024u;
   const int nk = K / kBigK;
-  // half j (0, 1) of the X / W operands of step `kt` (past the end: the last step's again, unused), into stage `stage`
-  const uint32_t xs0 = (uint32_t)(16 * wave * K * 2), xs1 = (uint32_t)((16 * wave + 128) * K * 2);
-  const uint32_t ws0 = (uint32_t)(2 * wave * N * 2), ws1 = (uint32_t)((2 * wave + 16) * N * 2);
+  // request j (0..3) of the X / W operands of step `kt` (past the end: the last step's again, unused), into stage `stage`
+  const uint32_t xs0 = (uint32_t)(16 * wave * K * 2), xsj = (uint32_t)(64 * K * 2);
+  const uint32_t ws0 = (uint32_t)(2 * wave * N * 2), wsj = (uint32_t)(8 * N * 2);
   const uint32_t wstep = (uint32_t)(kBigK * N * 2);
   auto request_x = [&](int stage, int kt, int j) {
     const uint32_t kc = (uint32_t)(kt < nk ? kt : nk - 1);
-    load_to_lds(x_rs, lds0 + stage * kBigStage + j * 8192, xvoff, (j ? xs1 : xs0) + kc * (kBigK * 2));
+    load_to_lds(x_rs, lds0 + stage * kBigStage + j * 4096, xvoff, xs0 + j * xsj + kc * (kBigK * 2));
   };
   auto request_w = [&](int stage, int kt, int j) {
     const uint32_t kc = (uint32_t)(kt < nk ? kt : nk - 1);
-    load_to_lds(w_rs, lds0 + stage * kBigStage + TM * kBigK * 2 + j * 8192, wvoff, (j ? ws1 : ws0) + kc * wstep);
+    load_to_lds(w_rs, lds0 + stage * kBigStage + TM * kBigK * 2 + j * 4096, wvoff, ws0 + j * wsj + kc * wstep);
   };
-  // fragment addresses: X rows 128*wm + 32*bm + li, chunk 2*ks + lh; W fragment bn of this wavefront's 64 columns
+  // fragment addresses: X rows 128*wm + 32*bm + li, chunk 2*ks + lh; W fragment bn of this wavefront's 128 columns
   int xaddr[4];
 #pragma unroll
   for (int bm = 0; bm < 4; bm++) xaddr[bm] = (128 * wm + 32 * bm + li) * 64;   // + ((2*ks + lh) ^ swizzle) * 16
   const int xsw = (li >> 2) & 3;   // (row/4) % 4: the rows of a fragment start at a multiple of 32
   const int a16 = lane & 15, g2 = (lane >> 4) & 1;
-  const int waddr = ((lh * 8 + (a16 >> 2)) * 32 + ((8 * wn + 2 * g2 + ((a16 >> 1) & 1)) ^ (4 * (a16 >> 2)))) * 16 + 8 * (a16 & 1);
+  const int waddr = ((lh * 8 + (a16 >> 2)) * 32 + ((16 * wn + 2 * g2 + ((a16 >> 1) & 1)) ^ (4 * (a16 >> 2)))) * 16 + 8 * (a16 & 1);
   auto read_x = [&](int buf, int bm, int ks) {
     return *reinterpret_cast<const s16x8*>(lds_big + buf * kBigStage + xaddr[bm] + (((2 * ks + lh) ^ xsw) << 4));
   };
@@ -419,19 +422,19 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
-  f32x16 acc[2][4];   // [bn][bm]: register 4*i4+e is C[128*wm + 32*bm + li][64*wn + 32*bn + 8*i4 + 4*lh + e]
+  f32x16 acc[4][4];   // [bn][bm]: register 4*i4+e is C[128*wm + 32*bm + li][128*wn + 32*bn + 8*i4 + 4*lh + e]
 #pragma unroll
-  for (int a = 0; a < 2; a++)
+  for (int a = 0; a < 4; a++)
 #pragma unroll
     for (int b = 0; b < 4; b++)
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
 
-  // A round of 16 k: two W and four X fragments for eight MFMAs, in two alternating fragment sets.  A round multiplies
-  // from set `set` while the six fragments of the NEXT round are read into the other set from (stage rbuf, round rks)
-  // in the order the next round's MFMAs need them, one LDS instruction per MFMA; after the fourth and the eighth MFMA the
-  // round makes request `j` for step `lkt`.  Every piece is pinned in place: the order IS the schedule.
-  s16x8 fw[2][2], fx[2][4];
+  // A round of 16 k: four W and four X fragments for sixteen MFMAs, in two alternating fragment sets.  A round multiplies
+  // from set `set` while the eight fragments of the NEXT round are read into the other set from (stage rbuf, round rks)
+  // in the order the next round's MFMAs need them; after every fourth MFMA the round makes one request for step `lkt`
+  // (requests 2*half.. of X, then of W).  Every piece is pinned in place: the order IS the schedule.
+  s16x8 fw[2][4], fx[2][4];
   auto mfma = [&](int set, int bm, int bn) {
     if constexpr (F16)
       acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fw[set][bn]), __builtin_bit_cast(f16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
@@ -439,40 +442,52 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
       acc[bn][bm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fw[set][bn]), __builtin_bit_cast(bf16x8, fx[set][bm]), acc[bn][bm], 0, 0, 0);
   };
   auto pin = [] { __builtin_amdgcn_sched_barrier(0); };
-  auto round = [&](int set, int rbuf, int rks, int lstage, int lkt, int j) {
+  auto round = [&](int set, int rbuf, int rks, int lstage, int lkt, int half) {
     const int o = set ^ 1;
     fw[o][0] = read_w(rbuf, 0, rks); mfma(set, 0, 0); pin();
     fx[o][0] = read_x(rbuf, 0, rks); mfma(set, 0, 1); pin();
-    fw[o][1] = read_w(rbuf, 1, rks); mfma(set, 1, 0); pin();
-    fx[o][1] = read_x(rbuf, 1, rks); mfma(set, 1, 1); pin();
-    request_x(lstage, lkt, j); pin();
+    fw[o][1] = read_w(rbuf, 1, rks); mfma(set, 0, 2); pin();
+    mfma(set, 0, 3); pin();
+    request_x(lstage, lkt, 2 * half); pin();
+    fw[o][2] = read_w(rbuf, 2, rks); mfma(set, 1, 0); pin();
+    fw[o][3] = read_w(rbuf, 3, rks); mfma(set, 1, 1); pin();
+    fx[o][1] = read_x(rbuf, 1, rks); mfma(set, 1, 2); pin();
+    mfma(set, 1, 3); pin();
+    request_x(lstage, lkt, 2 * half + 1); pin();
     fx[o][2] = read_x(rbuf, 2, rks); mfma(set, 2, 0); pin();
-    fx[o][3] = read_x(rbuf, 3, rks); mfma(set, 2, 1); pin();
-    mfma(set, 3, 0); pin();
+    mfma(set, 2, 1); pin();
+    mfma(set, 2, 2); pin();
+    mfma(set, 2, 3); pin();
+    request_w(lstage, lkt, 2 * half); pin();
+    fx[o][3] = read_x(rbuf, 3, rks); mfma(set, 3, 0); pin();
     mfma(set, 3, 1); pin();
-    request_w(lstage, lkt, j); pin();
+    mfma(set, 3, 2); pin();
+    mfma(set, 3, 3); pin();
+    request_w(lstage, lkt, 2 * half + 1); pin();
   };
 
   // Main loop: step kt multiplies 32 k from stage kt%4 (four steps per trip, so that every LDS address is a constant).
   //   round 0   MFMAs; reads round 1's fragments; second half of the requests for step kt+3
-  //   barrier   every wavefront waits for its own requests for step kt+1 (the eight newer ones stay in flight) and for
-  //             its LDS reads, then for the others: stage (kt+1)%4 is complete, nobody reads stage kt%4 any more
+  //   barrier   every wavefront waits for its own requests for step kt+1 (the sixteen newer ones stay in flight) and
+  //             for its LDS reads, then for the others: stage (kt+1)%4 is complete, nobody reads stage kt%4 any more
   //   round 1   MFMAs; reads round 0 of step kt+1; first half of the requests for step kt+4, into stage kt%4
   auto step = [&](int st, int kt) {
     round(0, st, 1, (st + 3) & 3, kt + 3, 1);
-    __builtin_amdgcn_s_waitcnt(0x0078);   // vmcnt(8) lgkmcnt(0)
+    __builtin_amdgcn_s_waitcnt(0x4070);   // vmcnt(16) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     pin();
     round(1, (st + 1) & 3, 0, st, kt + 4, 0);
   };
-  request_x(0, 0, 0); request_w(0, 0, 0); request_x(0, 0, 1); request_w(0, 0, 1);
-  request_x(1, 1, 0); request_w(1, 1, 0); request_x(1, 1, 1); request_w(1, 1, 1);
-  request_x(2, 2, 0); request_w(2, 2, 0); request_x(2, 2, 1); request_w(2, 2, 1);
-  request_x(3, 3, 0); request_w(3, 3, 0);
-  __builtin_amdgcn_s_waitcnt(0x007A);   // vmcnt(10) lgkmcnt(0): the requests for step 0 have landed
+#pragma unroll
+  for (int st = 0; st < 3; st++) {
+    request_x(st, st, 0); request_x(st, st, 1); request_w(st, st, 0); request_w(st, st, 1);
+    request_x(st, st, 2); request_x(st, st, 3); request_w(st, st, 2); request_w(st, st, 3);
+  }
+  request_x(3, 3, 0); request_x(3, 3, 1); request_w(3, 3, 0); request_w(3, 3, 1);
+  __builtin_amdgcn_s_waitcnt(0x4074);   // vmcnt(20) lgkmcnt(0): the requests for step 0 have landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int bn = 0; bn < 2; bn++) fw[0][bn] = read_w(0, bn, 0);
+  for (int bn = 0; bn < 4; bn++) fw[0][bn] = read_w(0, bn, 0);
 #pragma unroll
   for (int bm = 0; bm < 4; bm++) fx[0][bm] = read_x(0, bm, 0);
   int kt = 0;
@@ -486,20 +501,16 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
     step(0, kt);
     step(1, kt + 1);
   }
-  auto dma_barrier = [&]() {
-    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) and lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-  };
-  dma_barrier();   // the last round's reads of LDS and the last (unused) loads into it are done everywhere before the stages become C pieces
-  // every wavefront is past the last step's barrier and done with the operand stages: LDS becomes eight private C pieces
-  constexpr int kCS = 64 + 4;   // floats per row of a piece: 32 rows x 64 columns at a time
+  __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): the last reads of LDS and the last (unused) loads into it are done
+  __builtin_amdgcn_s_barrier();         // ... everywhere, before the stages become C pieces
+  constexpr int kCS = 128 + 4;   // floats per row of a piece: 32 rows x 128 columns at a time
   float* const cw = reinterpret_cast<float*>(lds_big) + wave * (32 * kCS);
-  const int r4 = lane >> 4, c16 = lane & 15;
-  const rsrc_t c_rs = buffer_at(C + (m0 + 128 * wm) * (size_t)N + n0 + 64 * wn);
+  const int r2 = lane >> 5, c32 = lane & 31;
+  const rsrc_t c_rs = buffer_at(C + (m0 + 128 * wm) * (size_t)N + n0 + 128 * wn);
 #pragma unroll
   for (int bm = 0; bm < 4; bm++) {
 #pragma unroll
-    for (int bn = 0; bn < 2; bn++)
+    for (int bn = 0; bn < 4; bn++)
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         f32x4 v;
@@ -511,9 +522,9 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
       }
     __builtin_amdgcn_wave_barrier();   // a wavefront's LDS operations complete in order
 #pragma unroll
-    for (int jj = 0; jj < 8; jj++) {
-      const f32x4 v = *reinterpret_cast<const f32x4*>(cw + (4 * jj + r4) * kCS + 4 * c16);
-      const uint32_t off = (uint32_t)(((32 * bm + 4 * jj + r4) * N + 4 * c16) * 4);
+    for (int jj = 0; jj < 16; jj++) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(cw + (2 * jj + r2) * kCS + 4 * c32);
+      const uint32_t off = (uint32_t)(((32 * bm + 2 * jj + r2) * N + 4 * c32) * 4);
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), c_rs, off, 0, 0);
     }
     __builtin_amdgcn_wave_barrier();
