@@ -389,21 +389,22 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
   auto load_to_lds = [](u32x4 rs, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rs), "s"(soff) : "memory");
   };
-  const u32x4 x_rs = words(X + m0 * (size_t)K), w_rs = words(W + n0);
+  const u32x4 x_rs = words(X + m0 * (size_t)K);
+  const uint16_t* const wbase = W + n0;
   typedef __attribute__((address_space(3))) void* lds_void_ptr;
   const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((lds_void_ptr)lds_big) + (uint32_t)wave * 1024u;
   const int nk = K / kBigK;
   // request j (0..3) of the X / W operands of step `kt` (past the end: the last step's again, unused), into stage `stage`
   const uint32_t xs0 = (uint32_t)(16 * wave * K * 2), xsj = (uint32_t)(64 * K * 2);
   const uint32_t ws0 = (uint32_t)(2 * wave * N * 2), wsj = (uint32_t)(8 * N * 2);
-  const uint32_t wstep = (uint32_t)(kBigK * N * 2);
   auto request_x = [&](int stage, int kt, int j) {
     const uint32_t kc = (uint32_t)(kt < nk ? kt : nk - 1);
     load_to_lds(x_rs, lds0 + stage * kBigStage + j * 4096, xvoff, xs0 + j * xsj + kc * (kBigK * 2));
   };
   auto request_w = [&](int stage, int kt, int j) {
     const uint32_t kc = (uint32_t)(kt < nk ? kt : nk - 1);
-    load_to_lds(w_rs, lds0 + stage * kBigStage + TM * kBigK * 2 + j * 4096, wvoff, ws0 + j * wsj + kc * wstep);
+    // the step goes into the descriptor's 64-bit base: W may be larger than the 2 GiB a descriptor spans
+    load_to_lds(words(wbase + (size_t)kc * kBigK * N), lds0 + stage * kBigStage + TM * kBigK * 2 + j * 4096, wvoff, ws0 + j * wsj);
   };
   // fragment addresses: X rows 128*wm + 32*bm + li, chunk 2*ks + lh; W fragment bn of this wavefront's 128 columns
   int xaddr[4];

@@ -575,3 +575,21 @@ def test_plain_product_config5_shape(ccn):
     want = float((X.double().sum(dim=0) * W.double().sum(dim=1)).sum())
     mag = float((X.double().abs().sum(dim=0) * W.double().abs().sum(dim=1)).sum())
     assert abs(total - want) <= K * 2.0 ** -24 * mag
+
+
+def test_plain_product_with_w_beyond_2_gib(ccn):
+    """W of 1088 x 2^20 16-bit elements is 2.1 GiB, more than one buffer descriptor spans: the large-tile kernel moves the
+    descriptor's base with every K-step.  A one-hot X picks rows of an integer W, so every element of C is known exactly
+    without a product on the host; the picked k are spread over the first and the last steps."""
+    M, N, K = 256, 1 << 20, 1088
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(77)
+    W = torch.randint(-64, 64, (K, N), device=DEV, generator=gen, dtype=torch.int16).to(torch.bfloat16)
+    sel = torch.cat([torch.arange(0, 64), torch.arange(K - 64, K), torch.randint(0, K, (M - 128,), generator=torch.Generator().manual_seed(3))]).to(DEV)
+    X = torch.zeros(M, K, device=DEV, dtype=torch.bfloat16)
+    X[torch.arange(M, device=DEV), sel] = 1.0
+    Cd = torch.full((M, N), -7.0, device=DEV)
+    ccn.matmul_bf16_f32(X, W, Cd, M, N, K)
+    torch.cuda.synchronize()
+    for m0 in range(0, M, 64):   # in pieces: the comparison's temporaries stay small
+        assert torch.equal(Cd[m0:m0 + 64], W[sel[m0:m0 + 64]].float())
