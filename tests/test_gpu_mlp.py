@@ -524,13 +524,15 @@ def test_plain_product(ccn):
     assert e.value.code == ccn.CCN_ERANGE
 
 
-@pytest.mark.parametrize("M,N,K,half", [(256, 256, 64, False), (512, 768, 192, False), (1024, 2048, 128, False), (256, 512, 1024, True),
-                                        (2048, 256, 64, False), (768, 1280, 320, False)])
+@pytest.mark.parametrize("M,N,K,half", [(2048, 4096, 64, False), (4096, 2304, 192, False), (2560, 3328, 320, False), (2048, 4096, 1024, True),
+                                        (8192, 1024, 128, False), (4096, 8192, 64, True), (256, 256, 64, False), (768, 1280, 320, False)])
 def test_plain_product_on_large_tiles(ccn, M, N, K, half):
-    """Whole multiples of 256 rows and columns take the 256 x 256-tile kernel of the plain product: exact on small integers
-    (a one-hot X picks rows of an integer W: any transposed, swizzled or mis-dealt index shows as a wrong integer; all-ones
+    """Whole multiples of 256 rows and columns, at least 128 tiles of 256 x 256 (half of the CUs), take the large-tile kernel
+    of the plain product; the last two shapes are fewer tiles and stay on 128 x 128 tiles.  Exact on small integers (a
+    one-hot X picks rows of an integer W: any transposed, swizzled or mis-dealt index shows as a wrong integer; all-ones
     gives K, the reference's own check at this boundary), within the fp32-accumulation bound of float64 on random operands.
-    Tile counts that do and do not divide into the blocks of 4 x 8 tiles the workgroups are dealt in."""
+    Tile counts that do and do not divide into the blocks of 4 x 8 tiles the workgroups are dealt in; K of 2, 4, 6, 10 and
+    32 ring steps (whole trips of four and the two left over)."""
     r = rng(300 + M // 256 + N // 256)
     to16 = (lambda a: a.astype(np.float16).view(np.uint16)) if half else (lambda a: orc.f32_to_bf16(a.astype(np.float32)))
     wide = (lambda b: b.view(np.float16).astype(np.float64)) if half else (lambda b: orc.bf16_to_f32(b).astype(np.float64))
