@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="adam_f32",
                     choices=["adam_f32", "adam_f32_scattered", "sgd_f32", "adam_f16g", "adam_bf16g", "lamb_f32",
-                             "lamb_nccl_f16g", "mlp_outproj", "matmul_bf16", "copy", "copy_stream"])
+                             "lamb_nccl_f16g", "mlp_outproj", "matmul_bf16", "matmul_bf16_c16", "copy", "copy_stream"])
     ap.add_argument("--log2n", type=int, default=None, help="override log2 of the parameter count")
     ap.add_argument("--ranks", type=int, default=None, help="override P")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -108,7 +108,7 @@ def cpu_baseline(wl, P, budget_s=8.0):
     threads = max(1, min(16, os.cpu_count() or 1))     # a one-GPU box gives a job 16 host threads
     r = np.random.Generator(np.random.Philox(key=[5, 0]))
     f32 = np.float32
-    if wl in ("mlp_outproj", "matmul_bf16"):
+    if wl in ("mlp_outproj", "matmul_bf16", "matmul_bf16_c16"):
         # a band of rows of the 8192 x 1024 x 8192 product with its 7 partial buffers
         rows, Nn, Kd, nP = 8 * threads, 8192, 1024, (7 if wl == "mlp_outproj" else 0)
         X = orc.f32_to_bf16(r.standard_normal((rows, Kd), dtype=f32))
@@ -288,19 +288,22 @@ def build_workload(a, wl, capi, torch, stream, allocator):
         kernel = "mlp_outproj_kernel<7>"
         config = {"workload": "mlp_outproj bf16 8192x1024x8192 + 7 fp32 partials + bias + dropout(0.1) + residual",
                   "M": M, "N": Nn, "K": Kd}
-    elif wl == "matmul_bf16":
-        # the MatMul step of the unfused schedules alone (the reference: cublasGemmEx, src/codegen.cpp:1058-1136)
+    elif wl in ("matmul_bf16", "matmul_bf16_c16"):
+        # the MatMul step of the unfused schedules alone (the reference: cublasGemmEx, src/codegen.cpp:1058-1136), with C in
+        # fp32 (what the unfused lowering here keeps) or in the operands' 16-bit type (what the reference's call writes)
         M = Nn = 8192
         Kd = 1024
+        c16 = wl == "matmul_bf16_c16"
         X = torch.randn(M, Kd, device="cuda", generator=gen).to(torch.bfloat16)
         Wm = (torch.randn(Kd, Nn, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
-        Cm = torch.empty(M, Nn, device="cuda")
-        step = lambda t: capi.matmul_bf16_f32(X, Wm, Cm, M, Nn, Kd, stream)
-        alg_bytes = float(M * Kd * 2 + Kd * Nn * 2 + M * Nn * 4)
+        Cm = torch.empty(M, Nn, device="cuda", dtype=torch.bfloat16 if c16 else torch.float32)
+        step = (lambda t: capi.matmul_16(X, Wm, Cm, M, Nn, Kd, stream)) if c16 else (lambda t: capi.matmul_bf16_f32(X, Wm, Cm, M, Nn, Kd, stream))
+        alg_bytes = float(M * Kd * 2 + Kd * Nn * 2 + M * Nn * (2 if c16 else 4))
         flops = 2.0 * M * Nn * Kd
         units = M * Nn
-        kernel = "mlp_outproj_kernel<0, true>"
-        config = {"workload": "matmul bf16 8192x1024x8192 -> fp32 (the unfused schedule's MatMul step)", "M": M, "N": Nn, "K": Kd}
+        kernel = "matmul_tile256_kernel<false, true>" if c16 else "matmul_tile256_kernel<false, false>"
+        config = {"workload": f"matmul bf16 8192x1024x8192 -> {'bf16' if c16 else 'fp32'} (the unfused schedule's MatMul step)",
+                  "M": M, "N": Nn, "K": Kd}
     elif wl == "copy_stream":
         # a 1R:1W stream through the library's own streaming kernel (ccn_reduce_f32 over one rank buffer is a copy): the
         # ceiling of this box for the launch shape the fused kernels use
@@ -379,7 +382,7 @@ def other_workloads(a, capi, torch, stream):
     except (ValueError, KeyError, IndexError):
         rows.append({"workload": "adam_f32 on plain allocations", "error": (child.stderr or child.stdout)[-300:]})
     for wl, allocator in (("adam_f32", "torch"), ("sgd_f32", "ccn"), ("sgd_f32_graph", "ccn"), ("sgd_f32_large", "ccn"),
-                          ("adam_f16g", "ccn"), ("lamb_f32", "ccn"), ("mlp_outproj", "ccn"), ("matmul_bf16", "ccn"),
+                          ("adam_f16g", "ccn"), ("lamb_f32", "ccn"), ("mlp_outproj", "ccn"), ("matmul_bf16", "ccn"), ("matmul_bf16_c16", "ccn"),
                           ("copy", "torch"), ("copy_stream", "ccn")):
         replay = 64 if wl == "sgd_f32_graph" else 0      # configuration 1 again, 64 recorded steps per graph launch
         own = capi.Stream() if replay else None          # the null stream cannot be recorded
@@ -404,7 +407,7 @@ def other_workloads(a, capi, torch, stream):
                "frac_of_hbm_peak": round(ach / HBM_PEAK_GBPS, 4), "kernel": kernel,
                "algorithmic_bytes_per_launch": alg_bytes,
                "traffic": traffic_from_profiles(f"{'sgd_f32' if wl == 'sgd_f32_large' else wl}.pmc.txt") if allocator == "ccn" else None}
-        if alg_bytes < 1e9 and wl != "matmul_bf16":
+        if alg_bytes < 1e9 and not wl.startswith("matmul_bf16"):
             row["note"] = "fits the caches and is bound by launches: not a roofline figure"
         if wl == "copy":
             row["note"] = "torch's device-to-device copy_ on this box"
@@ -476,7 +479,8 @@ def main():
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"adam_f16g": "f16 gradients, f32 state", "adam_bf16g": "bf16 gradients, f32 state",
                   "lamb_nccl_f16g": "f16 gradients (f16 sum), f32 state",
-                  "mlp_outproj": "bf16 x bf16 -> f32", "matmul_bf16": "bf16 x bf16 -> f32"}.get(wl, "f32"),
+                  "mlp_outproj": "bf16 x bf16 -> f32", "matmul_bf16": "bf16 x bf16 -> f32",
+                  "matmul_bf16_c16": "bf16 x bf16 -> f32 -> bf16"}.get(wl, "f32"),
         "data": "synthetic", "config": config,
         "params_per_s": round(units / (wall_ms * 1e-3), 1),
         "device": info,
@@ -489,7 +493,7 @@ def main():
     if flops:
         line["mfma"] = {"achieved": round(flops / (ev_ms * 1e-3) / 1e12, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                         "unit": "TFLOP/s", "frac": round(flops / (ev_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
-    if wl == "matmul_bf16":     # the one compute-bound kernel of the path: its roofline is the matrix cores'
+    if wl.startswith("matmul_bf16"):     # the one compute-bound kernel of the path: its roofline is the matrix cores'
         line["roofline"].update({"bound": "mfma", "achieved": line["mfma"]["achieved"], "peak": MFMA_BF16_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": line["mfma"]["frac"], "algorithmic_flops_per_launch": flops})
     default_run = (wl == "adam_f32" and a.allocator == "ccn" and a.graph_steps == 0 and a.log2n is None and a.ranks is None)
@@ -498,7 +502,7 @@ def main():
         release(keep, capi, torch)
         line["other_workloads"] = other_workloads(a, capi, torch, stream)
     if wl not in ("copy", "copy_stream") and not a.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(wl, P if wl not in ("mlp_outproj", "matmul_bf16") else 8)
+        line["cpu_baseline"] = cpu_baseline(wl, P if wl not in ("mlp_outproj", "matmul_bf16", "matmul_bf16_c16") else 8)
     print(json.dumps(line), flush=True)
 
 

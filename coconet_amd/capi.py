@@ -36,6 +36,7 @@ SYMBOLS = [
     "ccn_lamb_f32_scattered", "ccn_adam_bf16g", "ccn_lamb_nccl_f16g", "ccn_lamb_f32_static",
     "ccn_mlp_outproj_bf16_ex", "ccn_bias_dropout_residual_ex", "ccn_matmul_bf16_f32",
     "ccn_mlp_outproj_f16_ex", "ccn_bias_dropout_residual_f16_ex", "ccn_matmul_f16_f32",
+    "ccn_matmul_bf16", "ccn_matmul_f16",
 ]
 
 
@@ -115,6 +116,8 @@ def _declare(L):
     sig("ccn_mlp_outproj_f16_ex", [_vp, _vp, _pp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _u64, _i, _vp])
     sig("ccn_bias_dropout_residual_f16_ex", [_vp, _pp, _i, _vp, _vp, _vp, _i, _i, _f, _u64, _i, _sz, _vp])
     sig("ccn_matmul_f16_f32", [_vp, _vp, _vp, _i, _i, _i, _vp])
+    sig("ccn_matmul_bf16", [_vp, _vp, _vp, _i, _i, _i, _vp])
+    sig("ccn_matmul_f16", [_vp, _vp, _vp, _i, _i, _i, _vp])
     sig("ccn_scatter_plan_create", [C.POINTER(_sz), _i, _pp])
     sig("ccn_scatter_plan_destroy", [_vp])
     sig("ccn_sgd_f32_scattered", [_vp, _pp, _i, _pp, _f, _vp])
@@ -475,3 +478,11 @@ def matmul_bf16_f32(X, W, Cmat, M, N, K, stream=None, half=False):
         _check(load().ccn_matmul_f16_f32(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_f16_f32")
     else:
         _check(load().ccn_matmul_bf16_f32(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_bf16_f32")
+
+
+def matmul_16(X, W, Cmat, M, N, K, stream=None, half=False):
+    """The product alone with C in the operands' 16-bit type (ccn_matmul_bf16 / ccn_matmul_f16)."""
+    if half:
+        _check(load().ccn_matmul_f16(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_f16")
+    else:
+        _check(load().ccn_matmul_bf16(addr(X), addr(W), addr(Cmat), M, N, K, stream), "ccn_matmul_bf16")

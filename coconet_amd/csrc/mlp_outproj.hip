@@ -39,6 +39,10 @@ struct EpiPrm {
 // model-parallel example declares); accumulation is fp32 either way.
 template <bool F16> __device__ __forceinline__ float half_in(uint16_t h) { return F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h); }
 template <bool F16> __device__ __forceinline__ uint16_t half_out(float f) { return F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f); }
+template <bool F16> __device__ __forceinline__ u32x2 pack_quad(f32x4 v) {
+  return u32x2{(uint32_t)half_out<F16>(v[0]) | ((uint32_t)half_out<F16>(v[1]) << 16),
+               (uint32_t)half_out<F16>(v[2]) | ((uint32_t)half_out<F16>(v[3]) << 16)};
+}
 
 // Epilogue for four consecutive columns n..n+3 (n % 4 == 0) of row m, in two steps so that the loads of one quad can be
 // in flight while the previous one is finished.  NP, the number of partial buffers (0..8), is a compile-time constant:
@@ -139,14 +143,15 @@ constexpr int kMaxRowLen = 1 << 21;
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 7); }
 
-// PLAIN: the product alone, written as fp32 [M x N] through `out` (no partial buffers, bias, dropout or residual).
+// PLAIN: the product alone through `out` (no partial buffers, bias, dropout or residual): 1 writes fp32 [M x N], 2 rounds
+// to the operands' 16-bit type (round to nearest even).
 // REF: the epilogue applies one of the reference's dropout forms.
 // The rows are dealt to the wavefronts (see the top of the file) so that the epilogue needs no workgroup barrier: after
 // the main loop a wavefront turns its own accumulators into rows through a private piece of LDS (16 rows at a time) and
 // walks its 16 row pairs.  At step j the four wavefronts of the workgroup together touch 8 adjacent rows x 512 bytes of
 // every partial buffer; the operands of step j+1 are requested before step j is finished, step 0's under the last MFMA
 // step.  Three workgroups share a CU (168 registers, 33 KiB of LDS).
-template <int NP, bool PLAIN = false, bool REF = false, bool F16 = false>
+template <int NP, int PLAIN = 0, bool REF = false, bool F16 = false>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, const SrcTable<float, 8> parts,
                         const float* __restrict__ bias, const uint16_t* __restrict__ resid, uint16_t* __restrict__ out,
@@ -257,7 +262,7 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
 #pragma unroll
   for (int q = 0; q < (PLAIN ? 0 : NP); q++) p_rs[q] = buffer_at(parts.p[q] + tile0);
   const rsrc_t r_rs = buffer_at(resid ? resid + tile0 : nullptr);
-  const rsrc_t o_rs = buffer_at(PLAIN ? static_cast<void*>(reinterpret_cast<float*>(out) + tile0) : static_cast<void*>(out + tile0));
+  const rsrc_t o_rs = buffer_at(PLAIN == 1 ? static_cast<void*>(reinterpret_cast<float*>(out) + tile0) : static_cast<void*>(out + tile0));
   auto load_step = [&](EpiIn<PLAIN ? 0 : NP>& in, int j) {
 #pragma unroll
     for (int q = 0; q < (PLAIN ? 0 : NP); q++)
@@ -312,8 +317,10 @@ void mlp_outproj_kernel(const uint16_t* __restrict__ X, const uint16_t* __restri
     for (int jj = 0; jj < 8; jj++) {
       const int j = half * 8 + jj;
       const f32x4 v = *reinterpret_cast<const f32x4*>(cw + (2 * jj + lh) * kCStride + sc);
-      if constexpr (PLAIN) {
+      if constexpr (PLAIN == 1) {
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), o_rs, eoff * 4u, (uint32_t)j * estep * 4u, 0);
+      } else if constexpr (PLAIN == 2) {
+        __builtin_amdgcn_raw_buffer_store_b64(pack_quad<F16>(v), o_rs, eoff * 2u, (uint32_t)j * estep * 2u, 0);
       } else {
         const uint32_t ge = draw_quad<REF>(ep, tile0 + (size_t)j * estep + eoff);
         EpiIn<NP> nxt;
@@ -349,9 +356,9 @@ constexpr int kBigStage = (TM + TN) * kBigK * 2;     // one step of X and W: 32 
 constexpr int kBigStages = 4;
 constexpr int kBigLds = kBigStages * kBigStage;
 
-template <bool F16>
+template <bool F16, bool C16>
 __global__ __launch_bounds__(kBigBlock) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, float* __restrict__ C, const int N,
+void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W, void* __restrict__ Cout, const int N,
                            const int K, const int tilesM, const int tilesN) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_big[];
   // tile of this workgroup: blocks of 4 x 8 tiles dealt to the XCDs (workgroup b runs on XCD b % 8) when the grid divides
@@ -506,8 +513,9 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
   __builtin_amdgcn_s_barrier();         // ... everywhere, before the stages become C pieces
   constexpr int kCS = 128 + 4;   // floats per row of a piece: 32 rows x 128 columns at a time
   float* const cw = reinterpret_cast<float*>(lds_big) + wave * (32 * kCS);
-  const int r2 = lane >> 5, c32 = lane & 31;
-  const rsrc_t c_rs = buffer_at(C + (m0 + 128 * wm) * (size_t)N + n0 + 128 * wn);
+  const size_t c0 = (m0 + 128 * wm) * (size_t)N + n0 + 128 * wn;
+  const rsrc_t c_rs = C16 ? buffer_at(static_cast<uint16_t*>(Cout) + c0) : buffer_at(static_cast<float*>(Cout) + c0);
+  const int r2 = lane >> 5, c32 = lane & 31, r4 = lane >> 4, c16 = lane & 15;
 #pragma unroll
   for (int bm = 0; bm < 4; bm++) {
 #pragma unroll
@@ -522,11 +530,21 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
         *reinterpret_cast<f32x4*>(cw + li * kCS + bn * 32 + i4 * 8 + lh * 4) = v;
       }
     __builtin_amdgcn_wave_barrier();   // a wavefront's LDS operations complete in order
+    if constexpr (C16) {   // 8 columns per lane: four rows of 256 bytes per instruction
 #pragma unroll
-    for (int jj = 0; jj < 16; jj++) {
-      const f32x4 v = *reinterpret_cast<const f32x4*>(cw + (2 * jj + r2) * kCS + 4 * c32);
-      const uint32_t off = (uint32_t)(((32 * bm + 2 * jj + r2) * N + 4 * c32) * 4);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), c_rs, off, 0, 0);
+      for (int jj = 0; jj < 8; jj++) {
+        const float* src = cw + (4 * jj + r4) * kCS + 8 * c16;
+        const u32x2 lo = pack_quad<F16>(*reinterpret_cast<const f32x4*>(src)), hi = pack_quad<F16>(*reinterpret_cast<const f32x4*>(src + 4));
+        const uint32_t off = (uint32_t)(((32 * bm + 4 * jj + r4) * N + 8 * c16) * 2);
+        __builtin_amdgcn_raw_buffer_store_b128(u32x4{lo[0], lo[1], hi[0], hi[1]}, c_rs, off, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < 16; jj++) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(cw + (2 * jj + r2) * kCS + 4 * c32);
+        const uint32_t off = (uint32_t)(((32 * bm + 2 * jj + r2) * N + 4 * c32) * 4);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), c_rs, off, 0, 0);
+      }
     }
     __builtin_amdgcn_wave_barrier();
   }
@@ -556,7 +574,7 @@ __global__ __launch_bounds__(BS) void bias_dropout_residual_kernel(const float* 
 // epilogue is the same code.  nP is a run-time count here: the partial sums are added to the product in buffer order
 // before the shared epilogue sees it, which is the order the fixed-count epilogue uses.
 constexpr int GT = 64, GK = 32;
-template <bool PLAIN, bool REF, bool F16 = false>
+template <int PLAIN, bool REF, bool F16 = false>
 __global__ __launch_bounds__(kBlock) void outproj_any_shape_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ W,
                                                                    const SrcTable<float, 8> parts, const int nP,
                                                                    const float* __restrict__ bias,
@@ -616,8 +634,10 @@ __global__ __launch_bounds__(kBlock) void outproj_any_shape_kernel(const uint16_
     if (m >= M) continue;
     const size_t idx = (size_t)m * N + n;
     f32x4 sum = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
-    if constexpr (PLAIN) {
+    if constexpr (PLAIN == 1) {
       *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(out) + idx) = sum;
+    } else if constexpr (PLAIN == 2) {
+      *reinterpret_cast<u32x2*>(out + idx) = pack_quad<F16>(sum);
     } else {
       for (int q = 0; q < nP; q++) sum = sum + __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(parts.p[q] + idx));
       EpiIn<0> in;
@@ -675,10 +695,10 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
     const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
     if (tiles > 0x7fffffffull) return CCN_ERANGE;
     if (mode == CCN_DROPOUT_INVERTED)
-      hipLaunchKernelGGL((outproj_any_shape_kernel<false, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
+      hipLaunchKernelGGL((outproj_any_shape_kernel<0, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
                          bias, resid, out, M, N, K, ep);
     else
-      hipLaunchKernelGGL((outproj_any_shape_kernel<false, true, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
+      hipLaunchKernelGGL((outproj_any_shape_kernel<0, true, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, s, X, W, tbl, nPartials,
                          bias, resid, out, M, N, K, ep);
     CCN_HIP(hipGetLastError());
     return CCN_OK;
@@ -687,8 +707,8 @@ int outproj_launch(const uint16_t* X, const uint16_t* W, const float* const* par
   switch (nPartials) {
 #define CCN_CASE(Q)                                                                                                          \
   case Q:                                                                                                                    \
-    if (mode == CCN_DROPOUT_INVERTED) hipLaunchKernelGGL((mlp_outproj_kernel<Q, false, false, F16>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
-    else hipLaunchKernelGGL((mlp_outproj_kernel<Q, false, true, F16>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
+    if (mode == CCN_DROPOUT_INVERTED) hipLaunchKernelGGL((mlp_outproj_kernel<Q, 0, false, F16>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
+    else hipLaunchKernelGGL((mlp_outproj_kernel<Q, 0, true, F16>), grid, block, 0, s, X, W, tbl, bias, resid, out, N, K, ep); \
     break;
     CCN_CASE(0) CCN_CASE(1) CCN_CASE(2) CCN_CASE(3) CCN_CASE(4) CCN_CASE(5) CCN_CASE(6) CCN_CASE(7) CCN_CASE(8)
 #undef CCN_CASE
@@ -752,23 +772,24 @@ int epilogue_launch(const float* acc, const float* const* partials, int nPartial
   return CCN_OK;
 }
 
-template <bool F16>
-int matmul_launch(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
+template <bool F16, bool C16>
+int matmul_launch(const uint16_t* X, const uint16_t* W, void* C, int M, int N, int K, void* stream) {
   if (!X || !W || !C) return CCN_EINVAL;
   if (M <= 0 || N <= 0 || K <= 0) return CCN_EINVAL;
   if (N % 4) return CCN_ERANGE;
-  if (!aligned16(X) || !aligned16(W) || !aligned16(C)) return CCN_EINVAL;
+  if (!aligned16(X) || !aligned16(W) || !(C16 ? aligned8(C) : aligned16(C))) return CCN_EINVAL;
   const DeviceInfo* di = nullptr;
   const int rc = current_device_info(&di);
   if (rc != CCN_OK) return rc;
   SrcTable<float, 8> tbl;
   for (int q = 0; q < 8; q++) tbl.p[q] = nullptr;
   EpiPrm ep{};
+  constexpr int kPlain = C16 ? 2 : 1;
   if (M % BM || N % BN || K % BK || N > kMaxRowLen || K > kMaxRowLen) {
     const size_t tiles = (size_t)((M + GT - 1) / GT) * (size_t)((N + GT - 1) / GT);
     if (tiles > 0x7fffffffull) return CCN_ERANGE;
-    hipLaunchKernelGGL((outproj_any_shape_kernel<true, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, as_stream(stream), X, W,
-                       tbl, 0, (const float*)nullptr, (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), M, N, K, ep);
+    hipLaunchKernelGGL((outproj_any_shape_kernel<kPlain, false, F16>), dim3((unsigned)tiles), dim3(kBlock), 0, as_stream(stream), X, W,
+                       tbl, 0, (const float*)nullptr, (const uint16_t*)nullptr, static_cast<uint16_t*>(C), M, N, K, ep);
     CCN_HIP(hipGetLastError());
     return CCN_OK;
   }
@@ -777,18 +798,18 @@ int matmul_launch(const uint16_t* X, const uint16_t* W, float* C, int M, int N, 
   // against 21.4 us / 17.6 against 24.9 us; 128: 26.6 against 27.6; 256: 52.0 against 37.8).
   if (M % TM == 0 && N % TN == 0 && (size_t)128 * (size_t)N * 4 < 0x7fffffffull &&
       2 * (size_t)(M / TM) * (size_t)(N / TN) >= (size_t)di->cu_count) {
-    static const hipError_t attr = hipFuncSetAttribute((const void*)matmul_tile256_kernel<F16>,
+    static const hipError_t attr = hipFuncSetAttribute((const void*)matmul_tile256_kernel<F16, C16>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBigLds);
     if (attr != hipSuccess) return hip_fail(attr);
     const int tilesM = M / TM, tilesN = N / TN;
-    hipLaunchKernelGGL((matmul_tile256_kernel<F16>), dim3((unsigned)(tilesM * tilesN)), dim3(kBigBlock), kBigLds, as_stream(stream),
+    hipLaunchKernelGGL((matmul_tile256_kernel<F16, C16>), dim3((unsigned)(tilesM * tilesN)), dim3(kBigBlock), kBigLds, as_stream(stream),
                        X, W, C, N, K, tilesM, tilesN);
     CCN_HIP(hipGetLastError());
     return CCN_OK;
   }
   const dim3 grid((unsigned)((M / BM) * (N / BN))), block(kBlock);
-  hipLaunchKernelGGL((mlp_outproj_kernel<0, true, false, F16>), grid, block, 0, as_stream(stream), X, W, tbl, (const float*)nullptr,
-                     (const uint16_t*)nullptr, reinterpret_cast<uint16_t*>(C), N, K, ep);
+  hipLaunchKernelGGL((mlp_outproj_kernel<0, kPlain, false, F16>), grid, block, 0, as_stream(stream), X, W, tbl, (const float*)nullptr,
+                     (const uint16_t*)nullptr, static_cast<uint16_t*>(C), N, K, ep);
   CCN_HIP(hipGetLastError());
   return CCN_OK;
 }
@@ -822,7 +843,7 @@ int ccn_bias_dropout_residual_ex(const float* acc, const float* const* partials,
 }
 
 int ccn_matmul_bf16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
-  return matmul_launch<false>(X, W, C, M, N, K, stream);
+  return matmul_launch<false, false>(X, W, C, M, N, K, stream);
 }
 
 int ccn_mlp_outproj_f16_ex(const uint16_t* X, const uint16_t* W, const float* const* partials, int nPartials,
@@ -838,7 +859,15 @@ int ccn_bias_dropout_residual_f16_ex(const float* acc, const float* const* parti
 }
 
 int ccn_matmul_f16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream) {
-  return matmul_launch<true>(X, W, C, M, N, K, stream);
+  return matmul_launch<true, false>(X, W, C, M, N, K, stream);
+}
+
+int ccn_matmul_bf16(const uint16_t* X, const uint16_t* W, uint16_t* C, int M, int N, int K, void* stream) {
+  return matmul_launch<false, true>(X, W, C, M, N, K, stream);
+}
+
+int ccn_matmul_f16(const uint16_t* X, const uint16_t* W, uint16_t* C, int M, int N, int K, void* stream) {
+  return matmul_launch<true, true>(X, W, C, M, N, K, stream);
 }
 
 }  // extern "C"

@@ -292,6 +292,14 @@ int  ccn_bias_dropout_residual_f16_ex(const float* acc, const float* const* part
                                       int dropout_mode, size_t first_row, void* stream);
 int  ccn_matmul_f16_f32(const uint16_t* X, const uint16_t* W, float* C, int M, int N, int K, void* stream);
 
+/* ---- the product alone with C in the operands' 16-bit type, as the emitted cublasGemmEx call writes it (its C type is
+ *      the output stage's element type, CUDA_R_16F in the reference's example: src/codegen.cpp:1114-1131,
+ *      examples/model-parallel/model-parallel.cpp:13-18).  Accumulated in fp32 on the matrix cores and rounded to
+ *      nearest even once, where the reference accumulates in half: every element equals the fp32 call's, rounded.
+ *      C 8-byte aligned; shapes as for the fp32 calls. ---- */
+int  ccn_matmul_bf16(const uint16_t* X, const uint16_t* W, uint16_t* C, int M, int N, int K, void* stream);
+int  ccn_matmul_f16(const uint16_t* X, const uint16_t* W, uint16_t* C, int M, int N, int K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -595,3 +595,43 @@ def test_plain_product_with_w_beyond_2_gib(ccn):
     torch.cuda.synchronize()
     for m0 in range(0, M, 64):   # in pieces: the comparison's temporaries stay small
         assert torch.equal(Cd[m0:m0 + 64], W[sel[m0:m0 + 64]].float())
+
+
+@pytest.mark.parametrize("M,N,K,half", [(2048, 4096, 192, False), (2560, 3328, 64, True), (768, 1280, 320, False), (256, 384, 192, True),
+                                        (100, 36, 70, False), (1, 4, 1, True)])
+def test_plain_product_with_16_bit_c(ccn, M, N, K, half):
+    """ccn_matmul_bf16 / ccn_matmul_f16 (C in the operands' type, as the reference's emitted GEMM call writes it) on the
+    large-tile kernel, on 128 x 128 tiles and on the any-shape kernel: a one-hot X picks rows of an integer W exactly;
+    random operands land on the 16-bit neighbour of the float64 product that fp32 accumulation allows (the oracle's
+    round-to-nearest-even conversion of the float64 value, one unit in the last place where the fp32 error straddles a
+    rounding boundary); and every element equals the fp32-C call's, rounded to nearest even."""
+    r = rng(700 + M + N)
+    to16 = (lambda a: a.astype(np.float16).view(np.uint16)) if half else (lambda a: orc.f32_to_bf16(a.astype(np.float32)))
+    wide = (lambda b: b.view(np.float16).astype(np.float64)) if half else (lambda b: orc.bf16_to_f32(b).astype(np.float64))
+    C16 = torch.full((M, N), 0x7e01, dtype=torch.int16, device=DEV)
+    sel = r.integers(0, K, M)
+    Xf = np.zeros((M, K), np.float32)
+    Xf[np.arange(M), sel] = 1.0
+    Wf = r.integers(-64, 64, (K, N)).astype(np.float32)
+    ccn.matmul_16(u16_dev(to16(Xf)), u16_dev(to16(Wf)), C16, M, N, K, half=half)
+    torch.cuda.synchronize()
+    assert np.array_equal(wide(bf16_host(C16).reshape(M, N)), Wf[sel].astype(np.float64))
+    X = to16(r.standard_normal((M, K)))
+    W = to16(r.standard_normal((K, N)) * 0.02)
+    C32 = torch.empty(M, N, device=DEV)
+    ccn.matmul_16(u16_dev(X), u16_dev(W), C16, M, N, K, half=half)
+    ccn.matmul_bf16_f32(u16_dev(X), u16_dev(W), C32, M, N, K, half=half)
+    torch.cuda.synchronize()
+    got = bf16_host(C16).reshape(M, N)
+    c32 = C32.cpu().numpy()
+    rounded = c32.astype(np.float16).view(np.uint16) if half else orc.f32_to_bf16(c32)
+    assert np.array_equal(got, rounded)
+    ref = wide(X) @ wide(W)
+    want = ref.astype(np.float16).view(np.uint16) if half else orc.f32_to_bf16(ref.astype(np.float32))
+    d = f16_ulp_distance(got, want)
+    bound = K * 2.0 ** -24 * (np.abs(wide(X)) @ np.abs(wide(W)))
+    ulp = np.maximum(np.abs(wide(want)) * 2.0 ** (-10 if half else -7), 1e-30)
+    assert np.all((d <= 1) | (np.abs(wide(got) - ref) <= bound + ulp))
+    with pytest.raises(ccn.CoconetError) as e:
+        ccn.matmul_16(u16_dev(X), u16_dev(W), C16, M, N + 2, K, half=half)
+    assert e.value.code == ccn.CCN_ERANGE
