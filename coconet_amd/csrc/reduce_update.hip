@@ -548,9 +548,8 @@ int launch_scattered(ccn_scatter_plan* plan, const float* const* g, int P, float
   float* const* wtab = reinterpret_cast<float* const*>(const_cast<void**>(plan->table_dev) + (size_t)CCN_MAX_RANKS * plan->nbuff);
   // A wavefront here first finds its buffer and reads the buffer's pointers, and only then its data: two short round
   // trips (cache hits) more than the flat kernels.  Measured at P = 8: 8 to 10 wavefronts per CU give 78 % of HBM peak,
-  // 7 give 76 %, 13 give 77 %.  CCN_LDS_KB overrides, as for the flat kernels.
-  static const int f_lds = [] { const char* e = std::getenv("CCN_LDS_KB"); return e ? std::atoi(e) : -1; }();
-  const unsigned lds = f_lds >= 0 && f_lds <= 64 ? (unsigned)f_lds * 1024u : lds_for_residency(8);
+  // 7 give 76 %, 13 give 77 %.
+  const unsigned lds = lds_for_residency(8);
   const size_t gx = plan->ntiles < 0x40000000ull ? plan->ntiles : 0x40000000ull;
   const dim3 grid((unsigned)gx, (unsigned)((plan->ntiles + gx - 1) / gx));
   if (grid.x * (size_t)grid.y != plan->ntiles) return CCN_ERANGE;   // the kernel has no bounds check on the tile index

@@ -73,27 +73,23 @@ unsigned lds_for_residency(int per_cu) {
 }
 
 StreamShape stream_shape(int load_bytes, int store_bytes, int grad_bytes) {
-  // CCN_BLOCK / CCN_LDS_KB override the shape; meant for tuning runs.
-  static const int f_block = [] { const char* e = std::getenv("CCN_BLOCK"); return e ? std::atoi(e) : 0; }();
-  static const int f_lds = [] { const char* e = std::getenv("CCN_LDS_KB"); return e ? std::atoi(e) : -1; }();
   StreamShape sh;
   // Single-wavefront workgroups, and fewer of them per CU the more 16-byte loads each thread has in flight.
   // Measured optima on MI355X at N = 2^28 (2^27 beyond 8 ranks), fp32 Adam unless said otherwise, as
   // loads per thread -> wavefronts per CU (% of HBM peak): 2 -> 26 (SGD at 1 rank: 85.5; 256-thread workgroups at full
   // occupancy 82.5), 3 -> 16-20 (SGD at 2 ranks: 84.6; 13: 79), 4 -> 17 (SGD at 3 ranks: 84.6; 13: 81), 5 -> 11-14 (84),
   // 7 -> 12-13 (83), 9 -> 8 (86; SGD at 8 ranks: 84), 11 -> 7 (85.5; 6 or 8 give 82-83), 15 -> 8 (82), 19 -> 6-10 (79).
-  // Between 5 and 7 the optimum moves by one or two wavefronts with the width of the gradient loads (Adam, % of peak at
-  // 11 / 12 / 13 wavefronts): fp32 gradients 5 -> 84.9 / 83.4 / 82.5, 6 -> 85.1 / 84.8 / 83.7, 7 -> 82.2 / 82.9 / 82.9;
-  // 16-bit gradients (8-byte loads, so more of them per byte) 5 -> 80.1 / 83.0 / 82.0, 6 -> 81.0 / 82.0 / 81.4,
+  // Between 5 and 7 the optimum moves by one or two wavefronts with what else the thread does (% of peak at 11 / 12 /
+  // 13 wavefronts): one 16-byte store (SGD) 5 -> 82.9 / 83.8 / 84.4, 6 -> 83.5 / 84.6 / 84.5, 7 -> 85.0 / 83.8 / 82.7;
+  // fp32 Adam (three stores) 5 -> 84.9 / 83.4 / 82.5, 6 -> 85.1 / 84.8 / 83.7, 7 -> 82.2 / 82.9 / 82.9; Adam with 16-bit
+  // gradients (8-byte loads, so more of them per byte; four stores) 5 -> 80.1 / 83.0 / 82.0, 6 -> 81.0 / 82.0 / 81.4,
   // 7 -> 82.0 / 81.3 / 80.5.
   const int loads = (load_bytes + 15) / 16;
-  (void)store_bytes;
-  const int mid = grad_bytes == 2 ? (loads == 7 ? 11 : 12) : (loads <= 6 ? 11 : 12);
+  const int mid = store_bytes <= 16 ? (loads == 7 ? 11 : 13)
+                                    : (grad_bytes == 2 ? (loads == 7 ? 11 : 12) : (loads <= 6 ? 11 : 12));
   const int waves = loads <= 2 ? 26 : (loads <= 4 ? 17 : (loads <= 7 ? mid : (loads <= 10 ? 8 : (loads <= 13 ? 7 : 8))));
   sh.block = 64;
   sh.lds_bytes = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
-  if (f_block == 64 || f_block == 256) sh.block = f_block;
-  if (f_lds >= 0 && f_lds <= 64) sh.lds_bytes = (unsigned)f_lds * 1024u;
   return sh;
 }
 

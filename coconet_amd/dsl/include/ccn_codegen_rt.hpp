@@ -321,30 +321,27 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // Launch shape for a kernel whose threads load `loads` and store `stores` 16-byte packs, from measurements on MI355X
 // at 2^28 elements: single-wavefront workgroups, and fewer of them per CU the more loads a thread has in flight
-// (26 up to 2 loads, 20 up to 4, 13 up to 7, 7 up to 10, 6 up to 13, 8 beyond: from 8 loads on one fewer than the
+// (26 up to 2 loads, 20 up to 4, 11 or 12 up to 7, 7 up to 10, 6 up to 13, 8 beyond: from 8 loads on one fewer than the
 // library's kernels of the same shape, whose double-precision bias correction keeps a wavefront busy for longer), the
 // cap expressed as unused dynamic LDS.  Scalar (unaligned) launches keep 256 threads.
 struct LaunchShape {
   int block;
   unsigned lds;
 };
-inline LaunchShape shape_for(int loads, int stores, int vec, bool has_sums = false) {
-  // CCN_BLOCK (64 | 256) and CCN_LDS_KB override the shape, as in the library; meant for tuning runs.
-  static const int f_block = [] { const char* e = getenv("CCN_BLOCK"); return e ? atoi(e) : 0; }();
-  static const int f_lds = [] { const char* e = getenv("CCN_LDS_KB"); return e ? atoi(e) : -1; }();
+inline LaunchShape shape_for(int loads, int stores, int vec, bool has_sums = false, int grad_bytes = 4) {
   LaunchShape sh{kBlock, 0};
-  (void)stores;
   if (vec == 1) return sh;
-  // wavefronts per CU by 16-byte loads per thread, measured at N = 2^28: 2 -> 26, 3-4 -> 20, 5-7 -> 13, 8-10 -> 7, 11-13 -> 6
-  const int waves = loads <= 2 ? 26 : (loads <= 4 ? 20 : (loads <= 7 ? 13 : (loads <= 10 ? 7 : (loads <= 13 ? 6 : 8))));
+  // wavefronts per CU by 16-byte loads per thread, measured at N = 2^28: 2 -> 26, 3-4 -> 20, 5-7 -> 11-13 (the library's
+  // table: by the number of stores and the width of the gradient loads; the fp16-gradient Adam program: 1.753 ms per
+  // epoch at 11, 1.776 at 12, 1.795 at 13), 8-10 -> 7, 11-13 -> 6
+  const int mid = stores <= 1 ? (loads == 7 ? 11 : 13) : (grad_bytes == 2 ? (loads == 7 ? 11 : 12) : (loads <= 6 ? 11 : 12));
+  const int waves = loads <= 2 ? 26 : (loads <= 4 ? 20 : (loads <= 7 ? mid : (loads <= 10 ? 7 : (loads <= 13 ? 6 : 8))));
   sh.block = kWave;
   sh.lds = ((160u * 1024u / (unsigned)waves) / 1024u) * 1024u;
   if (has_sums) {   // float64 sums and a workgroup reduction: four 256-thread workgroups per CU hide them better
     sh.block = kBlock;   // (emitted LAMB at N = 2^28, P = 8: 3.02 ms per epoch against 3.07 ms with the shape above)
     sh.lds = 40u * 1024u;
   }
-  if (f_block == kWave || f_block == kBlock) sh.block = f_block;
-  if (f_lds >= 0 && f_lds <= 64) sh.lds = (unsigned)f_lds * 1024u;
   return sh;
 }
 
@@ -356,7 +353,7 @@ inline unsigned grid_for(size_t n, int vec, int block) {
 template <class Body, int VEC> unsigned launch_vec(const KernelArgs<Body>& a, hipStream_t s) {
   // 16-byte loads per thread: an fp16 gradient pack is half of one
   const int red_loads = Body::HAS_RED ? (a.nranks * (int)sizeof(typename Body::RedT) + 3) / 4 : 0;
-  const LaunchShape sh = shape_for(red_loads + Body::NIN, Body::NOUT, VEC, Body::NACC > 0);
+  const LaunchShape sh = shape_for(red_loads + Body::NIN, Body::NOUT, VEC, Body::NACC > 0, Body::HAS_RED ? (int)sizeof(typename Body::RedT) : 4);
   const unsigned grid = grid_for(a.n, VEC, sh.block);
   const int P = Body::HAS_RED ? a.nranks : 1;
   auto go = [&](auto ptag) {
