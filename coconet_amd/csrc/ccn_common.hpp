@@ -197,8 +197,9 @@ unsigned stream_grid(size_t units, size_t tile);
 // copy wants all the occupancy it can get.
 struct StreamShape { int block; unsigned lds_bytes; };
 // Shape for a kernel whose threads each load `load_bytes` and store `store_bytes`, one pack per array; `grad_bytes` is
-// the element size of the gradient arrays (narrow elements mean more load instructions for the same bytes).
-StreamShape stream_shape(int load_bytes, int store_bytes, int grad_bytes = 4);
+// the element size of the gradient arrays (narrow elements mean more load instructions for the same bytes);
+// `starts_alike`: most of the arrays start at the same offset within 64 KiB, so a thread's loads meet on one HBM channel.
+StreamShape stream_shape(int load_bytes, int store_bytes, int grad_bytes = 4, bool starts_alike = false);
 // Dynamic LDS request that keeps at most `per_cu` workgroups on a CU (0 = no request).
 unsigned lds_for_residency(int per_cu);
 

@@ -412,7 +412,15 @@ static int launch_one(const typename M::G* const* g, int nP, const StateTable<M:
   const size_t nvec = n / VEC;
   const int load_bytes = VEC * (nP * (int)sizeof(typename M::G) + M::NS * 4);
   const int store_bytes = VEC * (M::NS * 4 + (M::OUT16 ? 2 : 0) + (M::OUTF ? 4 : 0));
-  const StreamShape sh = stream_shape(load_bytes, store_bytes, (int)sizeof(typename M::G));
+  // do the arrays start alike?  (more than half of them in the same 4 KiB step of a 64 KiB period: plain allocations of
+  // equal size do, the library's allocator staggers them)
+  int slots[16] = {0};
+  for (int p = 0; p < nP; p++) slots[(reinterpret_cast<uintptr_t>(g[p]) >> 12) & 15]++;
+  for (int k = 0; k < M::NS; k++) slots[(reinterpret_cast<uintptr_t>(st.p[k]) >> 12) & 15]++;
+  int most = 0;
+  for (int k = 0; k < 16; k++) most = slots[k] > most ? slots[k] : most;
+  const bool alike = 2 * most > nP + M::NS;
+  const StreamShape sh = stream_shape(load_bytes, store_bytes, (int)sizeof(typename M::G), alike);
   size_t tiles = (nvec + (size_t)sh.block * UNROLL - 1) / ((size_t)sh.block * UNROLL);
   if (tiles < 1) tiles = 1;                                     // the n % VEC tail still needs workgroup 0
   const size_t gx = tiles < 0x40000000ull ? tiles : 0x40000000ull;
