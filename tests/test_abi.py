@@ -59,6 +59,13 @@ def test_argument_validation_happens_before_any_device_work():
     assert lib.ccn_mlp_outproj_bf16(None, 0x1000, null, 0, 0x1000, None, 0x1000, 128, 128, 64, 0.1, 0, None) == capi.CCN_EINVAL
     assert lib.ccn_mlp_outproj_bf16(0x1000, 0x1000, null, 0, 0x1000, None, 0x1000, 128, 130, 64, 0.1, 0, None) == capi.CCN_ERANGE   # N % 4
     assert lib.ccn_mlp_outproj_bf16(0x1000, 0x1000, null, 0, 0x1000, None, 0x1000, 128, 128, 64, 1.0, 0, None) == capi.CCN_EINVAL
+    for mm in (lib.ccn_matmul_bf16_f32, lib.ccn_matmul_f16_f32, lib.ccn_matmul_bf16, lib.ccn_matmul_f16):
+        assert mm(None, 0x1000, 0x1000, 128, 128, 64, None) == capi.CCN_EINVAL
+        assert mm(0x1000, 0x1000, None, 128, 128, 64, None) == capi.CCN_EINVAL
+        assert mm(0x1000, 0x1000, 0x1000, 128, 0, 64, None) == capi.CCN_EINVAL
+        assert mm(0x1000, 0x1000, 0x1000, 128, 130, 64, None) == capi.CCN_ERANGE   # N % 4
+        assert mm(0x1000, 0x1004, 0x1000, 128, 128, 64, None) == capi.CCN_EINVAL   # W not 16-byte aligned
+    assert lib.ccn_matmul_bf16(0x1000, 0x1000, 0x1004, 128, 128, 64, None) == capi.CCN_EINVAL   # a 16-bit C is 8-byte aligned
     plan = C.c_void_p()
     offs = (C.c_size_t * 3)(0, 10, 10)
     assert lib.ccn_lamb_plan_create(offs, 2, C.byref(plan)) == capi.CCN_EINVAL      # empty segment
