@@ -388,7 +388,8 @@ void matmul_tile256_kernel(const uint16_t* __restrict__ X, const uint16_t* __res
   const uint32_t wvoff = (uint32_t)(((lane >> 5) * N + 8 * ((lane & 31) ^ (4 * (2 * (wave & 1) + (lane >> 5))))) * 2);
   // The loads are written as assembly: the compiler orders every LDS read after a direct-to-LDS load it can see behind a
   // wait for ALL outstanding loads, which would put the memory latency into every step.  Here the only reads of a
-  // stage follow the wait and barrier below, so the waits are placed by hand.
+  // stage follow the wait and barrier below, so the waits are placed by hand.  (m0, which names the LDS destination, is
+  // a reserved register: the compiler sets it right before its own uses and keeps nothing in it across a statement.)
   auto words = [](const void* base) {
     const uint64_t a = reinterpret_cast<uint64_t>(base);
     return u32x4{(uint32_t)a, (uint32_t)(a >> 32), 0x7ffffffcu, 0x00020000u};   // no stride, no bounds, as buffer_at()
