@@ -797,7 +797,7 @@ int matmul_launch(const uint16_t* X, const uint16_t* W, void* C, int M, int N, i
   // Whole large tiles, and enough of them to occupy at least half of the CUs (one workgroup per CU): the matrix-core-bound
   // kernel.  Smaller products are faster on four times as many 128 x 128 tiles (16 / 64 large tiles at K = 1024: 13.5
   // against 21.4 us / 17.6 against 24.9 us; 128: 26.6 against 27.6; 256: 52.0 against 37.8).
-  if (M % TM == 0 && N % TN == 0 && (size_t)128 * (size_t)N * 4 < 0x7fffffffull &&
+  if (M % TM == 0 && N % TN == 0 && (size_t)128 * (size_t)N * 4 < 0x7fffffffull && aligned16(C) &&   // it stores 16 bytes per lane
       2 * (size_t)(M / TM) * (size_t)(N / TN) >= (size_t)di->cu_count) {
     static const hipError_t attr = hipFuncSetAttribute((const void*)matmul_tile256_kernel<F16, C16>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBigLds);

@@ -635,3 +635,10 @@ def test_plain_product_with_16_bit_c(ccn, M, N, K, half):
     with pytest.raises(ccn.CoconetError) as e:
         ccn.matmul_16(u16_dev(X), u16_dev(W), C16, M, N + 2, K, half=half)
     assert e.value.code == ccn.CCN_ERANGE
+    if M % 256 == 0 and N % 256 == 0:   # a C that is only 8-byte aligned: same values from the kernel that stores 8 bytes per lane
+        pad = torch.full((M * N + 4,), 0x7e01, dtype=torch.int16, device=DEV)
+        C8 = pad[4:].view(M, N)
+        assert C8.data_ptr() % 16 == 8
+        ccn.matmul_16(u16_dev(X), u16_dev(W), C8, M, N, K, half=half)
+        torch.cuda.synchronize()
+        assert torch.equal(C8, C16)
